@@ -1,0 +1,146 @@
+"""Settings of the engine that are not properties of a checkpoint.
+
+`EngineConfig` is what the engine reads. `ContinuousBatchingConfig`,
+`GenerationConfig` and `NeuronConfig` keep the reference's names and meanings of
+options (config.py:73-139, :206-363) for the ones that have a counterpart on one
+GPU, so that code written against the reference's API keeps working.
+"""
+from dataclasses import dataclass, field
+from typing import Optional
+
+import torch
+
+_DTYPES = {
+    "float32": torch.float32, "f32": torch.float32, "fp32": torch.float32,
+    "bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
+}
+
+
+def parse_dtype(name) -> torch.dtype:
+    """Compute dtype from the reference's `amp` names (dtypes.py:18-35) or torch's.
+    float16 storage is served in bfloat16: the kernels have one 16-bit format."""
+    if isinstance(name, torch.dtype):
+        if name in (torch.float32, torch.bfloat16):
+            return name
+        if name == torch.float16:
+            return torch.bfloat16
+        raise ValueError(f"unsupported dtype {name}")
+    key = str(name).lower()
+    if key in ("f16", "fp16", "float16"):
+        return torch.bfloat16
+    if key not in _DTYPES:
+        raise ValueError(f"unsupported dtype {name!r}; use one of {sorted(_DTYPES)}")
+    return _DTYPES[key]
+
+
+@dataclass
+class ContinuousBatchingConfig:
+    """Capacities for continuous batching, named as in config.py:73-103.
+
+    `block_size`/`num_blocks` are the page size and page count of the cache
+    (set there by `init_cache_engine`, :100-102)."""
+    max_num_seqs: Optional[int] = None
+    max_model_len: Optional[int] = None
+    optimized_paged_attention: bool = True
+    enable_chunked_prefill: bool = True
+    block_size: Optional[int] = None
+    num_blocks: Optional[int] = None
+    batch_size_for_shared_caches: Optional[int] = None
+
+    def __post_init__(self):
+        if self.max_num_seqs is None:
+            self.max_num_seqs = self.batch_size_for_shared_caches
+        if self.max_num_seqs is None:
+            raise ValueError("max_num_seqs (or batch_size_for_shared_caches) is required")
+        self.batch_size_for_shared_caches = self.max_num_seqs
+
+    def init_cache_engine(self, block_size, num_blocks):
+        self.block_size = block_size
+        self.num_blocks = num_blocks
+
+
+@dataclass
+class GenerationConfig:
+    """Generation options, named as in config.py:106-139."""
+    max_length: Optional[int] = None
+    do_sample: bool = False
+    top_k: int = 50
+    top_p: float = 1.0
+    top_p_min_tokens: int = 1
+    global_top_k: Optional[int] = None
+    eos_token_id: Optional[int] = None
+    temperature: float = 1.0
+    dynamic: bool = False
+    deterministic: bool = False
+    per_batch_line: bool = False
+
+    def __post_init__(self):
+        self.top_p = float(self.top_p)
+        self.temperature = float(self.temperature)
+
+
+@dataclass
+class NeuronConfig:
+    """The switches of config.py:206-363 that mean something on one GPU.
+
+    `continuous_batching` sizes the scheduler and the cache,
+    `on_device_generation` makes `sample` draw with these generation options,
+    `cast_logits_dtype` is always float32 here, `output_all_logits` makes
+    `forward` return the logits of every position. Other keywords of the
+    reference (tensor parallel layouts, quantization, compiler options) are
+    accepted and ignored when they are left at their defaults, and refused with
+    a clear message otherwise."""
+    continuous_batching: Optional[ContinuousBatchingConfig] = None
+    on_device_generation: Optional[GenerationConfig] = None
+    on_device_embedding: bool = True
+    cast_logits_dtype: str = "float32"
+    output_all_logits: bool = False
+    fuse_qkv: bool = True
+    padding_side: str = "left"
+
+    def __post_init__(self):
+        if isinstance(self.continuous_batching, dict):
+            self.continuous_batching = ContinuousBatchingConfig(**self.continuous_batching)
+        if self.cast_logits_dtype != "float32":
+            raise ValueError("logits are returned in float32; cast_logits_dtype must be 'float32'")
+
+
+@dataclass
+class EngineConfig:
+    """What the engine is built with.
+
+    dtype            compute and storage dtype: torch.bfloat16 or torch.float32
+    page_size        tokens per cache page (a multiple of 16)
+    num_pages        pages per cache group; None sizes the pool from `max_tokens`
+                     or, failing that, from free device memory
+    max_tokens       the most tokens live requests hold at a time
+    max_num_seqs     the most live requests (slots of per-request state)
+    max_num_batched_tokens   token budget of one step
+    max_model_len    longest request (prompt + generated); capped by the model
+    kernels          "hip" (the product path) or "reference" (the plain torch
+                     rendition of every kernel, for debugging on any device;
+                     never chosen by itself)
+    memory_fraction  share of free device memory the page pool may take when it
+                     is sized from memory
+    """
+    dtype: torch.dtype = torch.bfloat16
+    page_size: int = 64
+    num_pages: Optional[int] = None
+    max_tokens: Optional[int] = None
+    max_num_seqs: int = 64
+    max_num_batched_tokens: int = 2048
+    max_model_len: Optional[int] = None
+    kernels: str = "hip"
+    device: str = "cuda:0"
+    memory_fraction: float = 0.85
+    use_graphs: bool = True
+    seed: int = 0
+
+    def __post_init__(self):
+        self.dtype = parse_dtype(self.dtype)
+        if self.page_size <= 0 or self.page_size % 16:
+            raise ValueError(f"page_size must be a positive multiple of 16, got {self.page_size}")
+        if self.kernels not in ("hip", "reference"):
+            raise ValueError(f"kernels must be 'hip' or 'reference', got {self.kernels!r}")
+        if self.max_num_seqs <= 0 or self.max_num_batched_tokens <= 0:
+            raise ValueError("max_num_seqs and max_num_batched_tokens must be positive")

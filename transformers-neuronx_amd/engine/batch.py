@@ -1,0 +1,96 @@
+"""What one step runs on: the tokens it brings, whose they are, and where their
+requests' pages lie.
+
+A step is a concatenation of runs, one run per request: a portion of a prompt
+of any length, or a single decoded token. This is the one-dimensional form of
+the reference's chunked-prefill entry (base.py:384-408: `query_lens`,
+`context_lens`, block tables), with a decoded token as a run of length one.
+"""
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+
+@dataclass
+class StepEntry:
+    """A request's next tokens and the places among them whose logits are wanted."""
+    req: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class GroupView:
+    """A page group as a step sees it."""
+    block_table: torch.Tensor       # int32 [R, width], -1 where no page is held
+    page_size: int
+    width: int
+
+
+@dataclass
+class StepContext:
+    num_tokens: int                 # T
+    num_requests: int               # R
+    token_ids: torch.Tensor         # int32 [T]
+    positions: torch.Tensor         # int32 [T], index of each token in its own request
+    token_request: torch.Tensor     # int32 [T], run each token belongs to
+    run_start: torch.Tensor         # int32 [R+1], first token of each run
+    cached_lens: torch.Tensor       # int32 [R], tokens of each request stored before this step
+    slots: torch.Tensor             # int32 [R], state slot of each request
+    logits_rows: torch.Tensor       # int32 [M], tokens whose logits are wanted
+    groups: Dict[str, GroupView]
+    # The same on the host, for planning launches and for parts written in Python.
+    run_lens_host: np.ndarray = None
+    cached_lens_host: np.ndarray = None
+    slots_host: np.ndarray = None
+    plans: Dict = field(default_factory=dict)    # launch plans the kernel backend keeps per step
+
+    @property
+    def max_run(self) -> int:
+        return int(self.run_lens_host.max())
+
+    @property
+    def max_total(self) -> int:
+        return int((self.run_lens_host + self.cached_lens_host).max())
+
+
+def build_context(entries: List[StepEntry], cached: List[int], slots: List[int],
+                  tables: Dict[str, np.ndarray], page_size: int, device) -> StepContext:
+    """Pack a step's integers into one buffer, copy it once, and slice it."""
+    run_lens = np.array([len(e.tokens) for e in entries], dtype=np.int32)
+    cached_np = np.array(cached, dtype=np.int32)
+    r, t = len(entries), int(run_lens.sum())
+    run_start = np.zeros(r + 1, dtype=np.int32)
+    np.cumsum(run_lens, out=run_start[1:])
+    token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
+    token_request = np.repeat(np.arange(r, dtype=np.int32), run_lens)
+    positions = (np.arange(t, dtype=np.int32) - run_start[token_request] + cached_np[token_request]).astype(np.int32)
+    rows = []
+    for i, e in enumerate(entries):
+        for w in e.want:
+            if not 0 <= w < len(e.tokens):
+                raise ValueError(f"request {e.req!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
+            rows.append(run_start[i] + w)
+    rows = np.array(rows, dtype=np.int32)
+    pieces = [token_ids, positions, token_request, run_start, cached_np, np.array(slots, dtype=np.int32), rows]
+    names = list(tables)
+    pieces += [tables[g].reshape(-1) for g in names]
+    # each piece starts at a multiple of 4 integers, so that every view is 16-byte aligned
+    offsets, total = [], 0
+    for p in pieces:
+        offsets.append(total)
+        total += -(-p.size // 4) * 4
+    flat = np.zeros(max(total, 4), dtype=np.int32)
+    for off, p in zip(offsets, pieces):
+        flat[off:off + p.size] = p
+    dev = torch.from_numpy(flat).to(device)
+    views = [dev[off:off + p.size] for off, p in zip(offsets, pieces)]
+    groups = {}
+    for g, v in zip(names, views[7:]):
+        width = tables[g].shape[1]
+        groups[g] = GroupView(v.view(r, width), page_size, width)
+    return StepContext(t, r, views[0], views[1], views[2], views[3], views[4], views[5], views[6], groups,
+                       run_lens_host=run_lens, cached_lens_host=cached_np,
+                       slots_host=np.array(slots, dtype=np.int32))

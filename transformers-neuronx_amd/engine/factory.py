@@ -1,0 +1,64 @@
+"""From a model folder and an `EngineConfig` to a runner with its cache."""
+import os
+from typing import Optional
+
+import torch
+
+from ..cache.manager import CacheManager
+from ..config.engine_config import EngineConfig
+from ..config.registry import read_config, resolve
+from ..kernels import make_ops
+from ..weights.loader import Checkpoint, TensorDict
+from ..weights.random_init import random_tensors
+from .model import DecoderModel
+from .runner import ModelRunner
+
+
+def _device_of(cfg: EngineConfig) -> torch.device:
+    dev = torch.device(cfg.device)
+    if cfg.kernels == "hip" and dev.type != "cuda":
+        raise RuntimeError("the HIP kernels need a GPU device (cuda:N); "
+                           "kernels='reference' is the only backend that runs elsewhere")
+    return dev
+
+
+def size_page_pool(cfg: EngineConfig, bytes_per_page: int, device: torch.device) -> int:
+    """Pages per group: as told, or for `max_tokens`, or what free memory allows."""
+    if cfg.num_pages is not None:
+        return cfg.num_pages
+    if cfg.max_tokens is not None:
+        return max(1, -(-cfg.max_tokens // cfg.page_size))
+    if device.type == "cuda" and bytes_per_page:
+        free, _ = torch.cuda.mem_get_info(device)
+        return max(1, int(free * cfg.memory_fraction) // bytes_per_page)
+    return 256
+
+
+def build_runner(model_config, source, cfg: EngineConfig) -> ModelRunner:
+    """`model_config` a typed configuration, `source` a `Checkpoint` or `TensorDict`."""
+    device = _device_of(cfg)
+    arch = resolve(model_config.to_dict())
+    model = DecoderModel(arch.build_spec(model_config))
+    ops = make_ops(cfg.kernels, cfg.dtype, device)
+    model.load(source, ops, cfg.dtype, device)
+    needs = model.cache_needs()
+    num_pages = size_page_pool(cfg, CacheManager.bytes_per_page(needs, cfg.page_size, cfg.dtype), device)
+    cache = CacheManager(needs, cfg.page_size, num_pages, cfg.max_num_seqs, cfg.dtype, device)
+    return ModelRunner(model, cache, ops)
+
+
+def runner_from_folder(folder: str, cfg: EngineConfig) -> ModelRunner:
+    _, model_config = read_config(folder)
+    return build_runner(model_config, Checkpoint(folder), cfg)
+
+
+def runner_from_random(model_config, seed: int, cfg: EngineConfig) -> ModelRunner:
+    """Random weights drawn on the device, without a folder (for models too large
+    to write for a measurement)."""
+    device = _device_of(cfg)
+    arch = resolve(model_config.to_dict())
+    spec = arch.build_spec(model_config)
+    decls = DecoderModel(spec).param_decls()
+    storage = torch.float32 if cfg.dtype == torch.float32 else torch.bfloat16
+    tensors = random_tensors(decls, spec.init_std, seed, storage, device)
+    return build_runner(model_config, TensorDict(tensors), cfg)

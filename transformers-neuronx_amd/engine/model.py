@@ -1,0 +1,103 @@
+"""The decoder, put together from a `ModelSpec`.
+
+It owns the parts and their tensors and runs them in the order the spec lists.
+What takes the place of the reference's graph owner
+(`DecoderLmHeadForSamplingNoEmbedding`, decoder.py:43-1115, with its 26 named
+weight slots per layer, :1275-1312) is this loop over parts that launch kernels.
+"""
+from typing import Dict, List, Optional
+
+import torch
+
+from ..parts.base import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, CacheNeed, Stream
+from ..parts.spec import LayerSpec, ModelSpec, ParamDecl
+from ..weights.loader import load_tensors
+
+
+class _Layer:
+    def __init__(self, spec: LayerSpec):
+        self.spec = spec
+        self.mixer = MIXERS.build(spec.mixer)
+        self.feed_forward = FEED_FORWARDS.build(spec.feed_forward)
+        self.mixer_norm = NORMS.build(spec.mixer_norm)
+        self.feed_forward_norm = NORMS.build(spec.feed_forward_norm)
+        self.block = BLOCKS.build(
+            _spec_of(spec.block), self.mixer, self.feed_forward, self.mixer_norm, self.feed_forward_norm)
+
+    def _named(self):
+        s = self.spec
+        return [(self.mixer, s.prefix + s.mixer_name), (self.feed_forward, s.prefix + s.feed_forward_name),
+                (self.mixer_norm, s.prefix + s.mixer_norm_name),
+                (self.feed_forward_norm, s.prefix + s.feed_forward_norm_name)]
+
+    def param_decls(self) -> List[ParamDecl]:
+        return [d for part, prefix in self._named() for d in part.param_decls(prefix)]
+
+    def load(self, tensors, ops, dtype):
+        for part, prefix in self._named():
+            part.load(tensors, prefix, ops, dtype)
+
+
+def _spec_of(kind):
+    from ..parts.spec import PartSpec
+    return kind if isinstance(kind, PartSpec) else PartSpec(kind)
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec):
+        self.spec = spec
+        self.embedding = EMBEDDINGS.build(spec.embedding)
+        self.layers = [_Layer(ls) for ls in spec.layers]
+        self.head = HEADS.build(spec.head)
+        self.schedule = spec.resolved_schedule()
+        written = set()
+        for layer, cid, writes in self.schedule:
+            if writes:
+                written.add(cid)
+            elif cid not in written:
+                raise ValueError(f"layer {layer} reads cache {cid} before the call that writes it")
+        self.loaded = False
+
+    # ---------------------------------------------------------------- declarations
+
+    def param_decls(self) -> List[ParamDecl]:
+        decls, seen = [], set()
+        for d in (self.embedding.param_decls() + [d for l in self.layers for d in l.param_decls()]
+                  + self.head.param_decls()):
+            if d.name not in seen:
+                seen.add(d.name)
+                decls.append(d)
+        return decls
+
+    def cache_needs(self) -> Dict[int, Optional[CacheNeed]]:
+        """{cache id: need} of the calls that write a cache."""
+        return {cid: self.layers[layer].mixer.cache_need() for layer, cid, writes in self.schedule if writes}
+
+    # ---------------------------------------------------------------- weights
+
+    def load(self, source, ops, dtype: torch.dtype, device) -> "DecoderModel":
+        tensors = load_tensors(self.param_decls(), source, dtype, device)
+        self.embedding.load(tensors, "", ops, dtype)
+        for layer in self.layers:
+            layer.load(tensors, ops, dtype)
+        self.head.load(tensors, "", ops, dtype)
+        self.ops, self.dtype, self.device = ops, dtype, device
+        self.weight_bytes = sum(t.numel() * t.element_size() for t in {id(t): t for t in tensors.values()}.values())
+        self.loaded = True
+        return self
+
+    # ---------------------------------------------------------------- one step
+
+    def forward(self, ctx, caches) -> torch.Tensor:
+        """Logits float32 `[len(ctx.logits_rows), vocab]` for the step `ctx` describes."""
+        first_block = self.layers[self.schedule[0][0]].block if self.schedule else None
+        want_compute = bool(getattr(first_block, "reads_compute_copy", False))
+        stream: Stream = self.embedding.forward(ctx, want_compute)
+        for layer, cid, writes in self.schedule:
+            cache = caches[cid] if writes else caches[cid].reader()
+            stream = self.layers[layer].block.forward(stream, ctx, cache)
+        return self.head.forward(stream, ctx)
+
+
+def model_param_decls(spec: ModelSpec) -> List[ParamDecl]:
+    return DecoderModel(spec).param_decls()

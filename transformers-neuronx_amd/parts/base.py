@@ -1,0 +1,149 @@
+"""Interfaces of the parts and the registries they are found in.
+
+A part is built from the parameters of its `PartSpec`, declares the tensors it
+reads (`param_decls`), receives them (`load`) and is called by a block with the
+step's context. Mixers also declare what they keep between steps
+(`cache_need`). Registering a class under a new kind is all it takes to use it
+from a `ModelSpec`.
+"""
+from dataclasses import dataclass
+from typing import Callable, Dict, List, Optional, Tuple
+
+from .spec import ParamDecl, PartSpec
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    """What a mixer keeps per request between steps.
+
+    kind 'paged': grows with the tokens. `shapes` names per-token tensors as
+         {name: (layout, dims...)}; `window` (tokens) lets pages be given back
+         once every later query is past them, None keeps them all.
+    kind 'state': fixed size per request. `shapes` is {name: dims}; a slot is
+         zeroed when a request gets it.
+    """
+    kind: str
+    kv_heads: int = 0
+    head_size: int = 0
+    window: Optional[int] = None
+    state_shapes: Tuple[Tuple[str, Tuple[int, ...]], ...] = ()
+    state_dtype: str = "float32"
+
+    def group_key(self):
+        """Layers with equal keys share a page table."""
+        return (self.kind, self.window)
+
+
+class Part:
+    """Base of all parts. `ops` is the kernel backend, `dtype` the compute dtype."""
+
+    def param_decls(self, prefix: str) -> List[ParamDecl]:
+        return []
+
+    def load(self, tensors: Dict[str, "object"], prefix: str, ops, dtype) -> None:
+        self.ops = ops
+        self.dtype = dtype
+
+
+class Mixer(Part):
+    """Mixes information between the tokens of a request.
+
+    forward(h, ctx, cache, residual) -> float32 `[T, hidden]`: residual + mix(h).
+    `h` is `[T, hidden]` in the compute dtype, `cache` the `LayerCache` of the
+    call (None if `cache_need()` is None), `ctx` the step's `StepContext`. The
+    result must not depend on how a request's tokens were cut into steps.
+    """
+
+    def cache_need(self) -> Optional[CacheNeed]:
+        return None
+
+    def forward(self, h, ctx, cache, residual):
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """forward(h, ctx, residual) -> float32 `[T, hidden]`: residual + f(h), token by token."""
+
+    def forward(self, h, ctx, residual):
+        raise NotImplementedError
+
+
+class Norm(Part):
+    """forward(x, want_f32, want_compute) -> (float32 or None, compute dtype or None),
+    both `[T, hidden]`, from the float32 `x`. Statistics are taken in float32."""
+
+    def forward(self, x, want_f32: bool, want_compute: bool):
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Where positions enter. `at_input(x, positions)` adds to the embedded
+    tokens (learned or fixed tables); `on_query_key` is the hook of encodings
+    that turn queries and keys inside a mixer. A part leaves the hook it does
+    not use as it is."""
+
+    def at_input(self, x, positions, want_compute: bool):
+        return None
+
+    rotates_query_key = False
+
+
+class Block(Part):
+    """Arranges one layer's mixer, feed-forward and norms around the residual stream.
+
+    forward(stream, ctx, cache) -> stream, where stream is a `Stream`."""
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm):
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.mixer_norm = mixer_norm
+        self.feed_forward_norm = feed_forward_norm
+
+    def forward(self, stream, ctx, cache):
+        raise NotImplementedError
+
+
+@dataclass
+class Stream:
+    """The residual stream between layers: float32 `[T, hidden]`, and beside it a
+    copy in the compute dtype when the last part that wrote it made one."""
+    x: "object"
+    compute: Optional["object"] = None
+
+
+class _Registry:
+    def __init__(self, what: str):
+        self.what = what
+        self._classes: Dict[str, type] = {}
+
+    def register(self, kind: str) -> Callable[[type], type]:
+        def deco(cls):
+            self._classes[kind] = cls
+            cls.kind = kind
+            return cls
+        return deco
+
+    def build(self, spec: PartSpec, *args):
+        if spec.kind not in self._classes:
+            raise KeyError(f"no {self.what} is registered as {spec.kind!r}; known: {sorted(self._classes)}")
+        return self._classes[spec.kind](*args, **spec.params)
+
+    def kinds(self):
+        return sorted(self._classes)
+
+
+MIXERS = _Registry("mixer")
+FEED_FORWARDS = _Registry("feed-forward")
+NORMS = _Registry("norm")
+POSITIONS = _Registry("position encoding")
+BLOCKS = _Registry("block arrangement")
+EMBEDDINGS = _Registry("embedding")
+HEADS = _Registry("head")
+
+register_mixer = MIXERS.register
+register_feed_forward = FEED_FORWARDS.register
+register_norm = NORMS.register
+register_position = POSITIONS.register
+register_block = BLOCKS.register
+register_embedding = EMBEDDINGS.register
+register_head = HEADS.register
