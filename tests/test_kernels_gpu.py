@@ -1,0 +1,279 @@
+"""Each HIP kernel alone against its plain torch rendition, at sizes other than the engine's."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _ops(dtype):
+    from transformers_neuronx_amd.kernels.hip import HipOps
+    from transformers_neuronx_amd.kernels.reference import ReferenceOps
+    return HipOps(dtype, DEV), ReferenceOps(dtype, DEV)
+
+
+def _tol(dtype):
+    return dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,width", [(1, 48), (7, 96), (33, 1000), (5, 4096), (3, 5000), (2, 13000)])
+def test_layernorm(dtype, rows, width):
+    hip, ref = _ops(dtype)
+    g = torch.Generator(device=DEV).manual_seed(rows * 1000 + width)
+    x = torch.randn(rows, width, device=DEV, generator=g) * 3 + 1.5
+    w = torch.randn(width, device=DEV, generator=g)
+    b = torch.randn(width, device=DEV, generator=g)
+    for weight, bias in ((w, b), (None, None)):
+        for eps in (1e-5, 1e-2):
+            f_h, c_h = hip.layernorm(x, weight, bias, eps, dtype, True, True)
+            f_r, c_r = ref.layernorm(x, weight, bias, eps, dtype, True, True)
+            torch.testing.assert_close(f_h, f_r, rtol=2e-5, atol=2e-5)
+            torch.testing.assert_close(c_h.float(), c_r.float(), **_tol(dtype))
+    # library routine: torch's layer_norm
+    f_h, _ = hip.layernorm(x, w, b, 1e-5, dtype, True, False)
+    torch.testing.assert_close(f_h, torch.nn.functional.layer_norm(x, (width,), w, b, 1e-5), rtol=2e-5, atol=2e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gather_embed_positions_cast(dtype):
+    hip, ref = _ops(dtype)
+    g = torch.Generator(device=DEV).manual_seed(3)
+    table = torch.randn(777, 40, device=DEV, generator=g).to(dtype)
+    pos_table = torch.randn(50, 40, device=DEV, generator=g).to(dtype)
+    ids = torch.randint(0, 777, (19,), device=DEV, generator=g, dtype=torch.int32)
+    pos = torch.randint(0, 47, (19,), device=DEV, generator=g, dtype=torch.int32)
+    e_h, e_r = hip.embed(ids, table, dtype), ref.embed(ids, table, dtype)
+    assert torch.equal(e_h, e_r)
+    for want in (True, False):
+        xf_h, xc_h = hip.add_positions(e_h, pos, pos_table, 3, dtype, want)
+        xf_r, xc_r = ref.add_positions(e_r, pos, pos_table, 3, dtype, want)
+        assert torch.equal(xf_h, xf_r)
+        assert (xc_h is None) == (xc_r is None)
+        if want:
+            assert torch.equal(xc_h, xc_r)
+    xf_h, xc_h = hip.to_stream(e_h, dtype, True)
+    assert torch.equal(xf_h, e_r.float()) and torch.equal(xc_h, e_r)
+    big = torch.randn(100003, device=DEV, generator=g)
+    assert torch.equal(hip.cast(big, torch.bfloat16), big.to(torch.bfloat16))
+    assert torch.equal(hip.cast(big.to(torch.bfloat16), torch.float32), big.to(torch.bfloat16).float())
+    rows = torch.tensor([5, 0, 18, 5], device=DEV, dtype=torch.int32)
+    assert torch.equal(hip.gather_rows(xf_h, rows), xf_h[rows.long()])
+
+
+GEMM_SHAPES = [(1, 16, 8), (3, 50, 24), (8, 96, 96), (17, 1000, 48), (64, 320, 96), (65, 130, 72),
+               (130, 257, 136), (300, 96, 320), (5, 4096, 512), (40, 136, 1024)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
+def test_linear(dtype, m, n, k):
+    hip, ref = _ops(dtype)
+    g = torch.Generator(device=DEV).manual_seed(m * 7 + n * 3 + k)
+    x = torch.randn(m, k, device=DEV, generator=g).to(dtype)
+    w = (torch.randn(n, k, device=DEV, generator=g) / math.sqrt(k)).to(dtype)
+    bias = torch.randn(n, device=DEV, generator=g)
+    res = torch.randn(m, n, device=DEV, generator=g)
+    tol = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    tol32 = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(rtol=1e-3, atol=1e-3)
+    for act in (None, "relu", "gelu", "gelu_new"):
+        y_h = hip.linear(x, w, bias, act=act)
+        y_r = ref.linear(x, w, bias, act=act)
+        torch.testing.assert_close(y_h.float(), y_r.float(), **tol)
+    y_h = hip.linear(x, w, None, residual=res, out_f32=True)
+    y_r = ref.linear(x, w, None, residual=res, out_f32=True)
+    torch.testing.assert_close(y_h, y_r, **tol32)
+    # library routine
+    torch.testing.assert_close(hip.linear(x, w, bias, out_f32=True),
+                               torch.nn.functional.linear(x.float(), w.float(), bias), **tol32)
+    if dtype == torch.bfloat16:
+        # both bfloat16 kernels, whatever the row count
+        y_t = hip.linear(x, w, bias, act="relu", residual=res, out_f32=True, force_tiled=True)
+        y_r = ref.linear(x, w, bias, act="relu", residual=res, out_f32=True)
+        torch.testing.assert_close(y_t, y_r, **tol32)
+
+
+def test_linear_float32_matrix_in_bfloat16_engine():
+    hip, ref = _ops(torch.bfloat16)
+    g = torch.Generator(device=DEV).manual_seed(11)
+    x = torch.randn(9, 64, device=DEV, generator=g).to(torch.bfloat16)
+    w = torch.randn(33, 64, device=DEV, generator=g) / 8
+    torch.testing.assert_close(hip.linear(x, w, out_f32=True), x.float() @ w.t(), rtol=1e-4, atol=1e-4)
+
+
+def test_linear_refuses_bad_inner_size():
+    hip, _ = _ops(torch.bfloat16)
+    x = torch.zeros(4, 12, device=DEV, dtype=torch.bfloat16)
+    w = torch.zeros(8, 12, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        hip.linear(x, w)
+
+
+def _make_step(runs, cached, page_size, num_pages, seed, device=DEV):
+    """A step context over requests with `cached[i]` stored tokens and `runs[i]` new ones,
+    their pages drawn at random from the pool (so order in memory differs from order in the request)."""
+    from transformers_neuronx_amd.engine.batch import StepEntry, build_context
+    rng = np.random.default_rng(seed)
+    perm = rng.permutation(num_pages).tolist()
+    tables, width = [], 0
+    for r, c in zip(runs, cached):
+        nb = -(-(r + c) // page_size)
+        tables.append([perm.pop() for _ in range(nb)])
+        width = max(width, nb)
+    tab = np.full((len(runs), width + 1), -1, dtype=np.int32)
+    for i, t in enumerate(tables):
+        tab[i, :len(t)] = t
+    entries = [StepEntry(i, [0] * r, []) for i, r in enumerate(runs)]
+    return build_context(entries, list(cached), list(range(len(runs))), {"full": tab}, page_size, device)
+
+
+ATTN_CASES = [
+    # heads, kv heads, head size, page size, runs, cached
+    (4, 4, 16, 16, [5, 1, 17], [0, 30, 3]),
+    (3, 3, 32, 16, [40, 1, 1, 2], [0, 77, 15, 16]),
+    (6, 2, 48, 32, [70, 1], [0, 130]),
+    (5, 1, 80, 64, [3, 129, 1], [64, 0, 200]),
+    (2, 2, 128, 64, [1, 1, 65], [511, 63, 64]),
+    (1, 1, 256, 16, [20, 1], [0, 33]),
+]
+
+
+def _fill_cache_and_compare(dtype, heads, kv, hs, ps, runs, cached, window):
+    hip, ref = _ops(dtype)
+    num_pages = sum(-(-(r + c) // ps) for r, c in zip(runs, cached)) + 3
+    g = torch.Generator(device=DEV).manual_seed(heads * 100 + hs)
+    # the cache as earlier steps left it: filled by a first step that stores the cached tokens
+    kp = torch.full((num_pages, kv, ps, hs), float("nan"), device=DEV, dtype=dtype)
+    vp = torch.full((num_pages, kv, hs, ps), float("nan"), device=DEV, dtype=dtype)
+    kp_r, vp_r = kp.clone(), vp.clone()
+    width = (heads + 2 * kv) * hs
+    ctx_all = _make_step([r + c for r, c in zip(runs, cached)], [0] * len(runs), ps, num_pages, seed=hs)
+    # same pages, two steps: first the cached part, then the new runs
+    tab = ctx_all.groups["full"].block_table.cpu().numpy()
+    from transformers_neuronx_amd.engine.batch import StepEntry, build_context
+    live = [i for i, c in enumerate(cached) if c > 0]
+    bias = torch.randn(width, device=DEV, generator=g) * 0.1
+    scale = 1.0 / math.sqrt(hs)
+    if live:
+        ctx0 = build_context([StepEntry(i, [0] * cached[i], []) for i in live], [0] * len(live), live,
+                             {"full": tab[live]}, ps, DEV)
+        qkv0 = torch.randn(ctx0.num_tokens, width, device=DEV, generator=g).to(dtype)
+        hip.qkv_write(qkv0, bias, heads, kv, hs, scale, ctx0, ctx0.groups["full"], kp, vp)
+        ref.qkv_write(qkv0, bias, heads, kv, hs, scale, ctx0, ctx0.groups["full"], kp_r, vp_r)
+    ctx = build_context([StepEntry(i, [0] * r, []) for i, r in enumerate(runs)], list(cached),
+                        list(range(len(runs))), {"full": tab}, ps, DEV)
+    qkv = torch.randn(ctx.num_tokens, width, device=DEV, generator=g).to(dtype)
+    q_h = hip.qkv_write(qkv, bias, heads, kv, hs, scale, ctx, ctx.groups["full"], kp, vp)
+    q_r = ref.qkv_write(qkv, bias, heads, kv, hs, scale, ctx, ctx.groups["full"], kp_r, vp_r)
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(q_h.float(), q_r.float(), **tol)
+    # what was written is the same, and nothing else was touched (untouched places are still NaN)
+    assert torch.equal(torch.isnan(kp), torch.isnan(kp_r)) and torch.equal(torch.isnan(vp), torch.isnan(vp_r))
+    torch.testing.assert_close(torch.nan_to_num(kp.float()), torch.nan_to_num(kp_r.float()), **tol)
+    torch.testing.assert_close(torch.nan_to_num(vp.float()), torch.nan_to_num(vp_r.float()), **tol)
+    o_h = hip.attention(q_r, heads, kv, hs, ctx, ctx.groups["full"], kp_r, vp_r, window)
+    o_r = ref.attention(q_r, heads, kv, hs, ctx, ctx.groups["full"], kp_r, vp_r, window)
+    assert not torch.isnan(o_h.float()).any()
+    torch.testing.assert_close(o_h.float(), o_r.float(), **tol)
+    return ctx, q_r, kp_r, vp_r, o_h
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", ATTN_CASES)
+@pytest.mark.parametrize("window", [None, 24])
+def test_qkv_write_and_attention(dtype, case, window):
+    _fill_cache_and_compare(dtype, *case, window)
+
+
+def test_attention_is_library_attention_without_cache():
+    """One request from position 0, one head group: torch's scaled_dot_product_attention."""
+    dtype = torch.float32
+    hip, ref = _ops(dtype)
+    heads, hs, ps, n = 4, 32, 16, 50
+    ctx, q, kp, vp, o = _fill_cache_and_compare(dtype, heads, heads, hs, ps, [n], [0], None)
+    tab = ctx.groups["full"].block_table[0, :-(-n // ps)].long()
+    keys = kp[tab].permute(1, 0, 2, 3).reshape(heads, -1, hs)[:, :n]
+    vals = vp[tab].permute(1, 2, 0, 3).reshape(heads, hs, -1)[:, :, :n].transpose(1, 2)
+    qq = q.reshape(n, heads, hs).permute(1, 0, 2)
+    want = torch.nn.functional.scaled_dot_product_attention(qq, keys, vals, is_causal=True, scale=1.0)
+    torch.testing.assert_close(o, want.permute(1, 0, 2).reshape(n, heads * hs), rtol=1e-5, atol=1e-5)
+
+
+def test_attention_finds_a_far_key():
+    """One key among hundreds carries the value: scale one query and one key so that its score stands out."""
+    dtype = torch.bfloat16
+    hip, _ = _ops(dtype)
+    heads, hs, ps, cached = 2, 64, 16, 700
+    num_pages = -(-(cached + 1) // ps) + 2
+    ctx = _make_step([1], [cached], ps, num_pages, seed=5)
+    view = ctx.groups["full"]
+    g = torch.Generator(device=DEV).manual_seed(9)
+    kp = (torch.randn(num_pages, heads, ps, hs, device=DEV, generator=g) * 0.1).to(dtype)
+    vp = (torch.randn(num_pages, heads, hs, ps, device=DEV, generator=g) * 0.1).to(dtype)
+    far = 37
+    page = int(view.block_table[0, far // ps])
+    direction = torch.randn(hs, device=DEV, generator=g)
+    direction /= direction.norm()
+    kp[page, :, far % ps, :] = (direction * 40).to(dtype)
+    vp[page, :, :, far % ps] = 5.0
+    q = (direction * 10).repeat(heads).reshape(1, heads * hs).to(dtype)
+    out = hip.attention(q, heads, heads, hs, ctx, view, kp, vp, None)
+    torch.testing.assert_close(out.float(), torch.full_like(out, 5.0).float(), rtol=1e-2, atol=1e-2)
+    # with a window that ends before the far key it is not seen
+    out_w = hip.attention(q, heads, heads, hs, ctx, view, kp, vp, cached - far)
+    assert out_w.float().abs().max() < 1.0
+
+
+def test_attention_refuses_bad_head_size():
+    hip, _ = _ops(torch.float32)
+    ctx = _make_step([1], [0], 16, 2, seed=1)
+    q = torch.zeros(1, 24, device=DEV)
+    kp = torch.zeros(2, 1, 16, 24, device=DEV)
+    vp = torch.zeros(2, 1, 24, 16, device=DEV)
+    with pytest.raises(RuntimeError, match="head size"):
+        hip.attention(q, 1, 1, 24, ctx, ctx.groups["full"], kp, vp, None)
+
+
+@pytest.mark.parametrize("vocab", [1000, 50272, 333])
+def test_argmax_and_sampling(vocab):
+    hip, ref = _ops(torch.float32)
+    g = torch.Generator(device=DEV).manual_seed(vocab)
+    rows = 24
+    logits = torch.randn(rows, vocab, device=DEV, generator=g) * 3
+    logits[3, 17] = logits[3, 400 % vocab] = logits[3].max() + 1     # a tie: the lower id wins
+    assert torch.equal(hip.argmax(logits), ref.argmax(logits))
+    assert int(hip.argmax(logits)[3]) == 17
+    temp = torch.tensor([0.0, 1.0, 0.7, 1.3] * 6, device=DEV)
+    top_k = torch.tensor([0, 50, 1, 5, 0, vocab + 5] * 4, device=DEV, dtype=torch.int32)
+    top_p = torch.tensor([1.0, 1.0, 0.9, 0.5, 0.3, 0.99, 1.0, 0.05] * 3, device=DEV)
+    seeds = torch.arange(rows, device=DEV, dtype=torch.int64) * 7919 + 1
+    for step in range(6):
+        counters = torch.full((rows,), step, device=DEV, dtype=torch.int64)
+        t_h = hip.sample(logits, temp, top_k, top_p, seeds, counters)
+        t_r = ref.sample(logits, temp, top_k, top_p, seeds, counters)
+        assert (t_h == t_r).float().mean() >= 0.95, (t_h, t_r)    # a draw on a boundary may round either way
+
+
+def test_sampling_distribution():
+    """Frequencies over many draws follow the softmax over the kept tokens."""
+    hip, _ = _ops(torch.float32)
+    vocab, n = 64, 20000
+    g = torch.Generator(device=DEV).manual_seed(1)
+    row = torch.randn(vocab, device=DEV, generator=g) * 2
+    logits = row.repeat(n, 1).contiguous()
+    temp = torch.full((n,), 0.8, device=DEV)
+    top_k = torch.full((n,), 10, device=DEV, dtype=torch.int32)
+    top_p = torch.full((n,), 1.0, device=DEV)
+    seeds = torch.full((n,), 123, device=DEV, dtype=torch.int64)
+    counters = torch.arange(n, device=DEV, dtype=torch.int64)
+    toks = hip.sample(logits, temp, top_k, top_p, seeds, counters).long()
+    vals, idx = torch.topk(row / 0.8, 10)
+    probs = torch.softmax(vals, -1)
+    counts = torch.bincount(toks, minlength=vocab).float()
+    assert counts.sum() == counts[idx].sum()           # nothing outside the top k
+    chi2 = (((counts[idx] - probs * n) ** 2) / (probs * n)).sum().item()
+    assert chi2 < 40, chi2                              # 9 degrees of freedom; 40 is far in the tail

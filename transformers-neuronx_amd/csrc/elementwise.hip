@@ -1,0 +1,154 @@
+// Row gathers, the position add at the input, casts, LayerNorm.
+#include "common.h"
+
+TNX_DEFINE_ERROR_API
+
+// out[m, :] = src[idx[m], :], rows of `row_bytes` bytes (a multiple of 4).
+__global__ void gather_rows_kernel(const uint32_t* __restrict__ src, const int* __restrict__ idx,
+                                   uint32_t* __restrict__ out, int words, int src_rows) {
+  const int m = blockIdx.x;
+  const int r = idx[m];
+  if (r < 0 || r >= src_rows) return;  // the host checks ids; an id out of range writes nothing
+  const uint32_t* s = src + (size_t)r * words;
+  uint32_t* o = out + (size_t)m * words;
+  for (int i = threadIdx.x; i < words; i += blockDim.x) o[i] = s[i];
+}
+
+extern "C" int tnx_gather_rows(const void* src, const int* idx, void* out, int m, int row_bytes, int src_rows,
+                               hipStream_t stream) {
+  TNX_REQUIRE(row_bytes > 0 && row_bytes % 4 == 0, "gather_rows: row of %d bytes is not a multiple of 4", row_bytes);
+  TNX_REQUIRE(m >= 0 && src_rows > 0, "gather_rows: bad sizes m=%d rows=%d", m, src_rows);
+  if (m == 0) return 0;
+  gather_rows_kernel<<<m, 256, 0, stream>>>((const uint32_t*)src, idx, (uint32_t*)out, row_bytes / 4, src_rows);
+  TNX_CHECK_LAUNCH("gather_rows");
+  return 0;
+}
+
+// x[t, :] = src[t, :] + table[positions[t] + offset, :] in float32; a copy in `cd_dtype` beside it.
+__global__ void add_positions_kernel(const void* __restrict__ src, int src_dtype, const int* __restrict__ positions,
+                                     const void* __restrict__ table, int table_dtype, int table_rows, int offset,
+                                     float* __restrict__ out_f32, void* __restrict__ out_cd, int cd_dtype, int width) {
+  const int t = blockIdx.x;
+  size_t base = (size_t)t * width;
+  int row = table ? positions[t] + offset : 0;
+  if (table && (row < 0 || row >= table_rows)) row = 0;  // the host checks positions
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = load_any(src, src_dtype, base + i);
+    if (table) v += load_any(table, table_dtype, (size_t)row * width + i);
+    out_f32[base + i] = v;
+    if (out_cd) store_any(out_cd, cd_dtype, base + i, v);
+  }
+}
+
+extern "C" int tnx_add_positions(const void* src, int src_dtype, const int* positions, const void* table,
+                                 int table_dtype, int table_rows, int offset, float* out_f32, void* out_cd,
+                                 int cd_dtype, int tokens, int width, hipStream_t stream) {
+  TNX_REQUIRE(tokens >= 0 && width > 0, "add_positions: bad sizes tokens=%d width=%d", tokens, width);
+  if (tokens == 0) return 0;
+  add_positions_kernel<<<tokens, 256, 0, stream>>>(src, src_dtype, positions, table, table_dtype, table_rows, offset,
+                                                   out_f32, out_cd, cd_dtype, width);
+  TNX_CHECK_LAUNCH("add_positions");
+  return 0;
+}
+
+__global__ void cast_kernel(const void* __restrict__ src, int src_dtype, void* __restrict__ dst, int dst_dtype,
+                            size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) store_any(dst, dst_dtype, i, load_any(src, src_dtype, i));
+}
+
+extern "C" int tnx_cast(const void* src, int src_dtype, void* dst, int dst_dtype, long long n, hipStream_t stream) {
+  TNX_REQUIRE(n >= 0, "cast: negative size");
+  if (n == 0) return 0;
+  long long blocks = (n + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  cast_kernel<<<(int)blocks, 256, 0, stream>>>(src, src_dtype, dst, dst_dtype, (size_t)n);
+  TNX_CHECK_LAUNCH("cast");
+  return 0;
+}
+
+// LayerNorm of float32 rows: mean and biased variance in float32 (two passes over the row:
+// the variance is taken around the mean, not as E[x^2] - mean^2), then weight and bias.
+// One block of 256 threads per row; the row is kept in registers when it fits (width <= 256 * PER).
+template <int PER>
+__global__ void __launch_bounds__(256)
+layernorm_kernel(const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ bias,
+                 float eps, float* __restrict__ out_f32, void* __restrict__ out_cd, int cd_dtype, int width) {
+  __shared__ float scratch[4];
+  const int t = blockIdx.x;
+  const float* row = x + (size_t)t * width;
+  float v[PER];
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int i = threadIdx.x + j * 256;
+    v[j] = i < width ? row[i] : 0.f;
+    s += v[j];
+  }
+  const float mean = block_sum<4>(s, scratch) / (float)width;
+  float q = 0.f;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int i = threadIdx.x + j * 256;
+    const float d = i < width ? v[j] - mean : 0.f;
+    q += d * d;
+  }
+  const float var = block_sum<4>(q, scratch) / (float)width;
+  const float rstd = rsqrtf(var + eps);
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int i = threadIdx.x + j * 256;
+    if (i < width) {
+      float y = (v[j] - mean) * rstd;
+      if (weight) y *= weight[i];
+      if (bias) y += bias[i];
+      if (out_f32) out_f32[(size_t)t * width + i] = y;
+      if (out_cd) store_any(out_cd, cd_dtype, (size_t)t * width + i, y);
+    }
+  }
+}
+
+// Any width: three passes over the row in memory.
+__global__ void __launch_bounds__(256)
+layernorm_wide_kernel(const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ bias,
+                      float eps, float* __restrict__ out_f32, void* __restrict__ out_cd, int cd_dtype, int width) {
+  __shared__ float scratch[4];
+  const int t = blockIdx.x;
+  const float* row = x + (size_t)t * width;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < width; i += 256) s += row[i];
+  const float mean = block_sum<4>(s, scratch) / (float)width;
+  float q = 0.f;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    const float d = row[i] - mean;
+    q += d * d;
+  }
+  const float var = block_sum<4>(q, scratch) / (float)width;
+  const float rstd = rsqrtf(var + eps);
+  for (int i = threadIdx.x; i < width; i += 256) {
+    float y = (row[i] - mean) * rstd;
+    if (weight) y *= weight[i];
+    if (bias) y += bias[i];
+    if (out_f32) out_f32[(size_t)t * width + i] = y;
+    if (out_cd) store_any(out_cd, cd_dtype, (size_t)t * width + i, y);
+  }
+}
+
+extern "C" int tnx_layernorm(const float* x, const float* weight, const float* bias, float eps, float* out_f32,
+                             void* out_cd, int cd_dtype, int tokens, int width, hipStream_t stream) {
+  TNX_REQUIRE(tokens >= 0 && width > 0, "layernorm: bad sizes tokens=%d width=%d", tokens, width);
+  TNX_REQUIRE(eps > 0.f, "layernorm: eps must be positive");
+  TNX_REQUIRE(out_f32 != x, "layernorm: the float32 output may not alias the input");
+  if (tokens == 0) return 0;
+  if (width <= 256 * 4)
+    layernorm_kernel<4><<<tokens, 256, 0, stream>>>(x, weight, bias, eps, out_f32, out_cd, cd_dtype, width);
+  else if (width <= 256 * 16)
+    layernorm_kernel<16><<<tokens, 256, 0, stream>>>(x, weight, bias, eps, out_f32, out_cd, cd_dtype, width);
+  else if (width <= 256 * 48)
+    layernorm_kernel<48><<<tokens, 256, 0, stream>>>(x, weight, bias, eps, out_f32, out_cd, cd_dtype, width);
+  else
+    layernorm_wide_kernel<<<tokens, 256, 0, stream>>>(x, weight, bias, eps, out_f32, out_cd, cd_dtype, width);
+  TNX_CHECK_LAUNCH("layernorm");
+  return 0;
+}

@@ -1,0 +1,256 @@
+// Matrix products `out[M, N] = act(x[M, K] w[N, K]^T + bias[N]) + residual[M, N]` with float32 accumulation.
+//   gemm_f32        float32 operands, plain FMA (no matrix-core mode of reduced precision)
+//   gemm_bf16       bfloat16 operands on MFMA, 128x128 tiles staged through LDS (many rows: prompts)
+//   gemm_bf16_skinny  bfloat16 operands on MFMA for M <= 64 (decoding): streams the weight once
+// bias and residual are float32 and optional; the output is float32 or bfloat16.
+#include "common.h"
+
+TNX_DEFINE_ERROR_API
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+__device__ __forceinline__ void epilogue_store(float v, int m, int n, int N, const float* bias, const float* residual,
+                                               void* out, int out_dtype, int act) {
+  if (bias) v += bias[n];
+  v = apply_act(v, act);
+  const size_t o = (size_t)m * N + n;
+  if (residual) v += residual[o];
+  store_any(out, out_dtype, o, v);
+}
+
+// ------------------------------------------------------------------------------------------ float32
+
+#define F32_TILE 64
+#define F32_BK 16
+
+__global__ void __launch_bounds__(256)
+gemm_f32_kernel(const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias,
+                const float* __restrict__ residual, void* __restrict__ out, int out_dtype, int act, int M, int N,
+                int K) {
+  __shared__ float xs[F32_BK][F32_TILE + 4];
+  __shared__ float ws[F32_BK][F32_TILE + 4];
+  const int tid = threadIdx.x;
+  const int tx = tid & 15, ty = tid >> 4;
+  const int m0 = blockIdx.y * F32_TILE, n0 = blockIdx.x * F32_TILE;
+  const int lrow = tid >> 2, lk = (tid & 3) * 4;  // this thread stages row lrow, k lk..lk+3 of both tiles
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+  for (int k0 = 0; k0 < K; k0 += F32_BK) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int k = k0 + lk + e;
+      const int m = m0 + lrow, n = n0 + lrow;
+      xs[lk + e][lrow] = (m < M && k < K) ? x[(size_t)m * K + k] : 0.f;
+      ws[lk + e][lrow] = (n < N && k < K) ? w[(size_t)n * K + k] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < F32_BK; ++k) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = xs[k][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = ws[k][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = m0 + ty * 4 + i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n < N) epilogue_store(acc[i][j], m, n, N, bias, residual, out, out_dtype, act);
+    }
+  }
+}
+
+extern "C" int tnx_gemm_f32(const float* x, const float* w, const float* bias, const float* residual, void* out,
+                            int out_dtype, int act, int M, int N, int K, hipStream_t stream) {
+  TNX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_f32: bad sizes M=%d N=%d K=%d", M, N, K);
+  if (M == 0) return 0;
+  dim3 grid((N + F32_TILE - 1) / F32_TILE, (M + F32_TILE - 1) / F32_TILE);
+  TNX_REQUIRE(grid.y <= 65535, "gemm_f32: M=%d is too large", M);
+  gemm_f32_kernel<<<grid, 256, 0, stream>>>(x, w, bias, residual, out, out_dtype, act, M, N, K);
+  TNX_CHECK_LAUNCH("gemm_f32");
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------ bfloat16, tiled
+
+#define BT_M 128
+#define BT_N 128
+#define BT_K 32
+#define BT_STRIDE 40  // elements per staged row: 32 of data, 8 of padding against LDS bank conflicts
+
+__global__ void __launch_bounds__(256)
+gemm_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
+                 const float* __restrict__ residual, void* __restrict__ out, int out_dtype, int act, int M, int N,
+                 int K) {
+  __shared__ __attribute__((aligned(16))) bf16_t xs[BT_M * BT_STRIDE];
+  __shared__ __attribute__((aligned(16))) bf16_t ws[BT_N * BT_STRIDE];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;
+  const int m0 = blockIdx.y * BT_M, n0 = blockIdx.x * BT_N;
+  const int l32 = lane & 31, lhalf = lane >> 5;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  bf16x8 rx[2], rw[2];
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int c = tid + 256 * j;
+      const int row = c >> 2, k = k0 + (c & 3) * 8;
+      const bool k_ok = k + 8 <= K;
+      rx[j] = (k_ok && m0 + row < M) ? *(const bf16x8*)(x + (size_t)(m0 + row) * K + k) : zero;
+      rw[j] = (k_ok && n0 + row < N) ? *(const bf16x8*)(w + (size_t)(n0 + row) * K + k) : zero;
+    }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += BT_K) {
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int c = tid + 256 * j;
+      const int row = c >> 2, kc = (c & 3) * 8;
+      *(bf16x8*)(xs + row * BT_STRIDE + kc) = rx[j];
+      *(bf16x8*)(ws + row * BT_STRIDE + kc) = rw[j];
+    }
+    __syncthreads();
+    if (k0 + BT_K < K) fetch(k0 + BT_K);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      bf16x8 a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) a[i] = *(const bf16x8*)(xs + (wm + i * 32 + l32) * BT_STRIDE + ks * 16 + lhalf * 8);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) b[j] = *(const bf16x8*)(ws + (wn + j * 32 + l32) * BT_STRIDE + ks * 16 + lhalf * 8);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+  }
+  // acc[i][j][e] is row 8*(e/4) + 4*(lane/32) + e%4, column lane%32 of its 32x32 tile.
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = n0 + wn + j * 32 + l32;
+      if (n >= N) continue;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = m0 + wm + i * 32 + 8 * (e >> 2) + 4 * lhalf + (e & 3);
+        if (m < M) epilogue_store(acc[i][j][e], m, n, N, bias, residual, out, out_dtype, act);
+      }
+    }
+}
+
+// ------------------------------------------------------------------------------------------ bfloat16, few rows
+
+// One block of four waves makes 16 columns of the output (16 rows of `w`) for all M <= 16 * MT rows of `x`.
+// The waves share the K axis in steps of 128; inside a step a lane reads 64 contiguous bytes of its weight
+// row, which the four MFMA steps consume in the same order from `x`, so the order of the sum over K is the
+// lane's own and needs no shuffle. The partial sums of the four waves meet in LDS.
+template <int MT>
+__global__ void __launch_bounds__(256)
+gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
+                        const float* __restrict__ residual, void* __restrict__ out, int out_dtype, int act, int M,
+                        int N, int K) {
+  __shared__ float red[4][MT][4][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const bool n_ok = n0 + r < N;
+  const bf16_t* wrow = w + (size_t)(n_ok ? n0 + r : 0) * K;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  for (int kb = wave * 128; kb < K; kb += 512) {
+    const int k_lane = kb + 32 * g;
+    bf16x8 wf[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int k = k_lane + 8 * s;
+      wf[s] = (n_ok && k + 8 <= K) ? *(const bf16x8*)(wrow + k) : zero;
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const int m = t * 16 + r;
+      const bf16_t* xrow = x + (size_t)(m < M ? m : 0) * K;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const int k = k_lane + 8 * s;
+        const bf16x8 xf = (m < M && k + 8 <= K) ? *(const bf16x8*)(xrow + k) : zero;
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s], xf, acc[t], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][t][i][lane] = acc[t][i];
+  __syncthreads();
+  // acc[t][i] of lane l is output column n0 + 4*(l/16) + i, row 16*t + l%16.
+  for (int idx = tid; idx < MT * 256; idx += 256) {
+    const int t = idx >> 8, i = (idx >> 6) & 3, l = idx & 63;
+    const float v = red[0][t][i][l] + red[1][t][i][l] + red[2][t][i][l] + red[3][t][i][l];
+    const int n = n0 + 4 * (l >> 4) + i, m = t * 16 + (l & 15);
+    if (n < N && m < M) epilogue_store(v, m, n, N, bias, residual, out, out_dtype, act);
+  }
+}
+
+extern "C" int tnx_gemm_bf16(const void* x, const void* w, const float* bias, const float* residual, void* out,
+                             int out_dtype, int act, int M, int N, int K, int force_tiled, hipStream_t stream) {
+  TNX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
+  TNX_REQUIRE(K % 8 == 0, "gemm_bf16: the inner size K=%d must be a multiple of 8", K);
+  TNX_REQUIRE(((uintptr_t)x | (uintptr_t)w) % 16 == 0, "gemm_bf16: operands must be 16-byte aligned");
+  if (M == 0) return 0;
+  const bf16_t* xp = (const bf16_t*)x;
+  const bf16_t* wp = (const bf16_t*)w;
+  if (M <= 64 && !force_tiled) {
+    const int blocks = (N + 15) / 16;
+    switch ((M + 15) / 16) {
+      case 1:
+        gemm_bf16_skinny_kernel<1><<<blocks, 256, 0, stream>>>(xp, wp, bias, residual, out, out_dtype, act, M, N, K);
+        break;
+      case 2:
+        gemm_bf16_skinny_kernel<2><<<blocks, 256, 0, stream>>>(xp, wp, bias, residual, out, out_dtype, act, M, N, K);
+        break;
+      case 3:
+        gemm_bf16_skinny_kernel<3><<<blocks, 256, 0, stream>>>(xp, wp, bias, residual, out, out_dtype, act, M, N, K);
+        break;
+      default:
+        gemm_bf16_skinny_kernel<4><<<blocks, 256, 0, stream>>>(xp, wp, bias, residual, out, out_dtype, act, M, N, K);
+        break;
+    }
+    TNX_CHECK_LAUNCH("gemm_bf16_skinny");
+    return 0;
+  }
+  dim3 grid((N + BT_N - 1) / BT_N, (M + BT_M - 1) / BT_M);
+  TNX_REQUIRE(grid.y <= 65535, "gemm_bf16: M=%d is too large", M);
+  gemm_bf16_kernel<<<grid, 256, 0, stream>>>(xp, wp, bias, residual, out, out_dtype, act, M, N, K);
+  TNX_CHECK_LAUNCH("gemm_bf16");
+  return 0;
+}

@@ -1,0 +1,274 @@
+// Token selection from float32 logits: argmax, and temperature / top-k / top-p sampling with a draw by
+// inverse CDF from a counter-based random number (Philox-4x32-10, keyed by the request's seed, counter =
+// the request's step), so that a request's draws do not depend on what else is in the batch.
+//
+// Order among tokens is total: by logit, ties to the lower token id (a 64-bit key: ordered logit bits above
+// the inverted token id). Top-k keeps the k largest keys. Top-p keeps, of those, every token whose
+// predecessors in descending order hold less than top_p of the softmax mass (the first token always).
+// Both thresholds are found by radix selection, eight bits at a time, without sorting. The draw runs over
+// the kept tokens in ascending order of token id.
+#include "common.h"
+
+TNX_DEFINE_ERROR_API
+
+#define SAMPLE_THREADS 1024
+
+__device__ __forceinline__ uint64_t order_key(float x, int idx) {
+  if (x != x) x = -INFINITY;  // NaN orders last
+  uint32_t u = __float_as_uint(x);
+  u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+  return ((uint64_t)u << 32) | (uint32_t)(~(uint32_t)idx);
+}
+
+__device__ __forceinline__ float philox_uniform(uint64_t seed, uint64_t counter) {
+  const uint32_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u, W0 = 0x9E3779B9u, W1 = 0xBB67AE85u;
+  uint32_t c0 = (uint32_t)counter, c1 = (uint32_t)(counter >> 32), c2 = 0, c3 = 0;
+  uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint32_t hi0 = __umulhi(M0, c0), lo0 = M0 * c0;
+    const uint32_t hi1 = __umulhi(M1, c2), lo1 = M1 * c2;
+    const uint32_t n0 = hi1 ^ c1 ^ k0, n1 = lo1, n2 = hi0 ^ c3 ^ k1, n3 = lo0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += W0; k1 += W1;
+  }
+  return (float)(c0 >> 8) * (1.0f / 16777216.0f);
+}
+
+__global__ void __launch_bounds__(256)
+argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int vocab) {
+  __shared__ unsigned long long best[4];
+  const float* row = logits + (size_t)blockIdx.x * vocab;
+  uint64_t b = 0;
+  for (int i = threadIdx.x; i < vocab; i += 256) {
+    const uint64_t k = order_key(row[i], i);
+    b = k > b ? k : b;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const uint64_t other = __shfl_xor((unsigned long long)b, o, 64);
+    b = other > b ? other : b;
+  }
+  if ((threadIdx.x & 63) == 0) best[threadIdx.x >> 6] = b;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w) b = best[w] > b ? best[w] : b;
+    out[blockIdx.x] = (int)(~(uint32_t)b);
+  }
+}
+
+extern "C" int tnx_argmax(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
+  TNX_REQUIRE(rows >= 0 && vocab > 0, "argmax: bad sizes rows=%d vocab=%d", rows, vocab);
+  if (rows == 0) return 0;
+  argmax_kernel<<<rows, 256, 0, stream>>>(logits, out, vocab);
+  TNX_CHECK_LAUNCH("argmax");
+  return 0;
+}
+
+// One block per row.
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature, const int* __restrict__ top_k,
+              const float* __restrict__ top_p, const long long* __restrict__ seeds,
+              const long long* __restrict__ counters, int* __restrict__ out, int vocab) {
+  __shared__ unsigned int cnt[256];
+  __shared__ float mass[256];
+  __shared__ float part[SAMPLE_THREADS];
+  __shared__ float wsum[16];
+  __shared__ unsigned long long best[16];
+  __shared__ int sh_digit;
+  __shared__ unsigned int sh_remaining, sh_bin;
+  __shared__ float sh_above, sh_total;
+  __shared__ int sh_result, sh_last;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rowi = blockIdx.x;
+  const float* row = logits + (size_t)rowi * vocab;
+  const float temp = temperature[rowi];
+
+  // the largest key: argmax, and the maximum for the softmax
+  uint64_t b = 0;
+  for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
+    const uint64_t k = order_key(row[i], i);
+    b = k > b ? k : b;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const uint64_t other = __shfl_xor((unsigned long long)b, o, 64);
+    b = other > b ? other : b;
+  }
+  if (lane == 0) best[wave] = b;
+  __syncthreads();
+  b = best[0];
+  for (int w = 1; w < 16; ++w) b = best[w] > b ? best[w] : b;
+  const int arg = (int)(~(uint32_t)b);
+  if (!(temp > 0.f)) {
+    if (tid == 0) out[rowi] = arg;
+    return;
+  }
+  const float inv_temp = 1.f / temp;
+  const float xmax = row[arg] * inv_temp;
+
+  // top-k: the k-th largest key
+  uint64_t floor_key = 0;  // tokens with key >= floor_key are kept
+  const int k = top_k[rowi];
+  if (k > 0 && k < vocab) {
+    uint64_t prefix = 0, mask = 0;
+    unsigned int remaining = (unsigned int)k;
+    for (int pass = 0; pass < 8; ++pass) {
+      const int shift = 56 - 8 * pass;
+      if (tid < 256) cnt[tid] = 0;
+      __syncthreads();
+      for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
+        const uint64_t key = order_key(row[i], i);
+        if ((key & mask) == prefix) atomicAdd(&cnt[(unsigned int)(key >> shift) & 255u], 1u);
+      }
+      __syncthreads();
+      if (tid == 0) {
+        unsigned int rem = remaining;
+        int d = 255;
+        for (; d > 0; --d) {
+          if (cnt[d] >= rem) break;
+          rem -= cnt[d];
+        }
+        sh_digit = d;
+        sh_remaining = rem;
+        sh_bin = cnt[d];
+      }
+      __syncthreads();
+      prefix |= (uint64_t)sh_digit << shift;
+      mask |= 0xFFull << shift;
+      remaining = sh_remaining;
+      const bool whole_bin = sh_bin == remaining;
+      __syncthreads();
+      if (whole_bin) break;  // everything under this prefix is kept: the threshold is the prefix itself
+    }
+    floor_key = prefix;
+  }
+
+  // top-p: the smallest kept key is the last one whose predecessors hold less than p of the mass
+  const float p = top_p[rowi];
+  if (p < 1.f) {
+    float z = 0.f;
+    for (int i = tid; i < vocab; i += SAMPLE_THREADS)
+      if (order_key(row[i], i) >= floor_key) z += __expf(row[i] * inv_temp - xmax);
+    z = wave_sum(z);
+    if (lane == 0) wsum[wave] = z;
+    __syncthreads();
+    z = 0.f;
+    for (int w = 0; w < 16; ++w) z += wsum[w];
+    const float target = p * z;
+    uint64_t prefix = 0, mask = 0;
+    float above = 0.f;
+    for (int pass = 0; pass < 8; ++pass) {
+      const int shift = 56 - 8 * pass;
+      if (tid < 256) {
+        cnt[tid] = 0;
+        mass[tid] = 0.f;
+      }
+      __syncthreads();
+      for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
+        const uint64_t key = order_key(row[i], i);
+        if (key >= floor_key && (key & mask) == prefix) {
+          const unsigned int d = (unsigned int)(key >> shift) & 255u;
+          atomicAdd(&cnt[d], 1u);
+          atomicAdd(&mass[d], __expf(row[i] * inv_temp - xmax));
+        }
+      }
+      __syncthreads();
+      if (tid == 0) {
+        float running = above, chosen_above = above;
+        int chosen = -1;
+        for (int d = 255; d >= 0; --d) {
+          if (cnt[d] == 0) continue;
+          if (running < target || chosen < 0) {
+            chosen = d;
+            chosen_above = running;
+          } else {
+            break;
+          }
+          running += mass[d];
+        }
+        sh_digit = chosen;
+        sh_above = chosen_above;
+        sh_bin = cnt[chosen];
+      }
+      __syncthreads();
+      prefix |= (uint64_t)sh_digit << shift;
+      mask |= 0xFFull << shift;
+      above = sh_above;
+      const bool single = sh_bin == 1;
+      __syncthreads();
+      if (single) break;
+    }
+    floor_key = prefix > floor_key ? prefix : floor_key;
+  }
+
+  // the draw, over the kept tokens in ascending order of token id; thread t owns a contiguous segment
+  const int seg = (vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  const int i0 = tid * seg, i1 = min(vocab, i0 + seg);
+  float s = 0.f;
+  int last = -1;
+  for (int i = i0; i < i1; ++i)
+    if (order_key(row[i], i) >= floor_key) {
+      s += __expf(row[i] * inv_temp - xmax);
+      last = i;
+    }
+  if (tid == 0) {
+    sh_result = -1;
+    sh_last = -1;
+  }
+  part[tid] = s;
+  __syncthreads();
+  if (last >= 0) atomicMax(&sh_last, last);
+  // exclusive scan of part[] by one wave: 16 values per lane
+  if (wave == 0) {
+    float local[16];
+    float run = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      local[j] = run;
+      run += part[lane * 16 + j];
+    }
+    float incl = run;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const float v = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += v;
+    }
+    const float base = incl - run;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) part[lane * 16 + j] = base + local[j];
+    if (lane == 63) sh_total = incl;
+  }
+  __syncthreads();
+  const float u = philox_uniform((uint64_t)seeds[rowi], (uint64_t)counters[rowi]);
+  const float goal = u * sh_total;
+  // thread t owns [base_t, base_{t+1}): the scanned values tile the line without gaps
+  const float base = part[tid];
+  const float next = tid + 1 < SAMPLE_THREADS ? part[tid + 1] : INFINITY;
+  if (last >= 0 && base <= goal && goal < next) {
+    float run = base;
+    int pick = last;
+    for (int i = i0; i < i1; ++i)
+      if (order_key(row[i], i) >= floor_key) {
+        run += __expf(row[i] * inv_temp - xmax);
+        if (run > goal) {
+          pick = i;
+          break;
+        }
+      }
+    atomicMax(&sh_result, pick);
+  }
+  __syncthreads();
+  if (tid == 0) out[rowi] = sh_result >= 0 ? sh_result : sh_last;
+}
+
+extern "C" int tnx_sample(const float* logits, const float* temperature, const int* top_k, const float* top_p,
+                          const long long* seeds, const long long* counters, int* out, int rows, int vocab,
+                          hipStream_t stream) {
+  TNX_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
+  if (rows == 0) return 0;
+  sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, temperature, top_k, top_p, seeds, counters, out, vocab);
+  TNX_CHECK_LAUNCH("sample");
+  return 0;
+}

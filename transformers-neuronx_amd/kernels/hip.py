@@ -1,0 +1,267 @@
+"""The product kernel backend: hand-written HIP for gfx950 behind a C interface.
+
+Each call checks shapes and dtypes on the host, launches on torch's current
+stream and raises with the library's message if the library refuses. torch is
+the allocator and nothing else here. A missing library is compiled at first use;
+if that fails the call fails: there is no other path.
+"""
+import ctypes
+from typing import Dict, Optional
+
+import torch
+
+from . import build
+
+_F32, _BF16 = 0, 1
+_ACT = {None: 0, "none": 0, "relu": 1, "gelu": 2, "gelu_new": 3}
+_LIBS: Dict[str, ctypes.CDLL] = {}
+
+_c_void_p, _c_int, _c_float, _c_ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_longlong
+
+_SIGNATURES = {
+    "elementwise": {
+        "tnx_gather_rows": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_add_positions": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
+                              _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_cast": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_void_p],
+        "tnx_layernorm": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+                          _c_void_p],
+    },
+    "gemm": {
+        "tnx_gemm_f32": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
+                         _c_int, _c_void_p],
+        "tnx_gemm_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
+                          _c_int, _c_int, _c_void_p],
+    },
+    "attention": {
+        "tnx_qkv_write": [_c_void_p, _c_int, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
+                          _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_attention_any": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
+                              _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    },
+    "sampling": {
+        "tnx_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+        "tnx_sample": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
+                       _c_void_p],
+    },
+}
+
+
+def library(module: str) -> ctypes.CDLL:
+    """The compiled library of a kernel module, compiled now if it is not there."""
+    lib = _LIBS.get(module)
+    if lib is None:
+        path = build.find_library(module) or build.compile_module(module)
+        lib = ctypes.CDLL(path)
+        lib.tnx_last_error.restype = ctypes.c_char_p
+        for name, argtypes in _SIGNATURES[module].items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = _c_int
+        _LIBS[module] = lib
+    return lib
+
+
+def loaded_libraries() -> Dict[str, str]:
+    return {m: lib._name for m, lib in _LIBS.items()}
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return _F32
+    if dtype == torch.bfloat16:
+        return _BF16
+    raise TypeError(f"the kernels take float32 and bfloat16, not {dtype}")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _want(t: torch.Tensor, name: str, dtype=None, shape=None):
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be on the GPU")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+    return t
+
+
+class HipOps:
+    name = "hip"
+
+    def __init__(self, dtype: torch.dtype, device="cuda:0"):
+        self.dtype = dtype
+        self.device = torch.device(device)
+        if self.device.type != "cuda" or not torch.cuda.is_available():
+            raise RuntimeError("the HIP kernels need a GPU; none is visible to torch")
+        _code(dtype)
+
+    def _call(self, module: str, fn: str, *args):
+        lib = library(module)
+        rc = getattr(lib, fn)(*args)
+        if rc != 0:
+            raise RuntimeError(f"{fn}: {lib.tnx_last_error().decode()}")
+
+    # ---------------------------------------------------------------- input end
+
+    def gather_rows(self, x, rows):
+        _want(x, "x")
+        _want(rows, "rows", torch.int32)
+        if x.dim() != 2:
+            raise ValueError("gather_rows takes a matrix")
+        out = torch.empty(rows.numel(), x.shape[1], dtype=x.dtype, device=x.device)
+        self._call("elementwise", "tnx_gather_rows", _ptr(x), _ptr(rows), _ptr(out), rows.numel(),
+                   x.shape[1] * x.element_size(), x.shape[0], _stream())
+        return out
+
+    def embed(self, token_ids, table, dtype=None):
+        return self.gather_rows(table, token_ids)
+
+    def add_positions(self, src, positions, table, offset, dtype, want_compute):
+        _want(src, "src")
+        t, width = src.shape
+        _want(positions, "positions", torch.int32, (t,))
+        _want(table, "position table")
+        if table.shape[1] != width:
+            raise ValueError(f"position table is {table.shape[1]} wide, the tokens {width}")
+        out = torch.empty(t, width, dtype=torch.float32, device=src.device)
+        cd = torch.empty(t, width, dtype=dtype, device=src.device) if want_compute and dtype != torch.float32 else None
+        self._call("elementwise", "tnx_add_positions", _ptr(src), _code(src.dtype), _ptr(positions), _ptr(table),
+                   _code(table.dtype), table.shape[0], offset, _ptr(out), _ptr(cd), _code(dtype), t, width, _stream())
+        return out, ((cd if cd is not None else out) if want_compute else None)
+
+    def to_stream(self, src, dtype, want_compute):
+        _want(src, "src")
+        t, width = src.shape
+        out = torch.empty(t, width, dtype=torch.float32, device=src.device)
+        cd = torch.empty(t, width, dtype=dtype, device=src.device) if want_compute and dtype != torch.float32 else None
+        self._call("elementwise", "tnx_add_positions", _ptr(src), _code(src.dtype), None, None, 0, 0, 0, _ptr(out),
+                   _ptr(cd), _code(dtype), t, width, _stream())
+        return out, ((cd if cd is not None else out) if want_compute else None)
+
+    def cast(self, x, dtype):
+        _want(x, "x")
+        if x.dtype == dtype:
+            return x
+        out = torch.empty_like(x, dtype=dtype)
+        self._call("elementwise", "tnx_cast", _ptr(x), _code(x.dtype), _ptr(out), _code(dtype), x.numel(), _stream())
+        return out
+
+    # ---------------------------------------------------------------- norms
+
+    def layernorm(self, x, weight, bias, eps, dtype, want_f32, want_compute):
+        _want(x, "x", torch.float32)
+        t, width = x.shape
+        if weight is not None:
+            _want(weight, "norm weight", torch.float32, (width,))
+        if bias is not None:
+            _want(bias, "norm bias", torch.float32, (width,))
+        same = dtype == torch.float32
+        out_f32 = torch.empty_like(x) if (want_f32 or (want_compute and same)) else None
+        out_cd = torch.empty(t, width, dtype=dtype, device=x.device) if (want_compute and not same) else None
+        self._call("elementwise", "tnx_layernorm", _ptr(x), _ptr(weight), _ptr(bias), float(eps), _ptr(out_f32),
+                   _ptr(out_cd), _code(dtype), t, width, _stream())
+        return (out_f32 if want_f32 else None), ((out_f32 if same else out_cd) if want_compute else None)
+
+    # ---------------------------------------------------------------- matrix products
+
+    def linear(self, x, w, bias=None, act=None, residual=None, out_f32=False, force_tiled=False):
+        _want(x, "x")
+        _want(w, "w")
+        if act not in _ACT:
+            raise ValueError(f"unknown activation {act!r}")
+        m, k = x.shape
+        n, kw = w.shape
+        if kw != k:
+            raise ValueError(f"x is {k} wide, w takes {kw}")
+        if bias is not None:
+            _want(bias, "bias", torch.float32, (n,))
+        if residual is not None:
+            _want(residual, "residual", torch.float32, (m, n))
+        out_dtype = torch.float32 if out_f32 else self.dtype
+        out = torch.empty(m, n, dtype=out_dtype, device=x.device)
+        if w.dtype == torch.float32:
+            xa = self.cast(x, torch.float32)
+            self._call("gemm", "tnx_gemm_f32", _ptr(xa), _ptr(w), _ptr(bias), _ptr(residual), _ptr(out),
+                       _code(out_dtype), _ACT[act], m, n, k, _stream())
+        else:
+            xa = self.cast(x, torch.bfloat16)
+            self._call("gemm", "tnx_gemm_bf16", _ptr(xa), _ptr(w), _ptr(bias), _ptr(residual), _ptr(out),
+                       _code(out_dtype), _ACT[act], m, n, k, int(force_tiled), _stream())
+        return out
+
+    # ---------------------------------------------------------------- attention
+
+    def _check_pages(self, k_pages, v_pages, num_kv, head_size, page_size):
+        _want(k_pages, "key pages", self.dtype)
+        _want(v_pages, "value pages", self.dtype)
+        n = k_pages.shape[0]
+        if tuple(k_pages.shape) != (n, num_kv, page_size, head_size):
+            raise ValueError(f"key pages have shape {tuple(k_pages.shape)}, expected "
+                             f"{(n, num_kv, page_size, head_size)}")
+        if tuple(v_pages.shape) != (n, num_kv, head_size, page_size):
+            raise ValueError(f"value pages have shape {tuple(v_pages.shape)}, expected "
+                             f"{(n, num_kv, head_size, page_size)}")
+        return n
+
+    def qkv_write(self, qkv, bias, num_heads, num_kv_write, head_size, scale, ctx, view, k_pages, v_pages):
+        t = ctx.num_tokens
+        total = (num_heads + 2 * num_kv_write) * head_size
+        _want(qkv, "qkv", self.dtype, (t, total))
+        if bias is not None:
+            _want(bias, "qkv bias", torch.float32, (total,))
+        num_pages = 0
+        if num_kv_write:
+            num_pages = self._check_pages(k_pages, v_pages, num_kv_write, head_size, view.page_size)
+        _want(view.block_table, "block table", torch.int32, (ctx.num_requests, view.width))
+        q = torch.empty(t, num_heads * head_size, dtype=self.dtype, device=qkv.device)
+        self._call("attention", "tnx_qkv_write", _ptr(qkv), _code(self.dtype), _ptr(bias), float(scale),
+                   _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width, view.page_size,
+                   num_pages, _ptr(q), _ptr(k_pages) if num_kv_write else None,
+                   _ptr(v_pages) if num_kv_write else None, t, num_heads, num_kv_write, head_size, _stream())
+        return q
+
+    def attention(self, q, num_heads, num_kv_heads, head_size, ctx, view, k_pages, v_pages, window=None):
+        t = ctx.num_tokens
+        _want(q, "q", self.dtype, (t, num_heads * head_size))
+        num_pages = self._check_pages(k_pages, v_pages, num_kv_heads, head_size, view.page_size)
+        _want(view.block_table, "block table", torch.int32, (ctx.num_requests, view.width))
+        if ctx.max_total > view.width * view.page_size:
+            raise ValueError("a request is longer than its block table")
+        out = torch.empty_like(q)
+        self._call("attention", "tnx_attention_any", _ptr(q), _code(self.dtype), _ptr(k_pages), _ptr(v_pages),
+                   _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width, view.page_size,
+                   num_pages, _ptr(out), t, num_heads, num_kv_heads, head_size, int(window or 0), _stream())
+        return out
+
+    # ---------------------------------------------------------------- output end
+
+    def argmax(self, logits):
+        _want(logits, "logits", torch.float32)
+        out = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device)
+        self._call("sampling", "tnx_argmax", _ptr(logits), _ptr(out), logits.shape[0], logits.shape[1], _stream())
+        return out
+
+    def sample(self, logits, temperature, top_k, top_p, seeds, counters):
+        _want(logits, "logits", torch.float32)
+        m = logits.shape[0]
+        _want(temperature, "temperature", torch.float32, (m,))
+        _want(top_k, "top_k", torch.int32, (m,))
+        _want(top_p, "top_p", torch.float32, (m,))
+        _want(seeds, "seeds", torch.int64, (m,))
+        _want(counters, "counters", torch.int64, (m,))
+        out = torch.empty(m, dtype=torch.int32, device=logits.device)
+        self._call("sampling", "tnx_sample", _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(seeds),
+                   _ptr(counters), _ptr(out), m, logits.shape[1], _stream())
+        return out
+
+    def synchronize(self):
+        torch.cuda.synchronize(self.device)
