@@ -1,0 +1,155 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine at OPT-6.7B size with random weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One JSON line: `value` is decoded tokens per second at batch 8 and a 2,048-token context
+(a "step" is one decode step of the whole engine: schedule, model, sampling);
+`prefill` is one 2,048-token prompt in one step; `roofline` sets the bytes a decode step has
+to read (every weight once, and the cache of the live requests) against its time; `points`
+holds decoding at batch 1 and 64. The measuring follows the reference's own benchmark
+(generation_demo.py:107-187: warm-up runs, then timed ones; random token ids as prompts,
+:492-494). Weights and prompts are synthetic and seeded; there are no published numbers of
+the reference to compare with, so `vs_baseline` is null.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# OPT-6.7B: the sizes of BASELINE.json's configs[2]
+MODEL = dict(architectures=["OPTForCausalLM"], model_type="opt", vocab_size=50272, hidden_size=4096,
+             num_hidden_layers=32, num_attention_heads=32, ffn_dim=16384, max_position_embeddings=2048,
+             word_embed_proj_dim=4096, do_layer_norm_before=True, activation_function="relu", enable_bias=True,
+             layer_norm_elementwise_affine=True, init_std=0.02, torch_dtype="bfloat16")
+CONTEXT = 2048
+PREFILL_TOKENS = 2048
+PEAK_HBM_GBS = 8000.0                      # MI355X, published
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+
+def prefill_flops(cfg, tokens):
+    """Multiply-adds times two of one whole prompt: the matrix products of every layer, causal
+    attention (half of the square), and the head for the last token."""
+    h, f, l = cfg["hidden_size"], cfg["ffn_dim"], cfg["num_hidden_layers"]
+    linear = 2 * tokens * l * (4 * h * h + 2 * h * f)
+    attention = l * 2 * 2 * h * tokens * (tokens + 1) / 2
+    head = 2 * cfg["vocab_size"] * cfg["word_embed_proj_dim"]
+    return linear + attention + head
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
+        return 2
+
+    import torch
+    from transformers_neuronx_amd.config import EngineConfig, OPTConfig
+    from transformers_neuronx_amd.engine.engine import LLMEngine
+    from transformers_neuronx_amd.engine.factory import runner_from_random
+    from transformers_neuronx_amd.sampling import SamplingParams
+
+    raw = dict(MODEL)
+    layers_full = raw["num_hidden_layers"]
+    if args.layers:
+        raw["num_hidden_layers"] = args.layers
+    cfg = OPTConfig.from_dict(raw)
+    dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    max_batch = args.batch if args.no_points else max(args.batch, 64)
+    ecfg = EngineConfig(dtype=dtype, page_size=64, max_tokens=max_batch * CONTEXT, max_num_seqs=max_batch,
+                        max_num_batched_tokens=max(2048, PREFILL_TOKENS), max_model_len=CONTEXT)
+    t0 = time.time()
+    runner = runner_from_random(cfg, seed=0, cfg=ecfg)
+    torch.cuda.synchronize()
+    print(f"[bench] model ready in {time.time() - t0:.1f} s "
+          f"({runner.model.weight_bytes / 1e9:.2f} GB of weights)", file=sys.stderr, flush=True)
+    engine = LLMEngine(runner, ecfg)
+    item = 2 if dtype == torch.bfloat16 else 4
+    kv_bytes_per_token = 2 * cfg.num_hidden_layers * cfg.hidden_size * item
+    gen = torch.Generator().manual_seed(1)
+
+    def decode(batch, steps, warmup):
+        """Tokens per second, seconds per step and bytes per step of `steps` decode steps that end at
+        the full context."""
+        engine.reset()
+        prompt_len = CONTEXT - (steps + warmup) - 1
+        params = SamplingParams(max_new_tokens=steps + warmup + 1, do_sample=False, ignore_eos=True)
+        for _ in range(batch):
+            engine.add_request(torch.randint(3, cfg.vocab_size, (prompt_len,), generator=gen).tolist(), params)
+        while any(not r.decoding for r in engine.requests.values()):
+            engine.step()
+        for _ in range(warmup):
+            engine.step()
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        lens = 0
+        for _ in range(steps):
+            lens += sum(r.num_computed for r in engine.requests.values())
+            engine.step()
+        torch.cuda.synchronize()
+        sec = (time.perf_counter() - start) / steps
+        read = runner.model.weight_bytes + lens / steps * kv_bytes_per_token
+        return batch / sec, sec, read
+
+    def prefill(tokens):
+        engine.reset()
+        params = SamplingParams(max_new_tokens=1, do_sample=False, ignore_eos=True)
+        times = []
+        for i in range(3):
+            engine.add_request(torch.randint(3, cfg.vocab_size, (tokens,), generator=gen).tolist(), params)
+            torch.cuda.synchronize()
+            start = time.perf_counter()
+            engine.step()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - start)
+        return min(times[1:])
+
+    value, sec, read = decode(args.batch, args.steps, args.warmup)
+    print(f"[bench] decode batch {args.batch}: {value:.1f} tok/s, {sec * 1e3:.2f} ms/step", file=sys.stderr, flush=True)
+    achieved = read / sec / 1e9
+    out = {
+        "metric": "OPT-6.7B decode tok/s @ batch 1/8/64; prefill tok/s @ 2,048 tokens",
+        "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic (seeded random weights and token ids)",
+        "config": {"model": "OPT-6.7B", "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "none",
+                   "layers": cfg.num_hidden_layers, "layers_of_model": layers_full, "hidden_size": cfg.hidden_size,
+                   "heads": cfg.num_attention_heads, "head_size": cfg.head_size, "ffn_dim": cfg.ffn_dim,
+                   "vocab_size": cfg.vocab_size, "max_positions": cfg.max_position_embeddings,
+                   "prompt_len": CONTEXT - args.steps - args.warmup - 1, "page_size": ecfg.page_size,
+                   "activation": cfg.activation_function, "pre_norm": cfg.do_layer_norm_before,
+                   "prefill_tokens": PREFILL_TOKENS},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+    }
+    if not args.no_points:
+        sec_p = prefill(PREFILL_TOKENS)
+        flops = prefill_flops(raw, PREFILL_TOKENS)
+        out["prefill"] = {"value": round(PREFILL_TOKENS / sec_p, 1), "tokens": PREFILL_TOKENS,
+                          "ms": round(sec_p * 1e3, 3), "frac": round(flops / sec_p / PEAK_FLOPS[args.dtype], 4)}
+        print(f"[bench] prefill: {out['prefill']}", file=sys.stderr, flush=True)
+        points = {}
+        for b, k, w in ((1, min(args.steps, 64), args.warmup), (64, min(args.steps, 32), min(args.warmup, 4))):
+            v, s, _ = decode(b, k, w)
+            points[f"decode_b{b}"] = round(v, 2)
+            print(f"[bench] decode batch {b}: {v:.1f} tok/s, {s * 1e3:.2f} ms/step", file=sys.stderr, flush=True)
+        out["points"] = points
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -65,6 +65,20 @@ extern "C" int tnx_argmax(const float* logits, int* out, int rows, int vocab, hi
   return 0;
 }
 
+// logits[row, token[row]] = -inf where token[row] >= 0: a token that must not be chosen.
+__global__ void ban_tokens_kernel(float* __restrict__ logits, const int* __restrict__ token, int rows, int vocab) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r < rows && token[r] >= 0 && token[r] < vocab) logits[(size_t)r * vocab + token[r]] = -INFINITY;
+}
+
+extern "C" int tnx_ban_tokens(float* logits, const int* token, int rows, int vocab, hipStream_t stream) {
+  TNX_REQUIRE(rows >= 0 && vocab > 0, "ban_tokens: bad sizes rows=%d vocab=%d", rows, vocab);
+  if (rows == 0) return 0;
+  ban_tokens_kernel<<<(rows + 63) / 64, 64, 0, stream>>>(logits, token, rows, vocab);
+  TNX_CHECK_LAUNCH("ban_tokens");
+  return 0;
+}
+
 // One block per row.
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature, const int* __restrict__ top_k,

@@ -1,0 +1,216 @@
+"""The scheduler: admits requests, cuts prompts into portions under a token
+budget, lets running requests decode, finishes them and frees what they hold.
+
+The reference has none: `ContinuousBatchingConfig` (config.py:73-103) declares
+capacities for a scheduler outside the repository, and its demo drives a fixed
+batch in lock-step (generation_demo.py:474-500). The decisions below are ours.
+
+Every decision is a function of arrival order, lengths and capacities only:
+  * each step first gives one token to every running request that is decoding,
+    then continues prompts in admission order, then admits waiting requests
+    while a slot, pages and budget remain; a portion is what is left of the
+    prompt, of the portion limit and of the budget, at least one token;
+  * when the pool cannot cover a scheduled token, nothing new is admitted and
+    the most recently admitted running request is put back: its pages and slot
+    are freed, it rejoins the head of the waiting queue and is computed again
+    from its first token later, generated tokens included (they are kept). A
+    lone request that does not fit raises `OutOfPages`;
+  * a request ends at its end-of-sequence token (unless told to ignore it), at
+    `max_new_tokens`, or at the length limit, and frees its pages in that step.
+"""
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Deque, Hashable, List, Optional
+
+from ..cache.manager import CacheManager
+from ..cache.pages import OutOfPages
+from ..sampling.params import SamplingParams
+
+
+@dataclass
+class Request:
+    req_id: Hashable
+    prompt: List[int]
+    params: SamplingParams
+    output: List[int] = field(default_factory=list)
+    num_computed: int = 0           # tokens whose keys and values are stored
+    finished: bool = False
+    finish_reason: Optional[str] = None
+    preemptions: int = 0
+    arrival: int = 0
+
+    @property
+    def tokens(self) -> List[int]:
+        return self.prompt + self.output
+
+    @property
+    def num_tokens(self) -> int:
+        return len(self.prompt) + len(self.output)
+
+    @property
+    def decoding(self) -> bool:
+        """All tokens but the newest are stored: the next step brings that one token."""
+        return len(self.output) > 0 and self.num_computed == self.num_tokens - 1
+
+
+@dataclass
+class ScheduledRun:
+    request: Request
+    start: int                      # first position of the portion
+    count: int                      # tokens in the portion
+
+    @property
+    def samples(self) -> bool:
+        """The portion ends at the request's newest token: its last logits pick the next one."""
+        return self.start + self.count == self.request.num_tokens
+
+
+class Scheduler:
+    def __init__(self, cache: CacheManager, max_num_seqs: int, max_num_batched_tokens: int, max_model_len: int,
+                 max_portion: Optional[int] = None):
+        self.cache = cache
+        self.max_num_seqs = min(max_num_seqs, cache.max_seqs)
+        self.max_num_batched_tokens = max_num_batched_tokens
+        self.max_model_len = max_model_len
+        self.max_portion = max_portion or max_num_batched_tokens
+        self.waiting: Deque[Request] = deque()
+        self.running: List[Request] = []        # in admission order
+        self.finished: List[Request] = []
+        self._arrivals = 0
+        self.num_preemptions = 0
+
+    # ---------------------------------------------------------------- arrivals
+
+    def add(self, request: Request) -> None:
+        """Queue a request; one that can never fit the length limit is refused here
+        (reference: opt/model.py:50-57 refuses a sequence longer than the position table)."""
+        if not request.prompt:
+            raise ValueError(f"request {request.req_id!r} has an empty prompt")
+        # the last generated token is never fed back, so it needs no position
+        need = len(request.prompt) + request.params.max_new_tokens - 1
+        if need > self.max_model_len:
+            raise ValueError(f"request {request.req_id!r} needs {need} positions "
+                             f"({len(request.prompt)} prompt + {request.params.max_new_tokens} new); "
+                             f"the limit is {self.max_model_len}")
+        request.arrival = self._arrivals
+        self._arrivals += 1
+        self.waiting.append(request)
+
+    @property
+    def has_work(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    # ---------------------------------------------------------------- one step's plan
+
+    def _preempt_last(self, keep: Request) -> bool:
+        """Put back the most recently admitted running request other than `keep`."""
+        for victim in reversed(self.running):
+            if victim is not keep:
+                self.running.remove(victim)
+                self.cache.free_request(victim.req_id)
+                victim.num_computed = 0
+                victim.preemptions += 1
+                self.num_preemptions += 1
+                self.waiting.appendleft(victim)
+                return True
+        return False
+
+    def _reserve(self, req: Request, new_len: int, planned: List[ScheduledRun]) -> bool:
+        """Pages for `req` up to `new_len`, putting later requests back if need be.
+        False if `req` itself had to give way."""
+        while True:
+            try:
+                self.cache.grow(req.req_id, new_len)
+                return True
+            except OutOfPages:
+                victim_pool = [r for r in self.running if r is not req]
+                if not victim_pool:
+                    raise OutOfPages(f"request {req.req_id!r} alone does not fit the page pool "
+                                     f"({new_len} tokens wanted)")
+                victim = self.running[-1]
+                if victim is req:
+                    # the newest request gives way to the older ones that are already planned
+                    self.running.remove(req)
+                    self.cache.free_request(req.req_id)
+                    req.num_computed = 0
+                    req.preemptions += 1
+                    self.num_preemptions += 1
+                    self.waiting.appendleft(req)
+                    return False
+                self._preempt_last(req)
+                planned[:] = [p for p in planned if p.request is not victim]
+
+    def schedule(self) -> List[ScheduledRun]:
+        budget = self.max_num_batched_tokens
+        planned: List[ScheduledRun] = []
+        blocked = False                       # pages ran out: admit nothing new this step
+        # 1. one token for every decoding request, oldest first
+        for req in list(self.running):
+            if req not in self.running or not req.decoding or budget <= 0:
+                continue
+            before = self.num_preemptions
+            if self._reserve(req, req.num_computed + 1, planned):
+                planned.append(ScheduledRun(req, req.num_computed, 1))
+                budget -= 1
+            blocked |= self.num_preemptions != before
+        # 2. the next portion of every prompt under way
+        for req in list(self.running):
+            if req not in self.running or req.decoding or budget <= 0:
+                continue
+            if any(p.request is req for p in planned):
+                continue
+            count = min(req.num_tokens - req.num_computed, self.max_portion, budget)
+            before = self.num_preemptions
+            if self._reserve(req, req.num_computed + count, planned):
+                planned.append(ScheduledRun(req, req.num_computed, count))
+                budget -= count
+            blocked |= self.num_preemptions != before
+        # 3. admissions, in arrival order, while everything they need is there
+        while self.waiting and not blocked and budget > 0 and len(self.running) < self.max_num_seqs:
+            req = self.waiting[0]
+            count = min(req.num_tokens - req.num_computed, self.max_portion, budget)
+            if self.cache.slots.num_free == 0:
+                break
+            self.cache.add_request(req.req_id)
+            if not self.cache.can_grow(req.req_id, req.num_computed + count):
+                self.cache.free_request(req.req_id)
+                if not self.running:
+                    raise OutOfPages(f"request {req.req_id!r} alone does not fit the page pool "
+                                     f"({req.num_computed + count} tokens wanted)")
+                break
+            self.cache.grow(req.req_id, req.num_computed + count)
+            self.waiting.popleft()
+            self.running.append(req)
+            planned.append(ScheduledRun(req, req.num_computed, count))
+            budget -= count
+        # a request put back after it was planned is no longer in `running`
+        return [p for p in planned if p.request in self.running]
+
+    # ---------------------------------------------------------------- after the step
+
+    def update(self, runs: List[ScheduledRun], sampled: List[Optional[int]]) -> List[Request]:
+        """Record what the step computed and the tokens drawn for the runs that
+        sample (`sampled[i]` is None for the others). Returns the requests that ended."""
+        ended = []
+        for run, token in zip(runs, sampled):
+            req = run.request
+            req.num_computed = run.start + run.count
+            if not run.samples:
+                continue
+            if token is None:
+                raise ValueError(f"request {req.req_id!r} needs a token this step")
+            req.output.append(int(token))
+            p = req.params
+            if p.eos_token_id is not None and int(token) == p.eos_token_id and not p.ignore_eos:
+                req.finish_reason = "eos"
+            elif len(req.output) >= p.max_new_tokens:
+                req.finish_reason = "length"
+            elif req.num_tokens > self.max_model_len:
+                req.finish_reason = "model_length"
+            if req.finish_reason:
+                req.finished = True
+                self.running.remove(req)
+                self.cache.free_request(req.req_id)
+                self.finished.append(req)
+                ended.append(req)
+        return ended

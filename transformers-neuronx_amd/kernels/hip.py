@@ -40,6 +40,7 @@ _SIGNATURES = {
                               _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     },
     "sampling": {
+        "tnx_ban_tokens": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
         "tnx_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
         "tnx_sample": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                        _c_void_p],
@@ -243,6 +244,14 @@ class HipOps:
         return out
 
     # ---------------------------------------------------------------- output end
+
+    def ban_tokens(self, logits, tokens):
+        """In place: `logits[i, tokens[i]] = -inf` where `tokens[i] >= 0`."""
+        _want(logits, "logits", torch.float32)
+        _want(tokens, "tokens", torch.int32, (logits.shape[0],))
+        self._call("sampling", "tnx_ban_tokens", _ptr(logits), _ptr(tokens), logits.shape[0], logits.shape[1],
+                   _stream())
+        return logits
 
     def argmax(self, logits):
         _want(logits, "logits", torch.float32)

@@ -151,6 +151,11 @@ class ReferenceOps:
     def cast(self, x, dtype):
         return x.to(dtype)
 
+    def ban_tokens(self, logits, tokens):
+        rows = torch.nonzero(tokens >= 0).flatten()
+        logits[rows, tokens[rows].long()] = float("-inf")
+        return logits
+
     def argmax(self, logits):
         return logits.argmax(dim=-1).to(torch.int32)
 

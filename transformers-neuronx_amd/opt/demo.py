@@ -1,0 +1,132 @@
+"""Command line in the manner of the reference's `opt_demo` and `generation_demo`.
+
+    opt_demo [--amp f32|bf16] save DIR --random --config CONFIG.json [--seed N]
+    opt_demo [--amp f32|bf16] run DIR [--batch_size 4] [--n_positions 128] [--print_latency]
+             [--prompt_len N | --prompt_ids 5,6,7] [--top_k 50] [--top_p 1.0] [--temperature 1.0]
+             [--do_sample] [--max_new_tokens N] [--seed N] [--dump_logits DIR] [--benchmark]
+
+Option names and meanings are the reference's where it has them: gpt_demo.py:37-66
+(`--amp`, `save`, `--random`, `--config`, `run`, `--batch_size`, `--n_positions`,
+`--print_latency`) and generation_demo.py:201-280 (`--prompt_len`: random token ids of
+that length, :267, :492-494; `--top_k`, `--top_p`, `--temperature`, `--do_sample`,
+`--max_new_tokens`, `--dump_logits`, `--benchmark`). Without `--do_sample` `run` does what
+the reference's `run` does: `model.sample(input_ids, sequence_length=n_positions)` with
+top_k 50. There is no tokenizer here (no network to fetch one): prompts are token ids.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+
+def _parser():
+    parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    parser.add_argument("--amp", default="f32", choices=["f32", "f16", "bf16"])
+    sub = parser.add_subparsers(dest="which", required=True)
+    save = sub.add_parser("save")
+    save.add_argument("save", help="Directory to save the model")
+    save.add_argument("--random", action="store_true",
+                      help="Random weights flag. If true, config.json would be used to generate a model with "
+                           "random weight")
+    save.add_argument("--config", type=str, default="", help="Path to config.json file")
+    save.add_argument("--seed", type=int, default=0)
+    run = sub.add_parser("run")
+    run.add_argument("load")
+    run.add_argument("--batch_size", type=int, default=4, help="Input batch size")
+    run.add_argument("--n_positions", type=int, default=128, help="Input sequence length")
+    run.add_argument("--tp_degree", type=int, default=1, help="must be 1: one GPU")
+    run.add_argument("--print_latency", action="store_true", help="Print latency of each step")
+    run.add_argument("--prompt_len", type=int, default=None, help="random token ids of this length as the prompt")
+    run.add_argument("--prompt_ids", type=str, default=None, help="comma-separated token ids of the prompt")
+    run.add_argument("--do_sample", action="store_true")
+    run.add_argument("--top_k", type=int, default=50)
+    run.add_argument("--top_p", type=float, default=1.0)
+    run.add_argument("--temperature", type=float, default=1.0)
+    run.add_argument("--max_new_tokens", type=int, default=None)
+    run.add_argument("--max_length", type=int, default=None)
+    run.add_argument("--seed", type=int, default=15213)
+    run.add_argument("--dump_logits", type=str, default=None, help="folder for the logits of every step")
+    run.add_argument("--benchmark", action="store_true")
+    run.add_argument("--page_size", type=int, default=64)
+    return parser
+
+
+def save(args):
+    from .gen_random_pretrained import gen_random_pretrained
+    if not args.random:
+        raise SystemExit("save: only --random --config FILE is possible here (there is no network to fetch a model)")
+    if not args.config or not os.path.exists(args.config):
+        raise SystemExit("Please provide the config.json like: --config=./config.json")
+    dtype = {"f32": "float32", "f16": "float16", "bf16": "bfloat16"}[args.amp]
+    gen_random_pretrained(args.config, args.save, args.seed, dtype)
+    print(f"saved {args.save}")
+
+
+def run(args):
+    from ..config.engine_config import GenerationConfig
+    from .model import OPTForSampling
+    torch.manual_seed(args.seed)
+    print("running OPTForSampling.from_pretrained")
+    model = OPTForSampling.from_pretrained(args.load, batch_size=args.batch_size, amp=args.amp,
+                                           tp_degree=args.tp_degree, n_positions=args.n_positions,
+                                           page_size=args.page_size)
+    print("running model.load")
+    model.load()
+    vocab = model.config.vocab_size
+    if args.prompt_ids:
+        row = [int(t) for t in args.prompt_ids.split(",")]
+        input_ids = torch.tensor([row] * args.batch_size)
+    else:
+        n = args.prompt_len or 8
+        input_ids = torch.randint(3, vocab, (args.batch_size, n))
+    total = args.n_positions
+    if args.max_new_tokens is not None:
+        total = min(total, input_ids.shape[1] + args.max_new_tokens)
+    if args.max_length is not None:
+        total = min(total, args.max_length)
+    gen = None
+    if args.do_sample:
+        gen = GenerationConfig(do_sample=True, top_k=args.top_k, top_p=args.top_p, temperature=args.temperature)
+    if args.dump_logits:
+        os.makedirs(args.dump_logits, exist_ok=True)
+        logits = model(input_ids)
+        torch.save(logits.cpu(), os.path.join(args.dump_logits, "0.pt"))
+        model.reset()
+    if args.print_latency or args.benchmark:
+        model.engine.record_timings = True
+    print("running model.sample")
+    start = time.time()
+    out = model.sample(input_ids, sequence_length=total, top_k=args.top_k, temperature=args.temperature,
+                       top_p=args.top_p, seed=args.seed, generation_config=gen)
+    elapsed = time.time() - start
+    print("generated_sequence=", out)
+    if args.print_latency:
+        for rec in model.engine.timings:
+            print(f"Latency: {math.ceil(rec['seconds'] * 1000)} ms ({rec['tokens']} tokens)")
+    if args.benchmark:
+        t = model.engine.timings
+        prefill = [r for r in t if r["prefill_tokens"]]
+        decode = [r for r in t if not r["prefill_tokens"]]
+        new = (total - input_ids.shape[1]) * args.batch_size
+        report = {
+            "mean_context_encoding_latency_ms": 1000 * sum(r["seconds"] for r in prefill) / max(1, len(prefill)),
+            "mean_output_token_latency_ms": 1000 * sum(r["seconds"] for r in decode) / max(1, len(decode)),
+            "e2e_output_token_throughput": new / elapsed,
+        }
+        print(json.dumps(report))
+
+
+def main(argv=None):
+    args = _parser().parse_args(argv)
+    if args.which == "save":
+        save(args)
+    else:
+        run(args)
+
+
+if __name__ == "__main__":
+    main()

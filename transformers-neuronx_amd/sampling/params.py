@@ -1,0 +1,51 @@
+"""What a request asks of the sampler."""
+from dataclasses import dataclass
+from typing import Optional
+
+
+@dataclass
+class SamplingParams:
+    """Per-request sampling options.
+
+    The names and meanings follow the reference's host loops (sampling.py:131-180,
+    :311-378) and its `GenerationConfig` (config.py:106-139):
+    temperature  logits are divided by it before filtering (:337-338); 0 selects the
+                 argmax, as does do_sample=False
+    top_k        the k largest logits are kept (:151, :210-211); 0 keeps all
+    top_p        of those, the shortest prefix in descending order whose softmax mass
+                 reaches top_p (:213-249); 1.0 keeps all
+    seed         the request's own random stream: draw number n of the request uses the
+                 counter n, whatever else is in the batch
+    ban_eos      the end-of-sequence token is never chosen (`scores[:, eos] = -inf`,
+                 sampling.py:143-144, the OPT loop's behaviour)
+    ignore_eos   generation does not stop at the end-of-sequence token
+    max_new_tokens  the most tokens to generate
+    """
+    max_new_tokens: int = 16
+    do_sample: bool = True
+    temperature: float = 1.0
+    top_k: int = 0
+    top_p: float = 1.0
+    seed: int = 0
+    eos_token_id: Optional[int] = None
+    ban_eos: bool = False
+    ignore_eos: bool = False
+
+    def __post_init__(self):
+        if self.max_new_tokens < 0:
+            raise ValueError("max_new_tokens must not be negative")
+        if not isinstance(self.top_k, int) or self.top_k < 0:
+            raise ValueError("top_k has to be a non-negative int (0 keeps all tokens).")
+        if not 0.0 < float(self.top_p) <= 1.0:
+            raise ValueError("top_p has to be a strictly positive float that less than or equal to 1.0.")
+        if float(self.temperature) < 0:
+            raise ValueError("temperature has to be a non-negative float (0 is greedy).")
+
+    @property
+    def greedy(self) -> bool:
+        return (not self.do_sample) or self.temperature == 0.0 or self.top_k == 1
+
+    @staticmethod
+    def greedy_params(max_new_tokens: int, eos_token_id=None, ignore_eos=True) -> "SamplingParams":
+        return SamplingParams(max_new_tokens=max_new_tokens, do_sample=False, eos_token_id=eos_token_id,
+                              ignore_eos=ignore_eos)
