@@ -1,0 +1,91 @@
+"""Configuration and registry."""
+import json
+
+import pytest
+
+from conftest import TINY_A, TINY_B
+from transformers_neuronx_amd.config import (ConfigError, EngineConfig, NeuronConfig, ContinuousBatchingConfig,
+                                             OPTConfig, known_architectures, parse_dtype, read_config, resolve)
+
+
+def test_reads_every_key():
+    a = OPTConfig.from_dict(TINY_A)
+    assert (a.vocab_size, a.hidden_size, a.num_hidden_layers, a.num_attention_heads) == (512, 64, 2, 4)
+    assert (a.ffn_dim, a.max_position_embeddings, a.word_embed_proj_dim, a.head_size) == (256, 128, 64, 16)
+    assert a.do_layer_norm_before and a.enable_bias and a.layer_norm_elementwise_affine
+    b = OPTConfig.from_dict(TINY_B)
+    assert (b.word_embed_proj_dim, b.head_size, b.activation_function) == (48, 32, "gelu")
+    assert not b.do_layer_norm_before and not b.enable_bias and not b.layer_norm_elementwise_affine
+    assert b.layer_norm_eps == 3e-4 and b.init_std == 0.05
+
+
+def test_defaults_follow_the_family():
+    raw = {k: TINY_A[k] for k in ("vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads",
+                                  "ffn_dim", "max_position_embeddings")}
+    c = OPTConfig.from_dict(raw)
+    assert c.word_embed_proj_dim == c.hidden_size
+    assert c.do_layer_norm_before and c.enable_bias and c.activation_function == "relu"
+    assert c.layer_norm_eps == 1e-5 and c.eos_token_id == 2 and c.pad_token_id == 1
+
+
+@pytest.mark.parametrize("key", ["vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads",
+                                 "ffn_dim", "max_position_embeddings"])
+def test_missing_key_is_named(key):
+    raw = dict(TINY_A)
+    del raw[key]
+    with pytest.raises(ConfigError, match=key):
+        OPTConfig.from_dict(raw)
+
+
+@pytest.mark.parametrize("key,value,word", [
+    ("hidden_size", 66, "multiple"), ("activation_function", "swish", "activation_function"),
+    ("vocab_size", 0, "positive"), ("num_hidden_layers", "2", "integer"), ("enable_bias", 1, "true or false"),
+    ("layer_norm_eps", 0.0, "positive"), ("ffn_dim", 2.5, "integer")])
+def test_bad_values_are_refused(key, value, word):
+    raw = dict(TINY_A)
+    raw[key] = value
+    with pytest.raises(ConfigError, match=word):
+        OPTConfig.from_dict(raw)
+
+
+def test_unknown_keys_are_ignored_and_round_trip(tmp_path):
+    raw = dict(TINY_B, dropout=0.1, layerdrop=0.0, _name_or_path="x")
+    c = OPTConfig.from_dict(raw)
+    c.save(str(tmp_path))
+    arch, again = read_config(str(tmp_path))
+    assert again == c and arch.name == "OPTForCausalLM"
+    assert json.load(open(tmp_path / "config.json"))["architectures"] == ["OPTForCausalLM"]
+
+
+def test_registry():
+    assert "OPTForCausalLM" in known_architectures()
+    assert resolve({"architectures": ["OPTForCausalLM"]}).config_class is OPTConfig
+    assert resolve({"model_type": "opt"}).name == "OPTForCausalLM"
+    with pytest.raises(ConfigError, match="known architectures"):
+        resolve({"architectures": ["LlamaForCausalLM"], "model_type": "llama"})
+    from transformers_neuronx_amd.opt.model import OPTForSampling
+    assert resolve({"model_type": "opt"}).model_class is OPTForSampling
+
+
+def test_engine_config():
+    assert parse_dtype("bf16") == parse_dtype("bfloat16") and parse_dtype("f32") == parse_dtype("float32")
+    with pytest.raises(ValueError):
+        parse_dtype("int8")
+    with pytest.raises(ValueError, match="page_size"):
+        EngineConfig(page_size=24)
+    with pytest.raises(ValueError, match="kernels"):
+        EngineConfig(kernels="cpu")
+    cb = ContinuousBatchingConfig(batch_size_for_shared_caches=4, max_model_len=128)
+    assert cb.max_num_seqs == 4
+    cb.init_cache_engine(block_size=32, num_blocks=10)
+    assert NeuronConfig(continuous_batching=cb).continuous_batching.num_blocks == 10
+    with pytest.raises(ValueError, match="float32"):
+        NeuronConfig(cast_logits_dtype="bfloat16")
+
+
+def test_sequence_length_guard():
+    from transformers_neuronx_amd.opt.model import OPTForSampling
+    with pytest.raises(ValueError, match="position embedding"):
+        OPTForSampling(OPTConfig.from_dict(TINY_A), n_positions=129, amp="f32")
+    with pytest.raises(ValueError, match="one GPU"):
+        OPTForSampling(OPTConfig.from_dict(TINY_A), n_positions=64, amp="f32", tp_degree=2)

@@ -1,0 +1,189 @@
+"""The engine's host logic (cache, batching, scheduler, sampler) with the plain torch rendition of the
+kernels, on the CPU: the same comparisons the GPU tests make with the HIP kernels."""
+import io
+import json
+
+import numpy as np
+import pytest
+import torch
+
+import plain_opt
+import schedules
+from conftest import TINY
+from transformers_neuronx_amd.config import EngineConfig, OPTConfig
+from transformers_neuronx_amd.engine import StepEntry
+from transformers_neuronx_amd.engine.engine import LLMEngine
+from transformers_neuronx_amd.engine.factory import runner_from_folder
+from transformers_neuronx_amd.sampling import SamplingParams
+
+
+def _runner(folder, max_tokens, page_size=16, **kw):
+    cfg = EngineConfig(dtype="float32", kernels="reference", device="cpu", page_size=page_size,
+                       max_tokens=max_tokens, max_num_seqs=8, **kw)
+    return runner_from_folder(folder, cfg), cfg
+
+
+def _requests(vocab, lengths, seed):
+    g = torch.Generator().manual_seed(seed)
+    return {f"r{i}": torch.randint(3, vocab, (n,), generator=g).tolist() for i, n in enumerate(lengths)}
+
+
+@pytest.mark.parametrize("name,lengths", [("A", [5, 17, 31, 100]), ("B", [1, 9, 40, 77, 120])])
+def test_schedules_on_the_host(tiny_folders, tmp_path, name, lengths):
+    from transformers_neuronx_amd.engine.replay import replay
+    folder, cfg, weights = tiny_folders[name]
+    requests = _requests(cfg["vocab_size"], lengths, 2)
+    expected = {rid: plain_opt.forward_logits(weights, cfg, toks) for rid, toks in requests.items()}
+    for kind, (steps, place), max_tokens in [
+        ("whole", schedules.whole(requests), 128),
+        ("singles", schedules.head_then_singles(requests), 128),
+        ("portions", schedules.portions(requests), 128),
+        ("mixed", schedules.mixed(requests, max_tokens=256, seed=1), 256),
+    ]:
+        runner, _ = _runner(folder, max_tokens)
+        out = tmp_path / f"{name}_{kind}"
+        replay((json.dumps(s) for s in steps), runner, str(out), io.StringIO())
+        runner.cache.check()
+        for (step, row), (rid, pos) in place.items():
+            got = np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(-1, cfg["vocab_size"])[row]
+            assert np.abs(got - expected[rid][pos].numpy()).max() < 1e-5, (kind, step, rid, pos)
+
+
+def test_step_refuses_what_it_cannot_run(tiny_folders):
+    folder, cfg, _ = tiny_folders["A"]
+    runner, _ = _runner(folder, 64)
+    with pytest.raises(ValueError, match="vocabulary"):
+        runner.step([StepEntry("a", [5, 512], [0])])
+    with pytest.raises(ValueError, match="twice"):
+        runner.step([StepEntry("a", [5], [0]), StepEntry("a", [6], [0])])
+    with pytest.raises(ValueError, match="outside"):
+        runner.step([StepEntry("a", [5, 6], [2])])
+    with pytest.raises(ValueError, match="positions"):
+        runner.step([StepEntry("b", [5] * 129, [])])
+    assert runner.step([StepEntry("c", [5, 6, 7], [])]) is None          # nothing wanted: it still runs
+    assert runner.cache.num_tokens("c") == 3
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_generation_does_not_depend_on_the_schedule(tiny_folders, name):
+    """Greedy and sampled tokens are the same whether requests run alone, together, in small portions, or
+    with so few pages that some are put back and computed again."""
+    folder, cfg, weights = tiny_folders[name]
+    prompts = list(_requests(cfg["vocab_size"], [1, 9, 40, 77], 3).values())
+    params = [SamplingParams(max_new_tokens=12, do_sample=False, ignore_eos=True),
+              SamplingParams(max_new_tokens=12, temperature=0.8, seed=11, ignore_eos=True),
+              SamplingParams(max_new_tokens=12, temperature=1.2, top_k=20, top_p=0.9, seed=5, ignore_eos=True),
+              SamplingParams(max_new_tokens=12, do_sample=False, ignore_eos=True)]
+
+    def generate(max_tokens, budget, together):
+        runner, ecfg = _runner(folder, max_tokens, max_num_batched_tokens=budget)
+        engine = LLMEngine(runner, ecfg)
+        if together:
+            outs = engine.generate(prompts, params)
+        else:
+            outs = [engine.generate([p], [sp])[0] for p, sp in zip(prompts, params)]
+        runner.cache.check()
+        assert not runner.cache.requests
+        return outs, engine.scheduler.num_preemptions
+
+    alone, _ = generate(512, 512, together=False)
+    assert alone[0] == plain_opt.greedy(weights, cfg, prompts[0], 12)[len(prompts[0]):]
+    assert alone[3] == plain_opt.greedy(weights, cfg, prompts[3], 12)[len(prompts[3]):]
+    together, n0 = generate(512, 512, together=True)
+    portions, _ = generate(512, 24, together=True)
+    tight, n = generate(160, 32, together=True)            # 10 pages of 16 for 175 tokens: some go back
+    assert n0 == 0 and n > 0
+    assert alone == together == portions == tight
+
+
+def test_sampled_tokens_follow_the_plain_sampler(tiny_folders):
+    folder, cfg, weights = tiny_folders["A"]
+    prompt = _requests(cfg["vocab_size"], [13], 4)["r0"]
+    sp = SamplingParams(max_new_tokens=6, temperature=0.7, top_k=8, top_p=0.95, seed=99, ignore_eos=True)
+    runner, ecfg = _runner(folder, 128)
+    out = LLMEngine(runner, ecfg).generate([prompt], sp)[0]
+    toks = list(prompt)
+    for n in range(6):
+        logits = plain_opt.forward_logits(weights, cfg, toks)[-1]
+        tok = plain_opt.sample_row(logits, plain_opt.philox_uniform(99, n), top_k=8, top_p=0.95, temperature=0.7)
+        assert out[n] == tok
+        toks.append(tok)
+
+
+def test_entry_point_in_the_reference_manner(tiny_folders):
+    from transformers_neuronx_amd import OPTForSampling
+    folder, cfg, weights = tiny_folders["A"]
+    model = OPTForSampling.from_pretrained(folder, batch_size=2, amp="f32", n_positions=48, kernels="reference",
+                                           device="cpu", page_size=16)
+    with pytest.raises(RuntimeError, match="load"):
+        model.sample(torch.tensor([[5, 6]]), 8)
+    model.to_neuron()
+    ids = torch.tensor([[5, 9, 200, 31], [7, 7, 100, 3]])
+    out = model.sample(ids, sequence_length=12, top_k=1)
+    assert out.shape == (2, 12) and torch.equal(out[:, :4], ids)
+    for b in range(2):
+        assert out[b].tolist() == plain_opt.greedy(weights, cfg, ids[b].tolist(), 8)
+    sampled = model.sample(ids, sequence_length=12, top_k=50)
+    assert sampled.shape == (2, 12) and not (sampled == cfg.get("eos_token_id", 2))[:, 4:].any()
+    # forward in the reference's form: prompt pass, then one token at the next cache id
+    logits = model(ids)
+    want = torch.stack([plain_opt.forward_logits(weights, cfg, ids[b].tolist())[-1] for b in range(2)])
+    torch.testing.assert_close(logits, want, atol=1e-5, rtol=1e-5)
+    nxt = torch.tensor([[11], [12]])
+    logits = model(nxt, torch.tensor([4]))
+    want = torch.stack([plain_opt.forward_logits(weights, cfg, ids[b].tolist() + nxt[b].tolist())[-1]
+                        for b in range(2)])
+    torch.testing.assert_close(logits, want, atol=1e-5, rtol=1e-5)
+    with pytest.raises(ValueError, match="cache_ids"):
+        model(nxt, torch.tensor([9]))
+    # rows padded on the left up to start_ids: the padding is dropped
+    padded = torch.tensor([[1, 1, 5, 9], [7, 7, 100, 3]])
+    logits = model(padded, None, torch.tensor([2, 0]))
+    torch.testing.assert_close(logits[0], plain_opt.forward_logits(weights, cfg, [5, 9])[-1], atol=1e-5, rtol=1e-5)
+    model.reset()
+    assert not model.engine.runner.cache.requests
+
+
+def _toy_model(ops_kind, dtype, device):
+    import toy_parts
+    from transformers_neuronx_amd.cache import CacheManager
+    from transformers_neuronx_amd.engine import DecoderModel, ModelRunner
+    from transformers_neuronx_amd.kernels import make_ops
+    from transformers_neuronx_amd.weights import TensorDict, random_tensors
+    spec = toy_parts.toy_spec()
+    model = DecoderModel(spec)
+    tensors = random_tensors(model.param_decls(), spec.init_std, 3, torch.float32)
+    ops = make_ops(ops_kind, dtype, device)
+    model.load(TensorDict(tensors), ops, dtype, device)
+    needs = model.cache_needs()
+    cache = CacheManager(needs, 16, 12, 4, dtype, device)
+    return ModelRunner(model, cache, ops), tensors
+
+
+def run_toy_model(ops_kind, dtype, device, tol):
+    import toy_parts
+    runner, tensors = _toy_model(ops_kind, dtype, device)
+    cache = runner.cache
+    assert set(cache.groups) == {"full", "window24"}
+    assert len(cache.groups["full"].cache_ids) == 2 and len(cache.groups["window24"].cache_ids) == 1
+    states = [c for c in cache.caches.values() if c.state]
+    assert len(states) == 2                                    # the layer named twice has a state per call
+    requests = _requests(300, [70, 33, 100], 8)
+    expected = {rid: toy_parts.toy_plain_logits(tensors, toks) for rid, toks in requests.items()}
+    for steps, place in (schedules.whole(requests), schedules.portions(requests),
+                         schedules.mixed(requests, max_tokens=192, page=16, seed=2, tail=8, max_live=3)):
+        for rec in steps:
+            logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in rec["entries"]])
+            for row in range(logits.shape[0]):
+                rid, pos = place[(rec["step"], row)]
+                want = expected[rid][pos]
+                err = float((logits[row].cpu() - want).abs().max() / want.abs().max())
+                assert err < tol, (rec["step"], rid, pos, err)
+            for rid in rec["end"]:
+                runner.finish(rid)
+            cache.check()
+        assert not cache.requests
+
+
+def test_toy_parts_on_the_host():
+    run_toy_model("reference", torch.float32, "cpu", 2e-5)

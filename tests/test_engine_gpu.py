@@ -77,3 +77,99 @@ def test_schedules_agree_with_plain(tiny_folders, tiny_folders_bf16, tmp_path, d
     ]:
         out, _ = _run(folder, dtype, steps, max_tokens, page_size, tmp_path, f"{kind}")
         _compare(out, place, expected, cfg["vocab_size"], dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(tiny_folders, tiny_folders_bf16, tmp_path, dtype):
+    """A short prompt, then 240 tokens one by one, across many pages."""
+    folder, cfg, weights = (tiny_folders if dtype == "float32" else tiny_folders_bf16)["B"]
+    requests = _requests(cfg, [250], seed=9)
+    expected = _expected(weights, cfg, requests)
+    steps, place = schedules.head_then_singles(requests, tail=240)
+    out, _ = _run(folder, dtype, steps, 256, 16, tmp_path, "long")
+    _compare(out, place, expected, cfg["vocab_size"], dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens(tiny_folders, tiny_folders_bf16, tmp_path, dtype, name):
+    """Prompts of one and two tokens, then single tokens: the first positions of a sequence."""
+    folder, cfg, weights = (tiny_folders if dtype == "float32" else tiny_folders_bf16)[name]
+    requests = _requests(cfg, [6, 7], seed=1)
+    expected = _expected(weights, cfg, requests)
+    steps = []
+    for rid, first in (("r0", 1), ("r1", 2)):
+        toks = requests[rid]
+        steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": toks[:first],
+                                                       "want": list(range(first))}], "end": []})
+        for t in toks[first:]:
+            steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": [t], "want": [0]}], "end": []})
+        steps[-1]["end"] = [rid]
+    steps, place = schedules._finish(steps)
+    out, _ = _run(folder, dtype, steps, 64, 16, tmp_path, "first")
+    _compare(out, place, expected, cfg["vocab_size"], dtype)
+
+
+def test_pages_are_used_again_without_leaking(tiny_folders, tmp_path):
+    """One page pool of the smallest size, request after request: every request sees pages its
+    predecessor wrote, and its logits do not change."""
+    folder, cfg, weights = tiny_folders["A"]
+    requests = _requests(cfg, [60, 64, 33, 64, 17], seed=21)
+    expected = _expected(weights, cfg, requests)
+    steps, place = schedules.portions(requests, sizes=(19, 2, 30, 64))
+    out, runner = _run(folder, "float32", steps, 64, 16, tmp_path, "reuse")
+    assert runner.cache.groups["full"].pool.num_pages == 4
+    _compare(out, place, expected, cfg["vocab_size"], "float32")
+
+
+@pytest.mark.parametrize("amp", ["f32", "bf16"])
+def test_greedy_generation_through_the_entry_point(tiny_folders, amp):
+    from transformers_neuronx_amd import OPTForSampling
+    from transformers_neuronx_amd.kernels import hip
+    for name in ("A", "B"):
+        folder, cfg, weights = tiny_folders[name]
+        model = OPTForSampling.from_pretrained(folder, batch_size=3, amp=amp, n_positions=64, page_size=16,
+                                               num_pages=9, max_num_batched_tokens=24).load()
+        ids = torch.randint(3, cfg["vocab_size"], (3, 11), generator=torch.Generator().manual_seed(2))
+        out = model.sample(ids, sequence_length=40, top_k=1)
+        assert out.shape == (3, 40)
+        if amp == "f32":
+            for b in range(3):
+                assert out[b].tolist() == plain_opt.greedy(weights, cfg, ids[b].tolist(), 29)
+        else:
+            # bfloat16 may part from the float32 choice where two logits are close: every chosen token
+            # must be within the rounding of the best one under the plain implementation
+            for b in range(3):
+                toks = out[b].tolist()
+                logits = plain_opt.forward_logits(weights, cfg, toks[:-1])
+                for pos in range(10, 39):
+                    row = logits[pos]
+                    assert float(row.max() - row[toks[pos + 1]]) <= 3e-2 * float(row.abs().max())
+    assert set(hip.loaded_libraries()) >= {"elementwise", "gemm", "attention", "sampling"}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_toy_parts_on_the_gpu(dtype):
+    """A mixer with state of its own, registered by the test, beside full, windowed and cache-sharing
+    attention, in a run order that names layers twice."""
+    from test_engine_cpu import run_toy_model
+    run_toy_model("hip", dtype, DEV, 2e-5 if dtype == torch.float32 else 3e-2)
+
+
+def test_trace_run_as_a_program(tiny_folders, tmp_path):
+    import subprocess
+    import sys
+    folder, cfg, weights = tiny_folders["A"]
+    requests = _requests(cfg, [40, 70], seed=13)
+    expected = _expected(weights, cfg, requests)
+    steps, place = schedules.mixed(requests, max_tokens=192, seed=1)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for dtype in ("float32", "bfloat16"):
+        out = tmp_path / f"cli_{dtype}"
+        proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder,
+                               "--dtype", dtype, "--out", str(out), "--max-tokens", "192"],
+                              input="\n".join(json.dumps(s) for s in steps) + "\n", text=True,
+                              capture_output=True, timeout=110)
+        assert proc.returncode == 0, proc.stderr
+        assert proc.stdout.split() == [w for s in steps for w in ("done", str(s["step"]))]
+        _compare(str(out), place, expected, cfg["vocab_size"], dtype)

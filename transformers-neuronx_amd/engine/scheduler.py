@@ -58,11 +58,11 @@ class ScheduledRun:
     request: Request
     start: int                      # first position of the portion
     count: int                      # tokens in the portion
+    samples: bool = False           # the portion ends at the request's newest token: its last logits
+                                    # pick the next one
 
-    @property
-    def samples(self) -> bool:
-        """The portion ends at the request's newest token: its last logits pick the next one."""
-        return self.start + self.count == self.request.num_tokens
+    def __post_init__(self):
+        self.samples = self.start + self.count == self.request.num_tokens
 
 
 class Scheduler:
