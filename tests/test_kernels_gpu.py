@@ -277,3 +277,37 @@ def test_sampling_distribution():
     assert counts.sum() == counts[idx].sum()           # nothing outside the top k
     chi2 = (((counts[idx] - probs * n) ** 2) / (probs * n)).sum().item()
     assert chi2 < 40, chi2                              # 9 degrees of freedom; 40 is far in the tail
+
+
+FAST_CASES = [
+    # heads, kv heads, head size, page size, runs, cached
+    (4, 4, 64, 64, [300, 1, 1], [0, 1000, 255]),
+    (8, 2, 128, 64, [1, 1, 1, 1], [2047, 100, 0, 640]),
+    (4, 4, 128, 16, [129, 40, 1], [77, 0, 300]),
+    (2, 1, 256, 32, [1, 200], [500, 31]),
+    (3, 3, 32, 16, [1, 1, 2], [0, 1, 0]),
+    (2, 2, 16, 64, [1, 260], [900, 3]),
+    (2, 2, 96, 16, [150, 33], [10, 0]),
+]
+
+
+@pytest.mark.parametrize("case", FAST_CASES)
+@pytest.mark.parametrize("window", [None, 100])
+def test_bfloat16_attention_kernels_agree(case, window):
+    """The MFMA kernel for prompts and the split kernel for decoding against the torch rendition and
+    against the one-wave-per-query kernel, with contexts long enough to split."""
+    from transformers_neuronx_amd.kernels.hip import HipOps
+    ctx, q, kp, vp, o_fast = _fill_cache_and_compare(torch.bfloat16, *case, window)
+    heads, kv, hs = case[:3]
+    plain = HipOps(torch.bfloat16, DEV)
+    plain.force_plain_attention = True
+    o_plain = plain.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)
+    torch.testing.assert_close(o_fast.float(), o_plain.float(), rtol=2e-2, atol=2e-2)
+    many = HipOps(torch.bfloat16, DEV)
+    many.decode_blocks_wanted = 1 << 20           # as many splits as the contexts allow
+    o_many = many.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)
+    torch.testing.assert_close(o_many.float(), o_plain.float(), rtol=2e-2, atol=2e-2)
+    one = HipOps(torch.bfloat16, DEV)
+    one.decode_blocks_wanted = 1                  # no split at all
+    o_one = one.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)
+    torch.testing.assert_close(o_one.float(), o_plain.float(), rtol=2e-2, atol=2e-2)

@@ -174,3 +174,426 @@ extern "C" int tnx_attention_any(const void* q, int dtype, const void* k_pages, 
   TNX_CHECK_LAUNCH("attention_any");
   return 0;
 }
+
+// ------------------------------------------------------------------------------------------ bfloat16, prompts
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+#define PREFILL_Q_TILE 128  // queries per block: four waves of 32
+
+// Flash-style attention of a run of queries over its request's pages, on MFMA 16x16x32.
+// A wave owns 32 queries (two column blocks of 16) and walks the keys 64 at a time. It computes the
+// transposed scores S^T = K Q^T, so that the accumulator layout (lane = query, four consecutive keys per
+// register group) is at once the layout of the B operand of O^T += V^T P^T: the probabilities never leave
+// their registers. The keys of a 32-key MFMA step are taken in the order (16b + 4g + i), b the half, g the
+// lane group, which is the order the accumulators hold them in; the values are read in the same order.
+// NDB bounds the head size (16 * NDB); smaller head sizes run with the blocks beyond them switched off.
+template <int NDB>
+__global__ void __launch_bounds__(256)
+attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
+                         const bf16_t* __restrict__ v_pages, const int* __restrict__ run_start,
+                         const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
+                         int page_size, int num_pages, const int* __restrict__ tile_run,
+                         const int* __restrict__ tile_q0, bf16_t* __restrict__ out, int num_heads, int num_kv,
+                         int head_size, int window) {
+  constexpr int NKS = (NDB + 1) / 2;  // MFMA steps of 32 over the head size
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int run = tile_run[blockIdx.x], h = blockIdx.y;
+  const int kvh = h / (num_heads / num_kv);
+  const int t0 = run_start[run], qlen = run_start[run + 1] - t0, cached = cached_lens[run];
+  const int qw0 = tile_q0[blockIdx.x] + 32 * wave;
+  if (qw0 >= qlen) return;
+  const int nq = num_heads * head_size;
+  const int* tab = table + (size_t)run * table_width;
+  const int total = cached + qlen;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int ndb = head_size / 16;
+
+  bf16x8 qf[2][NKS];
+  int qpos[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int qi = qw0 + 16 * qb + r;
+    qpos[qb] = cached + qi;
+#pragma unroll
+    for (int s = 0; s < NKS; ++s) {
+      const int d0 = 32 * s + 8 * g;
+      qf[qb][s] = (qi < qlen && d0 < head_size) ? *(const bf16x8*)(q + (size_t)(t0 + qi) * nq + h * head_size + d0)
+                                                : zero8;
+    }
+  }
+  const int last_q = cached + min(qw0 + 31, qlen - 1);          // the wave's last query position
+  const int first_q = cached + qw0;
+  const int lo = window > 0 ? max(0, first_q - window + 1) : 0;  // no query of the wave reads before this
+
+  float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
+  f32x4 o[NDB][2];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) o[db][qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  for (int tile0 = (lo / 64) * 64; tile0 <= last_q; tile0 += 64) {
+    f32x4 s[4][2];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      const int key0 = tile0 + 16 * kb;
+      f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+      int page = -1;
+      if (key0 <= last_q) page = tab[key0 / page_size];
+      if (page >= 0 && page < num_pages) {
+        const bf16_t* kbase =
+            k_pages + (((size_t)page * num_kv + kvh) * page_size + key0 % page_size + r) * head_size;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+          const int d0 = 32 * ks + 8 * g;
+          const bf16x8 kf = d0 < head_size ? *(const bf16x8*)(kbase + d0) : zero8;
+          a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[0][ks], a0, 0, 0, 0);
+          a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[1][ks], a1, 0, 0, 0);
+        }
+      }
+      s[kb][0] = a0;
+      s[kb][1] = a1;
+    }
+    // what a query may not see becomes -inf: later keys, keys before its window, keys without a page
+    const bool full_tile = tile0 + 63 <= first_q && (window <= 0 || tile0 > last_q - window);
+    if (!full_tile) {
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = tile0 + 16 * kb + 4 * g + i;
+            const bool ok = key <= qpos[qb] && (window <= 0 || key > qpos[qb] - window);
+            if (!ok) s[kb][qb][i] = -INFINITY;
+          }
+    }
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s[kb][qb][i]);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m[qb], mx);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = __expf(m[qb] - m_safe);
+      float sum = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float p = __expf(s[kb][qb][i] - m_safe);
+          s[kb][qb][i] = p;
+          sum += p;
+        }
+      sum += __shfl_xor(sum, 16, 64);
+      sum += __shfl_xor(sum, 32, 64);
+      l[qb] = l[qb] * alpha + sum;
+      m[qb] = m_new;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[db][qb][i] *= alpha;
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      if (tile0 + 32 * t > last_q) continue;
+      bf16x8 pb[2];
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pb[qb][j] = (bf16_t)s[2 * t + (j >> 2)][qb][j & 3];
+      const bf16_t* vbase[2];
+      bool vok[2];
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const int key0 = tile0 + 32 * t + 16 * b;
+        int page = -1;
+        if (key0 <= last_q) page = tab[key0 / page_size];
+        vok[b] = page >= 0 && page < num_pages;
+        vbase[b] = v_pages + ((size_t)(vok[b] ? page : 0) * num_kv + kvh) * head_size * page_size +
+                   key0 % page_size + 4 * g;
+      }
+      const bool tail = tile0 + 32 * t + 32 > total;   // some keys of this step lie beyond the request
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) {
+        if (db >= ndb) continue;
+        const int d = 16 * db + r;
+        bf16x8 vf;
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          bf16x4 v4 = {0, 0, 0, 0};
+          if (vok[b]) v4 = *(const bf16x4*)(vbase[b] + (size_t)d * page_size);
+          if (tail) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (tile0 + 32 * t + 16 * b + 4 * g + i >= total) v4[i] = 0;
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) vf[4 * b + i] = v4[i];
+        }
+        o[db][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[0], o[db][0], 0, 0, 0);
+        o[db][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[1], o[db][1], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int qi = qw0 + 16 * qb + r;
+    if (qi >= qlen) continue;
+    const float inv = 1.f / l[qb];
+    bf16_t* orow = out + (size_t)(t0 + qi) * nq + h * head_size;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+      if (db >= ndb) continue;
+      bf16x4 v4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v4[i] = (bf16_t)(o[db][qb][i] * inv);
+      *(bf16x4*)(orow + 16 * db + 4 * g) = v4;
+    }
+  }
+}
+
+extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const void* v_pages, const int* run_start,
+                                     const int* cached_lens, const int* table, int table_width, int page_size,
+                                     int num_pages, const int* tile_run, const int* tile_q0, int num_tiles, void* out,
+                                     int num_heads, int num_kv, int head_size, int window, hipStream_t stream) {
+  TNX_REQUIRE(num_heads > 0 && num_kv > 0 && num_heads % num_kv == 0, "attention_prefill: bad head counts");
+  TNX_REQUIRE(head_size % 16 == 0 && head_size >= 16 && head_size <= 256,
+              "attention_prefill: head size %d is not a multiple of 16 in [16, 256]", head_size);
+  TNX_REQUIRE(page_size % 16 == 0 && page_size > 0, "attention_prefill: page size %d is not a multiple of 16",
+              page_size);
+  TNX_REQUIRE(num_heads <= 65535, "attention_prefill: too many heads");
+  if (num_tiles <= 0) return 0;
+  dim3 grid(num_tiles, num_heads);
+#define LAUNCH_PREFILL(NDB)                                                                                        \
+  attention_prefill_kernel<NDB><<<grid, 256, 0, stream>>>(                                                         \
+      (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, table_width, \
+      page_size, num_pages, tile_run, tile_q0, (bf16_t*)out, num_heads, num_kv, head_size, window)
+  if (head_size <= 64)
+    LAUNCH_PREFILL(4);
+  else if (head_size <= 128)
+    LAUNCH_PREFILL(8);
+  else
+    LAUNCH_PREFILL(16);
+#undef LAUNCH_PREFILL
+  TNX_CHECK_LAUNCH("attention_prefill");
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------ bfloat16, decoding
+
+// One query per request over its pages. The keys of a request are split over `num_splits` blocks; a block's
+// four waves take 64-key tiles in turn. A tile of keys of one head is read as it lies in memory, 16 bytes
+// a lane: lane l holds chunk l % CPR (8 head-size elements) of key l / CPR of each group of 64 / CPR keys,
+// so a score is a sum over CPR neighbouring lanes. Values lie transposed ([head_size][page_size]), so
+// lane l holds 8 keys (l % 8) of head-size element l / 8 of each group of 8 elements, and the output is a
+// sum over 8 neighbouring lanes, taken once at the end. Partial results (maximum, sum, weighted values,
+// all float32) of waves meet in LDS and those of splits in a workspace that a second kernel merges.
+template <int CPR>
+__global__ void __launch_bounds__(256)
+attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
+                        const bf16_t* __restrict__ v_pages, const int* __restrict__ run_start,
+                        const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
+                        int page_size, int num_pages, const int* __restrict__ decode_runs, bf16_t* __restrict__ out,
+                        float* __restrict__ part_o, float* __restrict__ part_ml, int num_heads, int num_kv,
+                        int window, int num_splits, int keys_per_split) {
+  constexpr int KPI = 64 / CPR;       // keys per load instruction of a wave
+  constexpr int DH = CPR * 8;
+  __shared__ float sm_p[4][64];
+  __shared__ float sm_o[4][DH];
+  __shared__ float sm_m[4], sm_l[4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int split = blockIdx.x, h = blockIdx.y, dz = blockIdx.z;
+  const int kvh = h / (num_heads / num_kv);
+  const int run = decode_runs[dz];
+  const int t = run_start[run];
+  const int pos = cached_lens[run];   // the query's own position; its key is stored already
+  const int* tab = table + (size_t)run * table_width;
+  const int nq = num_heads * DH;
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int k_begin = (lo / 64) * 64 + split * keys_per_split;
+  const int k_end = min(pos + 1, k_begin + keys_per_split);
+  const int dchunk = lane % CPR, kgrp = lane / CPR;
+
+  float qf[8];
+  {
+    const bf16x8 qv = *(const bf16x8*)(q + (size_t)t * nq + h * DH + dchunk * 8);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) qf[j] = (float)qv[j];
+  }
+  float m = -INFINITY, l = 0.f;
+  float acc[CPR];
+#pragma unroll
+  for (int i = 0; i < CPR; ++i) acc[i] = 0.f;
+
+  for (int tile0 = k_begin + 64 * wave; tile0 < k_end; tile0 += 256) {
+    float s[CPR];
+#pragma unroll
+    for (int i = 0; i < CPR; ++i) {
+      const int key = tile0 + i * KPI + kgrp;
+      bool valid = key >= lo && key < k_end;
+      float sum = 0.f;
+      if (valid) {
+        const int page = tab[key / page_size];
+        if (page >= 0 && page < num_pages) {
+          const bf16x8 kv = *(const bf16x8*)(k_pages + (((size_t)page * num_kv + kvh) * page_size +
+                                                        key % page_size) * DH + dchunk * 8);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) sum = fmaf(qf[j], (float)kv[j], sum);
+        } else {
+          valid = false;
+        }
+      }
+#pragma unroll
+      for (int o = 1; o < CPR; o <<= 1) sum += __shfl_xor(sum, o, 64);
+      s[i] = valid ? sum : -INFINITY;
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < CPR; ++i) mx = fmaxf(mx, s[i]);
+#pragma unroll
+    for (int o = CPR; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    const float m_new = fmaxf(m, mx);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = __expf(m - m_safe);
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < CPR; ++i) {
+      s[i] = __expf(s[i] - m_safe);
+      psum += s[i];
+    }
+#pragma unroll
+    for (int o = CPR; o < 64; o <<= 1) psum += __shfl_xor(psum, o, 64);
+    l = l * alpha + psum;
+    m = m_new;
+    if (dchunk == 0) {
+#pragma unroll
+      for (int i = 0; i < CPR; ++i) sm_p[wave][i * KPI + kgrp] = s[i];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int kc = lane & 7;
+    float pv[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) pv[j] = sm_p[wave][kc * 8 + j];
+    const int key0 = tile0 + kc * 8;
+    int page = -1;
+    if (key0 < k_end) page = tab[key0 / page_size];
+    const bool vok = page >= 0 && page < num_pages;
+    const bf16_t* vbase = v_pages + ((size_t)(vok ? page : 0) * num_kv + kvh) * DH * page_size + key0 % page_size;
+#pragma unroll
+    for (int i = 0; i < CPR; ++i) {
+      const int d = i * 8 + (lane >> 3);
+      float a = acc[i] * alpha;
+      if (vok) {
+        const bf16x8 vv = *(const bf16x8*)(vbase + (size_t)d * page_size);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) a += pv[j] != 0.f ? pv[j] * (float)vv[j] : 0.f;
+      }
+      acc[i] = a;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+#pragma unroll
+  for (int i = 0; i < CPR; ++i) {
+    float a = acc[i];
+    a += __shfl_xor(a, 1, 64);
+    a += __shfl_xor(a, 2, 64);
+    a += __shfl_xor(a, 4, 64);
+    if ((lane & 7) == 0) sm_o[wave][i * 8 + (lane >> 3)] = a;
+  }
+  if (lane == 0) {
+    sm_m[wave] = m;
+    sm_l[wave] = l;
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < DH; d += 256) {
+    float mm = fmaxf(fmaxf(sm_m[0], sm_m[1]), fmaxf(sm_m[2], sm_m[3]));
+    const float ms = mm == -INFINITY ? 0.f : mm;
+    float ll = 0.f, oo = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = __expf(sm_m[w] - ms);
+      ll += sm_l[w] * f;
+      oo += sm_o[w][d] * f;
+    }
+    if (num_splits == 1) {
+      out[(size_t)t * nq + h * DH + d] = (bf16_t)(oo / ll);
+    } else {
+      const size_t pi = ((size_t)dz * num_heads + h) * num_splits + split;
+      part_o[pi * DH + d] = oo;
+      if (d == 0) {
+        part_ml[pi * 2] = mm;
+        part_ml[pi * 2 + 1] = ll;
+      }
+    }
+  }
+}
+
+__global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                              const int* __restrict__ run_start, const int* __restrict__ decode_runs,
+                                              bf16_t* __restrict__ out, int num_heads, int head_size,
+                                              int num_splits) {
+  const int h = blockIdx.x, dz = blockIdx.y;
+  const int t = run_start[decode_runs[dz]];
+  const size_t base = ((size_t)dz * num_heads + h) * num_splits;
+  float mm = -INFINITY;
+  for (int s = 0; s < num_splits; ++s) mm = fmaxf(mm, part_ml[(base + s) * 2]);
+  for (int d = threadIdx.x; d < head_size; d += blockDim.x) {
+    float ll = 0.f, oo = 0.f;
+    for (int s = 0; s < num_splits; ++s) {
+      const float ms = part_ml[(base + s) * 2];
+      const float f = ms == -INFINITY ? 0.f : __expf(ms - mm);
+      ll += part_ml[(base + s) * 2 + 1] * f;
+      oo += part_o[(base + s) * head_size + d] * f;
+    }
+    out[((size_t)t * num_heads + h) * head_size + d] = (bf16_t)(oo / ll);
+  }
+}
+
+extern "C" int tnx_attention_decode(const void* q, const void* k_pages, const void* v_pages, const int* run_start,
+                                    const int* cached_lens, const int* table, int table_width, int page_size,
+                                    int num_pages, const int* decode_runs, int num_decode, void* out, float* part_o,
+                                    float* part_ml, int num_heads, int num_kv, int head_size, int window,
+                                    int num_splits, int keys_per_split, hipStream_t stream) {
+  TNX_REQUIRE(num_heads > 0 && num_kv > 0 && num_heads % num_kv == 0, "attention_decode: bad head counts");
+  TNX_REQUIRE(head_size == 16 || head_size == 32 || head_size == 64 || head_size == 128 || head_size == 256,
+              "attention_decode: head size %d is not one of 16, 32, 64, 128, 256", head_size);
+  TNX_REQUIRE(page_size % 16 == 0 && page_size > 0, "attention_decode: page size %d is not a multiple of 16",
+              page_size);
+  TNX_REQUIRE(num_splits >= 1 && keys_per_split > 0 && keys_per_split % 64 == 0,
+              "attention_decode: a split must hold a multiple of 64 keys");
+  TNX_REQUIRE(num_splits == 1 || (part_o && part_ml), "attention_decode: splits need a workspace");
+  TNX_REQUIRE(num_heads <= 65535 && num_decode <= 65535, "attention_decode: too many heads or requests");
+  if (num_decode <= 0) return 0;
+  dim3 grid(num_splits, num_heads, num_decode);
+#define LAUNCH_DECODE(CPR)                                                                                         \
+  attention_decode_kernel<CPR><<<grid, 256, 0, stream>>>(                                                          \
+      (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, table_width, \
+      page_size, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window, num_splits,     \
+      keys_per_split)
+  switch (head_size) {
+    case 16: LAUNCH_DECODE(2); break;
+    case 32: LAUNCH_DECODE(4); break;
+    case 64: LAUNCH_DECODE(8); break;
+    case 128: LAUNCH_DECODE(16); break;
+    default: LAUNCH_DECODE(32); break;
+  }
+#undef LAUNCH_DECODE
+  TNX_CHECK_LAUNCH("attention_decode");
+  if (num_splits > 1) {
+    attention_decode_merge_kernel<<<dim3(num_heads, num_decode), head_size < 64 ? 64 : head_size, 0, stream>>>(
+        part_o, part_ml, run_start, decode_runs, (bf16_t*)out, num_heads, head_size, num_splits);
+    TNX_CHECK_LAUNCH("attention_decode_merge");
+  }
+  return 0;
+}

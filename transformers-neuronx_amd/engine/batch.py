@@ -13,6 +13,9 @@ import numpy as np
 import torch
 
 
+QUERY_TILE = 128    # queries of one run that one block of the prompt attention kernel takes
+
+
 @dataclass
 class StepEntry:
     """A request's next tokens and the places among them whose logits are wanted."""
@@ -41,6 +44,9 @@ class StepContext:
     slots: torch.Tensor             # int32 [R], state slot of each request
     logits_rows: torch.Tensor       # int32 [M], tokens whose logits are wanted
     groups: Dict[str, GroupView]
+    decode_runs: torch.Tensor = None     # int32, the runs of one token (each attends with one query)
+    tile_run: torch.Tensor = None        # int32, for every tile of QUERY_TILE queries of the longer runs: its run
+    tile_start: torch.Tensor = None      # int32, and its first query within the run
     # The same on the host, for planning launches and for parts written in Python.
     run_lens_host: np.ndarray = None
     cached_lens_host: np.ndarray = None
@@ -74,7 +80,15 @@ def build_context(entries: List[StepEntry], cached: List[int], slots: List[int],
                 raise ValueError(f"request {e.req!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
             rows.append(run_start[i] + w)
     rows = np.array(rows, dtype=np.int32)
-    pieces = [token_ids, positions, token_request, run_start, cached_np, np.array(slots, dtype=np.int32), rows]
+    decode_runs = np.nonzero(run_lens == 1)[0].astype(np.int32)
+    tile_run, tile_start = [], []
+    for i in np.nonzero(run_lens > 1)[0]:
+        for q0 in range(0, int(run_lens[i]), QUERY_TILE):
+            tile_run.append(i)
+            tile_start.append(q0)
+    pieces = [token_ids, positions, token_request, run_start, cached_np, np.array(slots, dtype=np.int32), rows,
+              decode_runs, np.array(tile_run, dtype=np.int32), np.array(tile_start, dtype=np.int32)]
+    fixed = len(pieces)
     names = list(tables)
     pieces += [tables[g].reshape(-1) for g in names]
     # each piece starts at a multiple of 4 integers, so that every view is 16-byte aligned
@@ -88,9 +102,9 @@ def build_context(entries: List[StepEntry], cached: List[int], slots: List[int],
     dev = torch.from_numpy(flat).to(device)
     views = [dev[off:off + p.size] for off, p in zip(offsets, pieces)]
     groups = {}
-    for g, v in zip(names, views[7:]):
+    for g, v in zip(names, views[fixed:]):
         width = tables[g].shape[1]
         groups[g] = GroupView(v.view(r, width), page_size, width)
     return StepContext(t, r, views[0], views[1], views[2], views[3], views[4], views[5], views[6], groups,
-                       run_lens_host=run_lens, cached_lens_host=cached_np,
+                       decode_runs=views[7], tile_run=views[8], tile_start=views[9], run_lens_host=run_lens, cached_lens_host=cached_np,
                        slots_host=np.array(slots, dtype=np.int32))

@@ -38,6 +38,12 @@ _SIGNATURES = {
                           _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_attention_any": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                               _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_attention_prefill": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
+                                  _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
+                                  _c_void_p],
+        "tnx_attention_decode": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
+                                 _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+                                 _c_int, _c_int, _c_int, _c_void_p],
     },
     "sampling": {
         "tnx_ban_tokens": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
@@ -238,10 +244,48 @@ class HipOps:
         if ctx.max_total > view.width * view.page_size:
             raise ValueError("a request is longer than its block table")
         out = torch.empty_like(q)
-        self._call("attention", "tnx_attention_any", _ptr(q), _code(self.dtype), _ptr(k_pages), _ptr(v_pages),
-                   _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width, view.page_size,
-                   num_pages, _ptr(out), t, num_heads, num_kv_heads, head_size, int(window or 0), _stream())
+        window = int(window or 0)
+        fast = (self.dtype == torch.bfloat16 and not self.force_plain_attention
+                and (ctx.decode_runs.numel() == 0 or head_size in (16, 32, 64, 128, 256)))
+        if not fast:
+            self._call("attention", "tnx_attention_any", _ptr(q), _code(self.dtype), _ptr(k_pages), _ptr(v_pages),
+                       _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width,
+                       view.page_size, num_pages, _ptr(out), t, num_heads, num_kv_heads, head_size, window, _stream())
+            return out
+        if ctx.tile_run.numel():
+            self._call("attention", "tnx_attention_prefill", _ptr(q), _ptr(k_pages), _ptr(v_pages),
+                       _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(view.block_table), view.width,
+                       view.page_size, num_pages, _ptr(ctx.tile_run), _ptr(ctx.tile_start), ctx.tile_run.numel(),
+                       _ptr(out), num_heads, num_kv_heads, head_size, window, _stream())
+        n_dec = ctx.decode_runs.numel()
+        if n_dec:
+            splits, per_split = self._decode_splits(ctx, n_dec * num_heads, window)
+            part_o = part_ml = None
+            if splits > 1:
+                part_o = torch.empty(n_dec * num_heads * splits * head_size, dtype=torch.float32, device=q.device)
+                part_ml = torch.empty(n_dec * num_heads * splits * 2, dtype=torch.float32, device=q.device)
+            self._call("attention", "tnx_attention_decode", _ptr(q), _ptr(k_pages), _ptr(v_pages),
+                       _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(view.block_table), view.width,
+                       view.page_size, num_pages, _ptr(ctx.decode_runs), n_dec, _ptr(out), _ptr(part_o),
+                       _ptr(part_ml), num_heads, num_kv_heads, head_size, window, splits, per_split, _stream())
         return out
+
+    force_plain_attention = False     # tests set it to run the one-wave-per-query kernel in bfloat16 too
+    decode_blocks_wanted = 1024       # the keys of decoding requests are split until about this many blocks run
+
+    def _decode_splits(self, ctx, pairs: int, window: int):
+        """(splits, keys per split) for the decoding runs of a step: enough blocks to fill the chip,
+        no split shorter than 256 keys (one 64-key tile for each of a block's waves)."""
+        key = ("decode_splits", pairs, window)
+        if key not in ctx.plans:
+            single = ctx.run_lens_host == 1
+            longest = int((ctx.cached_lens_host[single] + 1).max())
+            if window:
+                longest = min(longest, window + 64)
+            splits = max(1, min(-(-self.decode_blocks_wanted // pairs), -(-longest // 256)))
+            per_split = -(-(-(-longest // splits)) // 64) * 64
+            ctx.plans[key] = (splits, per_split)
+        return ctx.plans[key]
 
     # ---------------------------------------------------------------- output end
 
