@@ -311,3 +311,38 @@ def test_bfloat16_attention_kernels_agree(case, window):
     one.decode_blocks_wanted = 1                  # no split at all
     o_one = one.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)
     torch.testing.assert_close(o_one.float(), o_plain.float(), rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv,hs,ps,runs,cached", [
+    (4, 4, 16, 16, [5, 1, 17], [0, 30, 3]), (6, 2, 48, 32, [70, 1], [0, 130]),
+    (2, 2, 128, 64, [1, 1, 65, 140], [511, 63, 64, 0]), (3, 1, 80, 16, [1], [4])])
+def test_fused_projection_writes_what_the_two_kernels_write(dtype, heads, kv, hs, ps, runs, cached):
+    hip, ref = _ops(dtype)
+    num_pages = sum(-(-(r + c) // ps) for r, c in zip(runs, cached)) + 2
+    ctx = _make_step(runs, cached, ps, num_pages, seed=hs)
+    view = ctx.groups["full"]
+    width = heads * hs
+    total = (heads + 2 * kv) * hs
+    g = torch.Generator(device=DEV).manual_seed(hs)
+    h = torch.randn(ctx.num_tokens, width, device=DEV, generator=g).to(dtype)
+    w = (torch.randn(total, width, device=DEV, generator=g) / math.sqrt(width)).to(dtype)
+    bias = torch.randn(total, device=DEV, generator=g) * 0.2
+    tol = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    variants = [0] if dtype == torch.float32 else [0, 1]
+    for b in (bias, None):
+        kp_r = torch.full((num_pages, kv, ps, hs), float("nan"), device=DEV, dtype=dtype)
+        vp_r = torch.full((num_pages, kv, hs, ps), float("nan"), device=DEV, dtype=dtype)
+        q_r = ref.qkv_project(h, w, b, heads, kv, hs, 0.3, ctx, view, kp_r, vp_r)
+        for variant in variants:
+            kp, vp = torch.full_like(kp_r, float("nan")), torch.full_like(vp_r, float("nan"))
+            q = hip.qkv_project(h, w, b, heads, kv, hs, 0.3, ctx, view, kp, vp, **({"force_tiled": variant}
+                                                                                  if dtype == torch.bfloat16 else {}))
+            torch.testing.assert_close(q.float(), q_r.float(), **tol)
+            assert torch.equal(torch.isnan(kp), torch.isnan(kp_r)) and torch.equal(torch.isnan(vp), torch.isnan(vp_r))
+            torch.testing.assert_close(torch.nan_to_num(kp.float()), torch.nan_to_num(kp_r.float()), **tol)
+            torch.testing.assert_close(torch.nan_to_num(vp.float()), torch.nan_to_num(vp_r.float()), **tol)
+    # a mixer that only reads another's cache projects queries alone
+    q = hip.qkv_project(h, w[:width].contiguous(), bias[:width].contiguous(), heads, 0, hs, 0.3, ctx, view, None, None)
+    q_r = ref.qkv_project(h, w[:width].contiguous(), bias[:width].contiguous(), heads, 0, hs, 0.3, ctx, view, None, None)
+    torch.testing.assert_close(q.float(), q_r.float(), **tol)

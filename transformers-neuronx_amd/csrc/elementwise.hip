@@ -70,41 +70,54 @@ extern "C" int tnx_cast(const void* src, int src_dtype, void* dst, int dst_dtype
 
 // LayerNorm of float32 rows: mean and biased variance in float32 (two passes over the row:
 // the variance is taken around the mean, not as E[x^2] - mean^2), then weight and bias.
-// One block of 256 threads per row; the row is kept in registers when it fits (width <= 256 * PER).
-template <int PER>
+// One block of 256 threads per row; the row lives in registers as PER float4 per thread
+// (width <= 1024 * PER, width % 4 == 0). Weight and bias are fetched before the reductions.
+template <int PER, bool AFFINE, bool F32_OUT, bool BF16_OUT>
 __global__ void __launch_bounds__(256)
 layernorm_kernel(const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ bias,
-                 float eps, float* __restrict__ out_f32, void* __restrict__ out_cd, int cd_dtype, int width) {
+                 float eps, float* __restrict__ out_f32, bf16_t* __restrict__ out_bf16, int width) {
+  typedef __attribute__((ext_vector_type(4))) float f4;
+  typedef __attribute__((ext_vector_type(4))) __bf16 b4;
   __shared__ float scratch[4];
   const int t = blockIdx.x;
-  const float* row = x + (size_t)t * width;
-  float v[PER];
+  const int w4 = width >> 2;
+  const f4* row = (const f4*)(x + (size_t)t * width);
+  f4 v[PER], gw[PER], gb[PER];
   float s = 0.f;
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
     const int i = threadIdx.x + j * 256;
-    v[j] = i < width ? row[i] : 0.f;
-    s += v[j];
+    const bool ok = i < w4;
+    v[j] = ok ? row[i] : (f4){0.f, 0.f, 0.f, 0.f};
+    if (AFFINE) {
+      gw[j] = ok ? ((const f4*)weight)[i] : (f4){0.f, 0.f, 0.f, 0.f};
+      gb[j] = ok ? ((const f4*)bias)[i] : (f4){0.f, 0.f, 0.f, 0.f};
+    }
+    s += (v[j].x + v[j].y) + (v[j].z + v[j].w);
   }
   const float mean = block_sum<4>(s, scratch) / (float)width;
   float q = 0.f;
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
-    const int i = threadIdx.x + j * 256;
-    const float d = i < width ? v[j] - mean : 0.f;
-    q += d * d;
+    if (threadIdx.x + j * 256 < w4) {
+      const f4 d = v[j] - mean;
+      q += (d.x * d.x + d.y * d.y) + (d.z * d.z + d.w * d.w);
+    }
   }
   const float var = block_sum<4>(q, scratch) / (float)width;
   const float rstd = rsqrtf(var + eps);
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
     const int i = threadIdx.x + j * 256;
-    if (i < width) {
-      float y = (v[j] - mean) * rstd;
-      if (weight) y *= weight[i];
-      if (bias) y += bias[i];
-      if (out_f32) out_f32[(size_t)t * width + i] = y;
-      if (out_cd) store_any(out_cd, cd_dtype, (size_t)t * width + i, y);
+    if (i < w4) {
+      f4 y = (v[j] - mean) * rstd;
+      if (AFFINE) y = y * gw[j] + gb[j];
+      if (F32_OUT) ((f4*)(out_f32 + (size_t)t * width))[i] = y;
+      if (BF16_OUT) {
+        b4 o;
+        o.x = (bf16_t)y.x; o.y = (bf16_t)y.y; o.z = (bf16_t)y.z; o.w = (bf16_t)y.w;
+        ((b4*)(out_bf16 + (size_t)t * width))[i] = o;
+      }
     }
   }
 }
@@ -141,14 +154,28 @@ extern "C" int tnx_layernorm(const float* x, const float* weight, const float* b
   TNX_REQUIRE(eps > 0.f, "layernorm: eps must be positive");
   TNX_REQUIRE(out_f32 != x, "layernorm: the float32 output may not alias the input");
   if (tokens == 0) return 0;
-  if (width <= 256 * 4)
-    layernorm_kernel<4><<<tokens, 256, 0, stream>>>(x, weight, bias, eps, out_f32, out_cd, cd_dtype, width);
-  else if (width <= 256 * 16)
-    layernorm_kernel<16><<<tokens, 256, 0, stream>>>(x, weight, bias, eps, out_f32, out_cd, cd_dtype, width);
-  else if (width <= 256 * 48)
-    layernorm_kernel<48><<<tokens, 256, 0, stream>>>(x, weight, bias, eps, out_f32, out_cd, cd_dtype, width);
-  else
+  const bool affine = weight != nullptr;
+  TNX_REQUIRE((weight != nullptr) == (bias != nullptr), "layernorm: weight and bias come together or not at all");
+  const bool vec = width % 4 == 0 && width <= 1024 * 16 && (cd_dtype == TNX_BF16 || out_cd == nullptr);
+  if (vec) {
+    bf16_t* ob = (bf16_t*)out_cd;
+#define LN_LAUNCH(PER, AFF, F, B) \
+  layernorm_kernel<PER, AFF, F, B><<<tokens, 256, 0, stream>>>(x, weight, bias, eps, out_f32, ob, width)
+#define LN_OUTS(PER, AFF)                                  \
+  if (out_f32 && ob) LN_LAUNCH(PER, AFF, true, true);      \
+  else if (ob) LN_LAUNCH(PER, AFF, false, true);           \
+  else LN_LAUNCH(PER, AFF, true, false)
+#define LN_AFF(PER)            \
+  if (affine) { LN_OUTS(PER, true); } else { LN_OUTS(PER, false); }
+    if (width <= 1024) { LN_AFF(1); }
+    else if (width <= 1024 * 4) { LN_AFF(4); }
+    else { LN_AFF(16); }
+#undef LN_AFF
+#undef LN_OUTS
+#undef LN_LAUNCH
+  } else {
     layernorm_wide_kernel<<<tokens, 256, 0, stream>>>(x, weight, bias, eps, out_f32, out_cd, cd_dtype, width);
+  }
   TNX_CHECK_LAUNCH("layernorm");
   return 0;
 }

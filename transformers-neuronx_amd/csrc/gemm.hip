@@ -20,6 +20,38 @@ __device__ __forceinline__ void epilogue_store(float v, int m, int n, int N, con
   store_any(out, out_dtype, o, v);
 }
 
+// Where the fused query/key/value projection puts its output: queries (scaled) into a dense matrix, the
+// keys and values of token m into the cache page `token_page[m]` at place `token_off[m]`
+// (keys [pages, kv_heads, page_size, head_size], values [pages, kv_heads, head_size, page_size]).
+struct QkvScatter {
+  const int* token_page;
+  const int* token_off;
+  bf16_t* q_out;
+  bf16_t* k_pages;
+  bf16_t* v_pages;
+  float scale;
+  int nq, nk, head_size, num_kv, page_size, num_pages;
+};
+
+__device__ __forceinline__ void qkv_store(float v, int m, int n, const float* bias, const QkvScatter& sc) {
+  if (bias) v += bias[n];
+  if (n < sc.nq) {
+    sc.q_out[(size_t)m * sc.nq + n] = (bf16_t)(v * sc.scale);
+    return;
+  }
+  const int page = sc.token_page[m], off = sc.token_off[m];
+  if (page < 0 || page >= sc.num_pages) return;
+  int j = n - sc.nq;
+  const bool is_key = j < sc.nk;
+  if (!is_key) j -= sc.nk;
+  const int h = j / sc.head_size, d = j - h * sc.head_size;
+  const size_t head = (size_t)page * sc.num_kv + h;
+  if (is_key)
+    sc.k_pages[(head * sc.page_size + off) * sc.head_size + d] = (bf16_t)v;
+  else
+    sc.v_pages[(head * sc.head_size + d) * sc.page_size + off] = (bf16_t)v;
+}
+
 // ------------------------------------------------------------------------------------------ float32
 
 #define F32_TILE 64
@@ -94,10 +126,11 @@ extern "C" int tnx_gemm_f32(const float* x, const float* w, const float* bias, c
 #define BT_K 32
 #define BT_STRIDE 40  // elements per staged row: 32 of data, 8 of padding against LDS bank conflicts
 
+template <bool QKV>
 __global__ void __launch_bounds__(256)
 gemm_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
                  const float* __restrict__ residual, void* __restrict__ out, int out_dtype, int act, int M, int N,
-                 int K) {
+                 int K, QkvScatter sc) {
   __shared__ __attribute__((aligned(16))) bf16_t xs[BT_M * BT_STRIDE];
   __shared__ __attribute__((aligned(16))) bf16_t ws[BT_N * BT_STRIDE];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -160,50 +193,75 @@ gemm_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, con
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int m = m0 + wm + i * 32 + 8 * (e >> 2) + 4 * lhalf + (e & 3);
-        if (m < M) epilogue_store(acc[i][j][e], m, n, N, bias, residual, out, out_dtype, act);
+        if (m < M) {
+          if (QKV)
+            qkv_store(acc[i][j][e], m, n, bias, sc);
+          else
+            epilogue_store(acc[i][j][e], m, n, N, bias, residual, out, out_dtype, act);
+        }
       }
     }
 }
 
 // ------------------------------------------------------------------------------------------ bfloat16, few rows
 
-// One block of four waves makes 16 columns of the output (16 rows of `w`) for all M <= 16 * MT rows of `x`.
-// The waves share the K axis in steps of 128; inside a step a lane reads 64 contiguous bytes of its weight
-// row, which the four MFMA steps consume in the same order from `x`, so the order of the sum over K is the
-// lane's own and needs no shuffle. The partial sums of the four waves meet in LDS.
-template <int MT>
-__global__ void __launch_bounds__(256)
+// One block of WAVES waves makes 16 columns of the output (16 rows of `w`) for all M <= 16 * MT rows of `x`.
+// The waves share the K axis in steps of 128; inside a step each of the four loads of a wave covers 64 contiguous bytes of
+// each of its 16 weight rows (the four lane groups side by side), and `x` is read the same way. DEPTH steps are loaded before the first is consumed, to keep enough
+// bytes in flight for the memory system. The partial sums of the waves meet in LDS.
+template <int MT, int WAVES, int DEPTH, bool QKV>
+__global__ void __launch_bounds__(WAVES * 64)
 gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
                         const float* __restrict__ residual, void* __restrict__ out, int out_dtype, int act, int M,
-                        int N, int K) {
-  __shared__ float red[4][MT][4][64];
+                        int N, int K, QkvScatter sc) {
+  __shared__ float red[WAVES][MT][4][64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 16;
   const bool n_ok = n0 + r < N;
-  const bf16_t* wrow = w + (size_t)(n_ok ? n0 + r : 0) * K;
+  const bf16_t* wrow = w + (size_t)(n_ok ? n0 + r : 0) * K + 8 * g;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   f32x4 acc[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-  for (int kb = wave * 128; kb < K; kb += 512) {
-    const int k_lane = kb + 32 * g;
-    bf16x8 wf[4];
+  const bf16_t* xrow[MT];
+  bool m_ok[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = t * 16 + r;
+    m_ok[t] = m < M;
+    xrow[t] = x + (size_t)(m_ok[t] ? m : 0) * K + 8 * g;
+  }
+  constexpr int STRIDE = WAVES * 128;
+  bf16x8 wf[DEPTH][4];
+  auto fetch = [&](int slot, int kb) {
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const int k = k_lane + 8 * s;
-      wf[s] = (n_ok && k + 8 <= K) ? *(const bf16x8*)(wrow + k) : zero;
+      const int k = kb + 8 * g + 32 * s;
+      wf[slot][s] = (n_ok && k + 8 <= K) ? *(const bf16x8*)(wrow + kb + 32 * s) : zero;
     }
+  };
+  const int kb0 = wave * 128;
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const int m = t * 16 + r;
-      const bf16_t* xrow = x + (size_t)(m < M ? m : 0) * K;
+  for (int d = 0; d < DEPTH; ++d) fetch(d, kb0 + d * STRIDE);
+  for (int kb = kb0; kb < K; kb += DEPTH * STRIDE) {
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const int k = k_lane + 8 * s;
-        const bf16x8 xf = (m < M && k + 8 <= K) ? *(const bf16x8*)(xrow + k) : zero;
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s], xf, acc[t], 0, 0, 0);
+    for (int d = 0; d < DEPTH; ++d) {
+      const int kc = kb + d * STRIDE;
+      bf16x8 cur[4];
+#pragma unroll
+      for (int s = 0; s < 4; ++s) cur[s] = wf[d][s];
+      fetch(d, kc + DEPTH * STRIDE);   // past the end of K it yields zeros and reads nothing
+      if (kc < K) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+#pragma unroll
+          for (int s = 0; s < 4; ++s) {
+            const int k = kc + 8 * g + 32 * s;
+            const bf16x8 xf = (m_ok[t] && k + 8 <= K) ? *(const bf16x8*)(xrow[t] + kc + 32 * s) : zero;
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[s], xf, acc[t], 0, 0, 0);
+          }
+        }
       }
     }
   }
@@ -213,44 +271,101 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
     for (int i = 0; i < 4; ++i) red[wave][t][i][lane] = acc[t][i];
   __syncthreads();
   // acc[t][i] of lane l is output column n0 + 4*(l/16) + i, row 16*t + l%16.
-  for (int idx = tid; idx < MT * 256; idx += 256) {
+  for (int idx = tid; idx < MT * 256; idx += WAVES * 64) {
     const int t = idx >> 8, i = (idx >> 6) & 3, l = idx & 63;
-    const float v = red[0][t][i][l] + red[1][t][i][l] + red[2][t][i][l] + red[3][t][i][l];
+    float v = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv) v += red[wv][t][i][l];
     const int n = n0 + 4 * (l >> 4) + i, m = t * 16 + (l & 15);
-    if (n < N && m < M) epilogue_store(v, m, n, N, bias, residual, out, out_dtype, act);
+    if (n < N && m < M) {
+      if (QKV)
+        qkv_store(v, m, n, bias, sc);
+      else
+        epilogue_store(v, m, n, N, bias, residual, out, out_dtype, act);
+    }
   }
 }
 
-extern "C" int tnx_gemm_bf16(const void* x, const void* w, const float* bias, const float* residual, void* out,
-                             int out_dtype, int act, int M, int N, int K, int force_tiled, hipStream_t stream) {
+template <int MT, int WAVES, int DEPTH>
+static void launch_skinny(const bf16_t* xp, const bf16_t* wp, const float* bias, const float* residual, void* out,
+                          int out_dtype, int act, int M, int N, int K, const QkvScatter* sc, hipStream_t stream) {
+  if (sc)
+    gemm_bf16_skinny_kernel<MT, WAVES, DEPTH, true><<<(N + 15) / 16, WAVES * 64, 0, stream>>>(
+        xp, wp, bias, residual, out, out_dtype, act, M, N, K, *sc);
+  else
+    gemm_bf16_skinny_kernel<MT, WAVES, DEPTH, false><<<(N + 15) / 16, WAVES * 64, 0, stream>>>(
+        xp, wp, bias, residual, out, out_dtype, act, M, N, K, QkvScatter{});
+}
+
+static int gemm_bf16_dispatch(const void* x, const void* w, const float* bias, const float* residual, void* out,
+                              int out_dtype, int act, int M, int N, int K, int force_tiled, const QkvScatter* sc,
+                              hipStream_t stream) {
   TNX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   TNX_REQUIRE(K % 8 == 0, "gemm_bf16: the inner size K=%d must be a multiple of 8", K);
   TNX_REQUIRE(((uintptr_t)x | (uintptr_t)w) % 16 == 0, "gemm_bf16: operands must be 16-byte aligned");
   if (M == 0) return 0;
   const bf16_t* xp = (const bf16_t*)x;
   const bf16_t* wp = (const bf16_t*)w;
-  if (M <= 64 && !force_tiled) {
-    const int blocks = (N + 15) / 16;
-    switch ((M + 15) / 16) {
-      case 1:
-        gemm_bf16_skinny_kernel<1><<<blocks, 256, 0, stream>>>(xp, wp, bias, residual, out, out_dtype, act, M, N, K);
-        break;
-      case 2:
-        gemm_bf16_skinny_kernel<2><<<blocks, 256, 0, stream>>>(xp, wp, bias, residual, out, out_dtype, act, M, N, K);
-        break;
-      case 3:
-        gemm_bf16_skinny_kernel<3><<<blocks, 256, 0, stream>>>(xp, wp, bias, residual, out, out_dtype, act, M, N, K);
-        break;
-      default:
-        gemm_bf16_skinny_kernel<4><<<blocks, 256, 0, stream>>>(xp, wp, bias, residual, out, out_dtype, act, M, N, K);
-        break;
+  if (M <= 64 && force_tiled != 1) {
+    // force_tiled > 1 picks a variant of the few-rows kernel, for measurements: 10 * waves + depth
+    const int variant = force_tiled > 1 ? force_tiled : (K >= 8192 ? 82 : 82);
+#define SKINNY(MT, WV, DP) launch_skinny<MT, WV, DP>(xp, wp, bias, residual, out, out_dtype, act, M, N, K, sc, stream)
+#define SKINNY_MT(WV, DP)                     \
+  switch ((M + 15) / 16) {                    \
+    case 1: SKINNY(1, WV, DP); break;         \
+    case 2: SKINNY(2, WV, DP); break;         \
+    case 3: SKINNY(3, WV, DP); break;         \
+    default: SKINNY(4, WV, DP); break;        \
+  }
+    switch (variant) {
+      case 41: SKINNY_MT(4, 1); break;
+      case 42: SKINNY_MT(4, 2); break;
+      case 81: SKINNY_MT(8, 1); break;
+      case 84: SKINNY_MT(8, 4); break;
+      case 44: SKINNY_MT(4, 4); break;
+      default: SKINNY_MT(8, 2); break;
     }
+#undef SKINNY_MT
+#undef SKINNY
     TNX_CHECK_LAUNCH("gemm_bf16_skinny");
     return 0;
   }
   dim3 grid((N + BT_N - 1) / BT_N, (M + BT_M - 1) / BT_M);
   TNX_REQUIRE(grid.y <= 65535, "gemm_bf16: M=%d is too large", M);
-  gemm_bf16_kernel<<<grid, 256, 0, stream>>>(xp, wp, bias, residual, out, out_dtype, act, M, N, K);
+  if (sc)
+    gemm_bf16_kernel<true><<<grid, 256, 0, stream>>>(xp, wp, bias, residual, out, out_dtype, act, M, N, K, *sc);
+  else
+    gemm_bf16_kernel<false><<<grid, 256, 0, stream>>>(xp, wp, bias, residual, out, out_dtype, act, M, N, K,
+                                                      QkvScatter{});
   TNX_CHECK_LAUNCH("gemm_bf16");
   return 0;
+}
+
+extern "C" int tnx_gemm_bf16(const void* x, const void* w, const float* bias, const float* residual, void* out,
+                             int out_dtype, int act, int M, int N, int K, int force_tiled, hipStream_t stream) {
+  return gemm_bf16_dispatch(x, w, bias, residual, out, out_dtype, act, M, N, K, force_tiled, nullptr, stream);
+}
+
+// The fused projection of queries, keys and values: `x w^T + bias` with w = [Wq; Wk; Wv] stacked by rows,
+// queries scaled and written densely, keys and values written straight into their cache pages.
+extern "C" int tnx_gemm_bf16_qkv(const void* x, const void* w, const float* bias, int M, int K, const int* token_page,
+                                 const int* token_off, void* q_out, void* k_pages, void* v_pages, float scale,
+                                 int num_heads, int num_kv, int head_size, int page_size, int num_pages,
+                                 int force_tiled, hipStream_t stream) {
+  TNX_REQUIRE(num_heads > 0 && num_kv >= 0 && head_size > 0 && page_size > 0, "gemm_bf16_qkv: bad sizes");
+  QkvScatter sc;
+  sc.token_page = token_page;
+  sc.token_off = token_off;
+  sc.q_out = (bf16_t*)q_out;
+  sc.k_pages = (bf16_t*)k_pages;
+  sc.v_pages = (bf16_t*)v_pages;
+  sc.scale = scale;
+  sc.nq = num_heads * head_size;
+  sc.nk = num_kv * head_size;
+  sc.head_size = head_size;
+  sc.num_kv = num_kv;
+  sc.page_size = page_size;
+  sc.num_pages = num_pages;
+  const int N = sc.nq + 2 * sc.nk;
+  return gemm_bf16_dispatch(x, w, bias, nullptr, nullptr, TNX_BF16, TNX_ACT_NONE, M, N, K, force_tiled, &sc, stream);
 }

@@ -30,6 +30,8 @@ class GroupView:
     block_table: torch.Tensor       # int32 [R, width], -1 where no page is held
     page_size: int
     width: int
+    token_page: torch.Tensor = None  # int32 [T], the page each token of the step is stored in
+    token_offset: torch.Tensor = None  # int32 [T], and its place inside that page
 
 
 @dataclass
@@ -91,6 +93,13 @@ def build_context(entries: List[StepEntry], cached: List[int], slots: List[int],
     fixed = len(pieces)
     names = list(tables)
     pieces += [tables[g].reshape(-1) for g in names]
+    for g in names:
+        blocks = positions // page_size
+        inside = blocks < tables[g].shape[1]
+        pieces.append(np.where(inside, tables[g][token_request, np.minimum(blocks, tables[g].shape[1] - 1)], -1)
+                      .astype(np.int32))
+    token_offset = (positions % page_size).astype(np.int32)
+    pieces.append(token_offset)
     # each piece starts at a multiple of 4 integers, so that every view is 16-byte aligned
     offsets, total = [], 0
     for p in pieces:
@@ -102,9 +111,11 @@ def build_context(entries: List[StepEntry], cached: List[int], slots: List[int],
     dev = torch.from_numpy(flat).to(device)
     views = [dev[off:off + p.size] for off, p in zip(offsets, pieces)]
     groups = {}
-    for g, v in zip(names, views[fixed:]):
+    n = len(names)
+    for i, g in enumerate(names):
         width = tables[g].shape[1]
-        groups[g] = GroupView(v.view(r, width), page_size, width)
+        groups[g] = GroupView(views[fixed + i].view(r, width), page_size, width,
+                              token_page=views[fixed + n + i], token_offset=views[fixed + 2 * n])
     return StepContext(t, r, views[0], views[1], views[2], views[3], views[4], views[5], views[6], groups,
                        decode_runs=views[7], tile_run=views[8], tile_start=views[9], run_lens_host=run_lens, cached_lens_host=cached_np,
                        slots_host=np.array(slots, dtype=np.int32))

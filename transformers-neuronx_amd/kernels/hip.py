@@ -32,6 +32,9 @@ _SIGNATURES = {
                          _c_int, _c_void_p],
         "tnx_gemm_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                           _c_int, _c_int, _c_void_p],
+        "tnx_gemm_bf16_qkv": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p,
+                              _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                              _c_void_p],
     },
     "attention": {
         "tnx_qkv_write": [_c_void_p, _c_int, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
@@ -218,6 +221,31 @@ class HipOps:
             raise ValueError(f"value pages have shape {tuple(v_pages.shape)}, expected "
                              f"{(n, num_kv, head_size, page_size)}")
         return n
+
+    def qkv_project(self, h, w, bias, num_heads, num_kv_write, head_size, scale, ctx, view, k_pages, v_pages,
+                    force_tiled=0):
+        """Queries, keys and values of the step's tokens: one matrix product whose epilogue scales the
+        queries and stores keys and values in their pages (bfloat16), or product and `qkv_write` apart."""
+        if self.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+            return self.qkv_write(self.linear(h, w, None), bias, num_heads, num_kv_write, head_size, scale, ctx,
+                                  view, k_pages, v_pages)
+        t = ctx.num_tokens
+        total = (num_heads + 2 * num_kv_write) * head_size
+        _want(h, "h", torch.bfloat16, (t, w.shape[1]))
+        _want(w, "w", torch.bfloat16, (total, h.shape[1]))
+        if bias is not None:
+            _want(bias, "qkv bias", torch.float32, (total,))
+        num_pages = 0
+        if num_kv_write:
+            num_pages = self._check_pages(k_pages, v_pages, num_kv_write, head_size, view.page_size)
+        _want(view.token_page, "token pages", torch.int32, (t,))
+        _want(view.token_offset, "token offsets", torch.int32, (t,))
+        q = torch.empty(t, num_heads * head_size, dtype=self.dtype, device=h.device)
+        self._call("gemm", "tnx_gemm_bf16_qkv", _ptr(h), _ptr(w), _ptr(bias), t, h.shape[1],
+                   _ptr(view.token_page), _ptr(view.token_offset), _ptr(q),
+                   _ptr(k_pages) if num_kv_write else None, _ptr(v_pages) if num_kv_write else None, float(scale),
+                   num_heads, num_kv_write, head_size, view.page_size, num_pages, int(force_tiled), _stream())
+        return q
 
     def qkv_write(self, qkv, bias, num_heads, num_kv_write, head_size, scale, ctx, view, k_pages, v_pages):
         t = ctx.num_tokens

@@ -89,6 +89,12 @@ class ReferenceOps:
 
     # ---------------------------------------------------------------- attention
 
+    def qkv_project(self, h, w, bias, num_heads, num_kv_write, head_size, scale, ctx, view, k_pages, v_pages):
+        """The projection to queries, keys and values (`w` holds the three stacked by rows), then
+        `qkv_write`."""
+        return self.qkv_write(self.linear(h, w, None), bias, num_heads, num_kv_write, head_size, scale, ctx, view,
+                              k_pages, v_pages)
+
     def qkv_write(self, qkv, bias, num_heads, num_kv_write, head_size, scale, ctx, view, k_pages, v_pages):
         """Bias, query scale, and the step's keys and values into their pages:
         page `table[run][position // page_size]`, place `position % page_size`."""

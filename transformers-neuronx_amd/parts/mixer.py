@@ -72,9 +72,9 @@ class Attention(Mixer):
         if cache.writes != self.own_kv:
             raise ValueError("an attention mixer with own_kv writes its cache; one without reads another's")
         view = ctx.groups[cache.group]
-        qkv = self.ops.linear(h, self.w_qkv, None)
-        q = self.ops.qkv_write(qkv, self.b_qkv, self.num_heads, self.num_kv_heads if self.own_kv else 0,
-                               self.head_size, self.scale, ctx, view, cache.k_pages, cache.v_pages)
+        q = self.ops.qkv_project(h, self.w_qkv, self.b_qkv, self.num_heads,
+                                 self.num_kv_heads if self.own_kv else 0, self.head_size, self.scale, ctx, view,
+                                 cache.k_pages, cache.v_pages)
         c = self.ops.attention(q, self.num_heads, self.num_kv_heads, self.head_size, ctx, view,
                                cache.k_pages, cache.v_pages, self.window)
         return self.ops.linear(c, self.w_out, self.b_out, residual=residual, out_f32=True)
