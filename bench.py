@@ -70,7 +70,8 @@ def main():
     dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     ecfg = EngineConfig(dtype=dtype, page_size=64, max_tokens=max_batch * CONTEXT, max_num_seqs=max_batch,
-                        max_num_batched_tokens=max(2048, PREFILL_TOKENS), max_model_len=CONTEXT)
+                        max_num_batched_tokens=max(2048, PREFILL_TOKENS), max_model_len=CONTEXT,
+                        prompts_first=True)
     t0 = time.time()
     runner = runner_from_random(cfg, seed=0, cfg=ecfg)
     torch.cuda.synchronize()
@@ -90,19 +91,21 @@ def main():
         for _ in range(batch):
             engine.add_request(torch.randint(3, cfg.vocab_size, (prompt_len,), generator=gen).tolist(), params)
         while any(not r.decoding for r in engine.requests.values()):
-            engine.step()
+            engine.step()                 # prompts first: nothing decodes until every prompt is in
+        assert all(len(r.output) == 1 for r in engine.requests.values())
         for _ in range(warmup):
             engine.step()
         torch.cuda.synchronize()
         start = time.perf_counter()
-        lens = 0
+        lens = made = 0
         for _ in range(steps):
             lens += sum(r.num_computed for r in engine.requests.values())
-            engine.step()
+            made += len(engine.step())
         torch.cuda.synchronize()
         sec = (time.perf_counter() - start) / steps
+        assert made == batch * steps, f"{made} tokens in {steps} steps of batch {batch}"
         read = runner.model.weight_bytes + lens / steps * kv_bytes_per_token
-        return batch / sec, sec, read
+        return made / (sec * steps), sec, read
 
     def prefill(tokens):
         engine.reset()

@@ -147,3 +147,17 @@ def test_decisions_depend_on_arrivals_and_lengths_only():
             out.append([(r.request.req_id, r.start, r.count) for r in runs])
         return out
     assert trace(iter(range(10, 1000))) == trace(iter(range(500, 1500)))
+
+
+def test_prompts_first_holds_decoding_until_every_prompt_is_in():
+    cache = CacheManager({0: CacheNeed("paged", kv_heads=1, head_size=16)}, 16, 32, 4, torch.float32, "cpu",
+                         allocate=False)
+    s = Scheduler(cache, 4, 40, 256, prompts_first=True)
+    s.add(_req("a", 30, new=5))
+    s.add(_req("b", 60, new=5))
+    seen = []
+    for _ in range(4):
+        runs, _ = _step(s, cache)
+        seen.append([(r.request.req_id, r.start, r.count) for r in runs])
+    # a is in after the first step and waits, with one token drawn, until b's prompt is in too
+    assert seen == [[("a", 0, 30), ("b", 0, 10)], [("b", 10, 40)], [("b", 50, 10)], [("a", 30, 1), ("b", 60, 1)]]

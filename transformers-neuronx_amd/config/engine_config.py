@@ -120,6 +120,8 @@ class EngineConfig:
     kernels          "hip" (the product path) or "reference" (the plain torch
                      rendition of every kernel, for debugging on any device;
                      never chosen by itself)
+    prompts_first    scheduling: take in every waiting prompt before the next decode step (default: decode
+                     steps go first and prompts fill what is left of the token budget)
     memory_fraction  share of free device memory the page pool may take when it
                      is sized from memory
     """
@@ -134,6 +136,7 @@ class EngineConfig:
     device: str = "cuda:0"
     memory_fraction: float = 0.85
     use_graphs: bool = True
+    prompts_first: bool = False
     seed: int = 0
 
     def __post_init__(self):

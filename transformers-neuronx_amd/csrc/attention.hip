@@ -392,17 +392,20 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
 
 // One query per request over its pages. The keys of a request are split over `num_splits` blocks; a block's
 // four waves take 64-key tiles in turn. A tile of keys of one head is read as it lies in memory, 16 bytes
-// a lane: lane l holds chunk l % CPR (8 head-size elements) of key l / CPR of each group of 64 / CPR keys,
-// so a score is a sum over CPR neighbouring lanes. Values lie transposed ([head_size][page_size]), so
-// lane l holds 8 keys (l % 8) of head-size element l / 8 of each group of 8 elements, and the output is a
-// sum over 8 neighbouring lanes, taken once at the end. Partial results (maximum, sum, weighted values,
-// all float32) of waves meet in LDS and those of splits in a workspace that a second kernel merges.
+// a lane: lane l holds chunk l % CPR (8 head-size elements) of key l / CPR of each group of 64 / CPR keys.
+// The partial dot products are summed over the CPR lanes of a key by a butterfly that halves what each lane
+// keeps at every step, so that in the end every lane holds the score of one key of the tile. Values lie
+// transposed ([head_size][page_size]), so lane l holds 8 keys (l % 8) of head-size element l / 8 of each
+// group of 8 elements, and the output is a sum over 8 neighbouring lanes, taken once at the end.
+// No load depends on a branch: keys beyond the request read a valid place and get weight zero.
+// Partial results (maximum, sum, weighted values, all float32) of waves meet in LDS and those of splits in
+// a workspace that a second kernel merges. The page size is a power of two here.
 template <int CPR>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, (CPR <= 8 ? 4 : (CPR == 16 ? 2 : 1)))
 attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                         const bf16_t* __restrict__ v_pages, const int* __restrict__ run_start,
                         const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
-                        int page_size, int num_pages, const int* __restrict__ decode_runs, bf16_t* __restrict__ out,
+                        int page_shift, int num_pages, const int* __restrict__ decode_runs, bf16_t* __restrict__ out,
                         float* __restrict__ part_o, float* __restrict__ part_ml, int num_heads, int num_kv,
                         int window, int num_splits, int keys_per_split) {
   constexpr int KPI = 64 / CPR;       // keys per load instruction of a wave
@@ -418,10 +421,12 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
   const int pos = cached_lens[run];   // the query's own position; its key is stored already
   const int* tab = table + (size_t)run * table_width;
   const int nq = num_heads * DH;
+  const int page_size = 1 << page_shift, pmask = page_size - 1;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int k_begin = (lo / 64) * 64 + split * keys_per_split;
   const int k_end = min(pos + 1, k_begin + keys_per_split);
   const int dchunk = lane % CPR, kgrp = lane / CPR;
+  const size_t head_stride = (size_t)page_size * DH;   // elements of one head of one page
 
   float qf[8];
   {
@@ -435,70 +440,64 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
   for (int i = 0; i < CPR; ++i) acc[i] = 0.f;
 
   for (int tile0 = k_begin + 64 * wave; tile0 < k_end; tile0 += 256) {
-    float s[CPR];
+    bf16x8 kv[CPR];
 #pragma unroll
     for (int i = 0; i < CPR; ++i) {
-      const int key = tile0 + i * KPI + kgrp;
-      bool valid = key >= lo && key < k_end;
-      float sum = 0.f;
-      if (valid) {
-        const int page = tab[key / page_size];
-        if (page >= 0 && page < num_pages) {
-          const bf16x8 kv = *(const bf16x8*)(k_pages + (((size_t)page * num_kv + kvh) * page_size +
-                                                        key % page_size) * DH + dchunk * 8);
-#pragma unroll
-          for (int j = 0; j < 8; ++j) sum = fmaf(qf[j], (float)kv[j], sum);
-        } else {
-          valid = false;
-        }
-      }
-#pragma unroll
-      for (int o = 1; o < CPR; o <<= 1) sum += __shfl_xor(sum, o, 64);
-      s[i] = valid ? sum : -INFINITY;
+      const int key = min(tile0 + i * KPI + kgrp, pos);
+      const int page = min(max(tab[key >> page_shift], 0), num_pages - 1);
+      kv[i] = *(const bf16x8*)(k_pages + ((size_t)page * num_kv + kvh) * head_stride + (size_t)(key & pmask) * DH +
+                               dchunk * 8);
     }
-    float mx = -INFINITY;
+    float part[CPR];
 #pragma unroll
-    for (int i = 0; i < CPR; ++i) mx = fmaxf(mx, s[i]);
+    for (int i = 0; i < CPR; ++i) {
+      float a = 0.f;
 #pragma unroll
-    for (int o = CPR; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-    const float m_new = fmaxf(m, mx);
+      for (int j = 0; j < 8; ++j) a = fmaf(qf[j], (float)kv[i][j], a);
+      part[i] = a;
+    }
+#pragma unroll
+    for (int half = CPR / 2; half >= 1; half >>= 1) {
+      const bool upper = (dchunk & half) != 0;
+#pragma unroll
+      for (int i = 0; i < half; ++i) {
+        const float keep = upper ? part[i + half] : part[i];
+        const float send = upper ? part[i] : part[i + half];
+        part[i] = keep + __shfl_xor(send, half, 64);
+      }
+    }
+    // this lane now holds the score of key tile0 + dchunk * KPI + kgrp
+    const int mine = dchunk * KPI + kgrp;
+    const bool valid = tile0 + mine >= lo && tile0 + mine < k_end;
+    const float sc = valid ? part[0] : -INFINITY;
+    const float m_new = fmaxf(m, wave_max(sc));
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
     const float alpha = __expf(m - m_safe);
-    float psum = 0.f;
-#pragma unroll
-    for (int i = 0; i < CPR; ++i) {
-      s[i] = __expf(s[i] - m_safe);
-      psum += s[i];
-    }
-#pragma unroll
-    for (int o = CPR; o < 64; o <<= 1) psum += __shfl_xor(psum, o, 64);
-    l = l * alpha + psum;
+    const float p = valid ? __expf(sc - m_safe) : 0.f;
+    l = l * alpha + wave_sum(p);
     m = m_new;
-    if (dchunk == 0) {
-#pragma unroll
-      for (int i = 0; i < CPR; ++i) sm_p[wave][i * KPI + kgrp] = s[i];
-    }
+    sm_p[wave][mine] = p;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // values of this tile: 8 keys a lane; fetched after the scores so that the registers of the keys are free
+    // again (more waves fit a SIMD, and it is other waves that hide the latency)
+    __builtin_amdgcn_sched_barrier(0);
     const int kc = lane & 7;
+    const int vkey = min(tile0 + kc * 8, pos & ~7);
+    const int vpage = min(max(tab[vkey >> page_shift], 0), num_pages - 1);
+    const bf16_t* vbase = v_pages + ((size_t)vpage * num_kv + kvh) * head_stride + (vkey & pmask);
+    bf16x8 vv[CPR];
+#pragma unroll
+    for (int i = 0; i < CPR; ++i) vv[i] = *(const bf16x8*)(vbase + (size_t)(i * 8 + (lane >> 3)) * page_size);
     float pv[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) pv[j] = sm_p[wave][kc * 8 + j];
-    const int key0 = tile0 + kc * 8;
-    int page = -1;
-    if (key0 < k_end) page = tab[key0 / page_size];
-    const bool vok = page >= 0 && page < num_pages;
-    const bf16_t* vbase = v_pages + ((size_t)(vok ? page : 0) * num_kv + kvh) * DH * page_size + key0 % page_size;
 #pragma unroll
     for (int i = 0; i < CPR; ++i) {
-      const int d = i * 8 + (lane >> 3);
       float a = acc[i] * alpha;
-      if (vok) {
-        const bf16x8 vv = *(const bf16x8*)(vbase + (size_t)d * page_size);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) a += pv[j] != 0.f ? pv[j] * (float)vv[j] : 0.f;
-      }
+      for (int j = 0; j < 8; ++j) a += pv[j] != 0.f ? pv[j] * (float)vv[i][j] : 0.f;
       acc[i] = a;
     }
     __builtin_amdgcn_wave_barrier();
@@ -568,8 +567,10 @@ extern "C" int tnx_attention_decode(const void* q, const void* k_pages, const vo
   TNX_REQUIRE(num_heads > 0 && num_kv > 0 && num_heads % num_kv == 0, "attention_decode: bad head counts");
   TNX_REQUIRE(head_size == 16 || head_size == 32 || head_size == 64 || head_size == 128 || head_size == 256,
               "attention_decode: head size %d is not one of 16, 32, 64, 128, 256", head_size);
-  TNX_REQUIRE(page_size % 16 == 0 && page_size > 0, "attention_decode: page size %d is not a multiple of 16",
-              page_size);
+  TNX_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0,
+              "attention_decode: page size %d is not a power of two from 16 up", page_size);
+  int page_shift = 0;
+  while ((1 << page_shift) < page_size) ++page_shift;
   TNX_REQUIRE(num_splits >= 1 && keys_per_split > 0 && keys_per_split % 64 == 0,
               "attention_decode: a split must hold a multiple of 64 keys");
   TNX_REQUIRE(num_splits == 1 || (part_o && part_ml), "attention_decode: splits need a workspace");
@@ -579,7 +580,7 @@ extern "C" int tnx_attention_decode(const void* q, const void* k_pages, const vo
 #define LAUNCH_DECODE(CPR)                                                                                         \
   attention_decode_kernel<CPR><<<grid, 256, 0, stream>>>(                                                          \
       (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, table_width, \
-      page_size, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window, num_splits,     \
+      page_shift, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window, num_splits,    \
       keys_per_split)
   switch (head_size) {
     case 16: LAUNCH_DECODE(2); break;

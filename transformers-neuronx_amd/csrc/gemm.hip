@@ -206,10 +206,14 @@ gemm_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, con
 // ------------------------------------------------------------------------------------------ bfloat16, few rows
 
 // One block of WAVES waves makes 16 columns of the output (16 rows of `w`) for all M <= 16 * MT rows of `x`.
-// The waves share the K axis in steps of 128; inside a step each of the four loads of a wave covers 64 contiguous bytes of
-// each of its 16 weight rows (the four lane groups side by side), and `x` is read the same way. DEPTH steps are loaded before the first is consumed, to keep enough
-// bytes in flight for the memory system. The partial sums of the waves meet in LDS.
-template <int MT, int WAVES, int DEPTH, bool QKV>
+// The waves share the K axis in steps of 128; inside a step each of the four loads of a wave covers 64
+// contiguous bytes of each of its 16 weight rows (the four lane groups side by side), and `x` is read the
+// same way. The weight is fetched two steps ahead of its use, `x` one step. No load in the main loop
+// is conditional: rows beyond N or M and steps beyond K read a valid address and their products are
+// dropped, so the compiler can keep many loads in flight. What is left of K after the last whole step of
+// 128 (K % 128, a multiple of 8) is done by wave 0 with guarded loads. The partial sums of the waves meet
+// in LDS.
+template <int MT, int WAVES, bool QKV>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
                         const float* __restrict__ residual, void* __restrict__ out, int out_dtype, int act, int M,
@@ -218,50 +222,70 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 16;
-  const bool n_ok = n0 + r < N;
-  const bf16_t* wrow = w + (size_t)(n_ok ? n0 + r : 0) * K + 8 * g;
+  const bf16_t* wrow = w + (size_t)min(n0 + r, N - 1) * K + 8 * g;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   f32x4 acc[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
   const bf16_t* xrow[MT];
-  bool m_ok[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int m = t * 16 + r;
-    m_ok[t] = m < M;
-    xrow[t] = x + (size_t)(m_ok[t] ? m : 0) * K + 8 * g;
-  }
+  for (int t = 0; t < MT; ++t) xrow[t] = x + (size_t)min(t * 16 + r, M - 1) * K + 8 * g;
   constexpr int STRIDE = WAVES * 128;
-  bf16x8 wf[DEPTH][4];
-  auto fetch = [&](int slot, int kb) {
+  const int k_full = K & ~127;          // whole steps end here
+  const int k_last = k_full - 128;      // the last whole step (negative if there is none)
+  if (k_full > 0) {
+    // Software pipeline over this wave's steps kb0, kb0 + STRIDE, ...: the weight is fetched two steps
+    // ahead and `x` one step ahead; the scheduling barriers keep the fetches of later steps in front of
+    // the products of the current one, so a product waits only for its own operands.
+    const int kb0 = wave * 128;
+    bf16x8 wf[3][4], xf[2][MT][4];
+    auto fetch_w = [&](int slot, int kc) {
+      const int k = min(kc, k_last);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) wf[slot][s] = *(const bf16x8*)(wrow + k + 32 * s);
+    };
+    auto fetch_x = [&](int slot, int kc) {
+      const int k = min(kc, k_last);
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) xf[slot][t][s] = *(const bf16x8*)(xrow[t] + k + 32 * s);
+    };
+    auto product = [&](int wslot, int xslot) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[wslot][s], xf[xslot][t][s], acc[t], 0, 0, 0);
+    };
+    fetch_x(0, kb0);
+    fetch_w(0, kb0);
+    fetch_w(1, kb0 + STRIDE);
+    // six steps a round, so that every buffer index is a constant (3 weight buffers, 2 x buffers)
+    for (int kb = kb0; kb < k_full; kb += 6 * STRIDE) {
+#pragma unroll
+      for (int u = 0; u < 6; ++u) {
+        const int kc = kb + u * STRIDE;
+        if (kc < k_full) {
+          fetch_x((u + 1) & 1, kc + STRIDE);
+          fetch_w((u + 2) % 3, kc + 2 * STRIDE);
+          __builtin_amdgcn_sched_barrier(0);
+          product(u % 3, u & 1);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+  }
+  if (wave == 0 && k_full < K) {
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const int k = kb + 8 * g + 32 * s;
-      wf[slot][s] = (n_ok && k + 8 <= K) ? *(const bf16x8*)(wrow + kb + 32 * s) : zero;
-    }
-  };
-  const int kb0 = wave * 128;
+      const int k = k_full + 32 * s + 8 * g;
+      const bool ok = k + 8 <= K;
+      const bf16x8 wv = ok ? *(const bf16x8*)(wrow + k_full + 32 * s) : zero;
 #pragma unroll
-  for (int d = 0; d < DEPTH; ++d) fetch(d, kb0 + d * STRIDE);
-  for (int kb = kb0; kb < K; kb += DEPTH * STRIDE) {
-#pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {
-      const int kc = kb + d * STRIDE;
-      bf16x8 cur[4];
-#pragma unroll
-      for (int s = 0; s < 4; ++s) cur[s] = wf[d][s];
-      fetch(d, kc + DEPTH * STRIDE);   // past the end of K it yields zeros and reads nothing
-      if (kc < K) {
-#pragma unroll
-        for (int t = 0; t < MT; ++t) {
-#pragma unroll
-          for (int s = 0; s < 4; ++s) {
-            const int k = kc + 8 * g + 32 * s;
-            const bf16x8 xf = (m_ok[t] && k + 8 <= K) ? *(const bf16x8*)(xrow[t] + kc + 32 * s) : zero;
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[s], xf, acc[t], 0, 0, 0);
-          }
-        }
+      for (int t = 0; t < MT; ++t) {
+        const bf16x8 xv = ok ? *(const bf16x8*)(xrow[t] + k_full + 32 * s) : zero;
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, xv, acc[t], 0, 0, 0);
       }
     }
   }
@@ -286,14 +310,14 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
   }
 }
 
-template <int MT, int WAVES, int DEPTH>
+template <int MT, int WAVES>
 static void launch_skinny(const bf16_t* xp, const bf16_t* wp, const float* bias, const float* residual, void* out,
                           int out_dtype, int act, int M, int N, int K, const QkvScatter* sc, hipStream_t stream) {
   if (sc)
-    gemm_bf16_skinny_kernel<MT, WAVES, DEPTH, true><<<(N + 15) / 16, WAVES * 64, 0, stream>>>(
+    gemm_bf16_skinny_kernel<MT, WAVES, true><<<(N + 15) / 16, WAVES * 64, 0, stream>>>(
         xp, wp, bias, residual, out, out_dtype, act, M, N, K, *sc);
   else
-    gemm_bf16_skinny_kernel<MT, WAVES, DEPTH, false><<<(N + 15) / 16, WAVES * 64, 0, stream>>>(
+    gemm_bf16_skinny_kernel<MT, WAVES, false><<<(N + 15) / 16, WAVES * 64, 0, stream>>>(
         xp, wp, bias, residual, out, out_dtype, act, M, N, K, QkvScatter{});
 }
 
@@ -307,23 +331,21 @@ static int gemm_bf16_dispatch(const void* x, const void* w, const float* bias, c
   const bf16_t* xp = (const bf16_t*)x;
   const bf16_t* wp = (const bf16_t*)w;
   if (M <= 64 && force_tiled != 1) {
-    // force_tiled > 1 picks a variant of the few-rows kernel, for measurements: 10 * waves + depth
-    const int variant = force_tiled > 1 ? force_tiled : (K >= 8192 ? 82 : 82);
-#define SKINNY(MT, WV, DP) launch_skinny<MT, WV, DP>(xp, wp, bias, residual, out, out_dtype, act, M, N, K, sc, stream)
-#define SKINNY_MT(WV, DP)                     \
-  switch ((M + 15) / 16) {                    \
-    case 1: SKINNY(1, WV, DP); break;         \
-    case 2: SKINNY(2, WV, DP); break;         \
-    case 3: SKINNY(3, WV, DP); break;         \
-    default: SKINNY(4, WV, DP); break;        \
+    // Eight waves a block when the sum over K is long and the rows are few (more bytes in flight for each
+    // of the few blocks), four otherwise. force_tiled 4 or 8 picks the count, for measurements.
+    const int waves = force_tiled == 4 || force_tiled == 8 ? force_tiled : (K >= 8192 && N <= 8192 ? 8 : 4);
+#define SKINNY(MT, WV) launch_skinny<MT, WV>(xp, wp, bias, residual, out, out_dtype, act, M, N, K, sc, stream)
+#define SKINNY_MT(WV)                     \
+  switch ((M + 15) / 16) {                \
+    case 1: SKINNY(1, WV); break;         \
+    case 2: SKINNY(2, WV); break;         \
+    case 3: SKINNY(3, WV); break;         \
+    default: SKINNY(4, WV); break;        \
   }
-    switch (variant) {
-      case 41: SKINNY_MT(4, 1); break;
-      case 42: SKINNY_MT(4, 2); break;
-      case 81: SKINNY_MT(8, 1); break;
-      case 84: SKINNY_MT(8, 4); break;
-      case 44: SKINNY_MT(4, 4); break;
-      default: SKINNY_MT(8, 2); break;
+    if (waves == 8) {
+      SKINNY_MT(8);
+    } else {
+      SKINNY_MT(4);
     }
 #undef SKINNY_MT
 #undef SKINNY

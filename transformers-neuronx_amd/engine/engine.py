@@ -29,7 +29,8 @@ class LLMEngine:
     def __init__(self, runner: ModelRunner, config: EngineConfig):
         self.runner, self.config = runner, config
         max_len = min(config.max_model_len or runner.max_positions, runner.max_positions)
-        self.scheduler = Scheduler(runner.cache, config.max_num_seqs, config.max_num_batched_tokens, max_len)
+        self.scheduler = Scheduler(runner.cache, config.max_num_seqs, config.max_num_batched_tokens, max_len,
+                                   prompts_first=config.prompts_first)
         self.sampler = Sampler(runner.ops, runner.model.device)
         self.requests: Dict[Hashable, Request] = {}
         self._ids = itertools.count()

@@ -67,12 +67,15 @@ class ScheduledRun:
 
 class Scheduler:
     def __init__(self, cache: CacheManager, max_num_seqs: int, max_num_batched_tokens: int, max_model_len: int,
-                 max_portion: Optional[int] = None):
+                 max_portion: Optional[int] = None, prompts_first: bool = False):
         self.cache = cache
         self.max_num_seqs = min(max_num_seqs, cache.max_seqs)
         self.max_num_batched_tokens = max_num_batched_tokens
         self.max_model_len = max_model_len
         self.max_portion = max_portion or max_num_batched_tokens
+        # prompts_first: while any prompt is waiting or under way, decoding requests wait (all prompts
+        # are taken in before the first decode step); otherwise decoding requests go first every step
+        self.prompts_first = prompts_first
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []        # in admission order
         self.finished: List[Request] = []
@@ -145,8 +148,9 @@ class Scheduler:
         planned: List[ScheduledRun] = []
         blocked = False                       # pages ran out: admit nothing new this step
         # 1. one token for every decoding request, oldest first
+        hold = self.prompts_first and (bool(self.waiting) or any(not r.decoding for r in self.running))
         for req in list(self.running):
-            if req not in self.running or not req.decoding or budget <= 0:
+            if hold or req not in self.running or not req.decoding or budget <= 0:
                 continue
             before = self.num_preemptions
             if self._reserve(req, req.num_computed + 1, planned):
