@@ -173,3 +173,48 @@ def test_trace_run_as_a_program(tiny_folders, tmp_path):
         assert proc.returncode == 0, proc.stderr
         assert proc.stdout.split() == [w for s in steps for w in ("done", str(s["step"]))]
         _compare(str(out), place, expected, cfg["vocab_size"], dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recorded_decode_steps_equal_open_ones(tiny_folders, tiny_folders_bf16, dtype):
+    """Decode steps replayed from a recording give the logits of steps launched in the open, replay after
+    replay, with prompt steps and other batch sizes in between."""
+    from transformers_neuronx_amd.config import EngineConfig
+    from transformers_neuronx_amd.engine import StepEntry
+    from transformers_neuronx_amd.engine.factory import runner_from_folder
+    folder, cfg, weights = (tiny_folders if dtype == "float32" else tiny_folders_bf16)["B"]
+    requests = _requests(cfg, [60, 3, 90], seed=17)
+    expected = _expected(weights, cfg, requests)
+
+    def run(use_graphs):
+        ecfg = EngineConfig(dtype=dtype, page_size=16, max_tokens=512, max_num_seqs=4, use_graphs=use_graphs)
+        runner = runner_from_folder(folder, ecfg)
+        rows = {}
+        pos = {rid: 0 for rid in requests}
+
+        def step(parts):
+            entries = [StepEntry(rid, requests[rid][pos[rid]:pos[rid] + n], [n - 1]) for rid, n in parts]
+            logits = runner.step(entries).clone()
+            for i, (rid, n) in enumerate(parts):
+                pos[rid] += n
+                rows[(rid, pos[rid] - 1)] = logits[i].cpu()
+        step([("r0", 20), ("r2", 50)])
+        for _ in range(6):
+            step([("r0", 1), ("r2", 1)])                 # recorded at batch 2
+        step([("r1", 1)])                                 # a first token, batch 1
+        for _ in range(2):
+            step([("r0", 1), ("r1", 1), ("r2", 1)])      # batch 3
+        step([("r0", 5), ("r2", 1)])                      # mixed: not recorded
+        for _ in range(8):
+            step([("r0", 1), ("r2", 1)])                 # batch 2 again: replayed
+        return rows, runner.graph_replays
+
+    open_rows, n_open = run(False)
+    rec_rows, n_rec = run(True)
+    assert n_open == 0 and n_rec == 6 + 1 + 2 + 8
+    assert open_rows.keys() == rec_rows.keys()
+    for key in open_rows:
+        rid, p = key
+        assert torch.equal(open_rows[key], rec_rows[key]), key
+        want = expected[rid][p]
+        assert float((rec_rows[key] - want).abs().max() / expected[rid].abs().max()) <= TOL[dtype]

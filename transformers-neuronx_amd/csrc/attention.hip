@@ -407,7 +407,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                         const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
                         int page_shift, int num_pages, const int* __restrict__ decode_runs, bf16_t* __restrict__ out,
                         float* __restrict__ part_o, float* __restrict__ part_ml, int num_heads, int num_kv,
-                        int window, int num_splits, int keys_per_split) {
+                        int window, int num_splits, const int* __restrict__ longest_ptr) {
   constexpr int KPI = 64 / CPR;       // keys per load instruction of a wave
   constexpr int DH = CPR * 8;
   __shared__ float sm_p[4][64];
@@ -423,6 +423,10 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
   const int nq = num_heads * DH;
   const int page_size = 1 << page_shift, pmask = page_size - 1;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  // The longest range of keys any decoding request of the step reads is given in device memory, so that a
+  // recorded launch stays valid while the requests grow; every split takes an equal share of it, in 64s.
+  const int longest = window > 0 ? min(longest_ptr[0], window + 64) : longest_ptr[0];
+  const int keys_per_split = (((longest + num_splits - 1) / num_splits) + 63) & ~63;
   const int k_begin = (lo / 64) * 64 + split * keys_per_split;
   const int k_end = min(pos + 1, k_begin + keys_per_split);
   const int dchunk = lane % CPR, kgrp = lane / CPR;
@@ -563,7 +567,7 @@ extern "C" int tnx_attention_decode(const void* q, const void* k_pages, const vo
                                     const int* cached_lens, const int* table, int table_width, int page_size,
                                     int num_pages, const int* decode_runs, int num_decode, void* out, float* part_o,
                                     float* part_ml, int num_heads, int num_kv, int head_size, int window,
-                                    int num_splits, int keys_per_split, hipStream_t stream) {
+                                    int num_splits, const int* longest, hipStream_t stream) {
   TNX_REQUIRE(num_heads > 0 && num_kv > 0 && num_heads % num_kv == 0, "attention_decode: bad head counts");
   TNX_REQUIRE(head_size == 16 || head_size == 32 || head_size == 64 || head_size == 128 || head_size == 256,
               "attention_decode: head size %d is not one of 16, 32, 64, 128, 256", head_size);
@@ -571,8 +575,7 @@ extern "C" int tnx_attention_decode(const void* q, const void* k_pages, const vo
               "attention_decode: page size %d is not a power of two from 16 up", page_size);
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
-  TNX_REQUIRE(num_splits >= 1 && keys_per_split > 0 && keys_per_split % 64 == 0,
-              "attention_decode: a split must hold a multiple of 64 keys");
+  TNX_REQUIRE(num_splits >= 1 && longest != nullptr, "attention_decode: bad split count or no length given");
   TNX_REQUIRE(num_splits == 1 || (part_o && part_ml), "attention_decode: splits need a workspace");
   TNX_REQUIRE(num_heads <= 65535 && num_decode <= 65535, "attention_decode: too many heads or requests");
   if (num_decode <= 0) return 0;
@@ -581,7 +584,7 @@ extern "C" int tnx_attention_decode(const void* q, const void* k_pages, const vo
   attention_decode_kernel<CPR><<<grid, 256, 0, stream>>>(                                                          \
       (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, table_width, \
       page_shift, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window, num_splits,    \
-      keys_per_split)
+      longest)
   switch (head_size) {
     case 16: LAUNCH_DECODE(2); break;
     case 32: LAUNCH_DECODE(4); break;

@@ -49,6 +49,11 @@ class StepContext:
     decode_runs: torch.Tensor = None     # int32, the runs of one token (each attends with one query)
     tile_run: torch.Tensor = None        # int32, for every tile of QUERY_TILE queries of the longer runs: its run
     tile_start: torch.Tensor = None      # int32, and its first query within the run
+    longest_decode: torch.Tensor = None  # int32 [1], the most keys a one-token run of this step reads
+    longest_decode_host: int = 0
+    # When a step is recorded for replay, nothing in its launches may depend on the lengths of this
+    # particular step: `length_bound` then stands in for them where a launch is sized.
+    length_bound: Optional[int] = None
     # The same on the host, for planning launches and for parts written in Python.
     run_lens_host: np.ndarray = None
     cached_lens_host: np.ndarray = None
@@ -64,9 +69,33 @@ class StepContext:
         return int((self.run_lens_host + self.cached_lens_host).max())
 
 
-def build_context(entries: List[StepEntry], cached: List[int], slots: List[int],
-                  tables: Dict[str, np.ndarray], page_size: int, device) -> StepContext:
-    """Pack a step's integers into one buffer, copy it once, and slice it."""
+@dataclass
+class PackedStep:
+    """A step's integers in one host array, and where each piece lies."""
+    flat: np.ndarray
+    offsets: List[int]
+    sizes: List[int]
+    num_tokens: int
+    num_requests: int
+    group_names: List[str]
+    widths: Dict[str, int]
+    page_size: int
+    run_lens: np.ndarray
+    cached: np.ndarray
+    slots: np.ndarray
+    longest_decode: int
+
+    def layout(self):
+        """What two steps must share for one to reuse the other's device buffer and views."""
+        return (tuple(self.offsets), tuple(self.sizes), self.num_tokens, self.num_requests,
+                tuple(self.group_names), tuple(sorted(self.widths.items())), self.page_size)
+
+
+_FIXED_PIECES = 11   # pieces before the per-group ones, see pack_step
+
+
+def pack_step(entries: List[StepEntry], cached: List[int], slots: List[int], tables: Dict[str, np.ndarray],
+              page_size: int) -> PackedStep:
     run_lens = np.array([len(e.tokens) for e in entries], dtype=np.int32)
     cached_np = np.array(cached, dtype=np.int32)
     r, t = len(entries), int(run_lens.sum())
@@ -82,15 +111,18 @@ def build_context(entries: List[StepEntry], cached: List[int], slots: List[int],
                 raise ValueError(f"request {e.req!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
             rows.append(run_start[i] + w)
     rows = np.array(rows, dtype=np.int32)
-    decode_runs = np.nonzero(run_lens == 1)[0].astype(np.int32)
+    single = run_lens == 1
+    decode_runs = np.nonzero(single)[0].astype(np.int32)
+    longest = int((cached_np[single] + 1).max()) if single.any() else 0
     tile_run, tile_start = [], []
     for i in np.nonzero(run_lens > 1)[0]:
         for q0 in range(0, int(run_lens[i]), QUERY_TILE):
             tile_run.append(i)
             tile_start.append(q0)
     pieces = [token_ids, positions, token_request, run_start, cached_np, np.array(slots, dtype=np.int32), rows,
-              decode_runs, np.array(tile_run, dtype=np.int32), np.array(tile_start, dtype=np.int32)]
-    fixed = len(pieces)
+              decode_runs, np.array(tile_run, dtype=np.int32), np.array(tile_start, dtype=np.int32),
+              np.array([longest], dtype=np.int32)]
+    assert len(pieces) == _FIXED_PIECES
     names = list(tables)
     pieces += [tables[g].reshape(-1) for g in names]
     for g in names:
@@ -98,8 +130,7 @@ def build_context(entries: List[StepEntry], cached: List[int], slots: List[int],
         inside = blocks < tables[g].shape[1]
         pieces.append(np.where(inside, tables[g][token_request, np.minimum(blocks, tables[g].shape[1] - 1)], -1)
                       .astype(np.int32))
-    token_offset = (positions % page_size).astype(np.int32)
-    pieces.append(token_offset)
+    pieces.append((positions % page_size).astype(np.int32))
     # each piece starts at a multiple of 4 integers, so that every view is 16-byte aligned
     offsets, total = [], 0
     for p in pieces:
@@ -108,14 +139,28 @@ def build_context(entries: List[StepEntry], cached: List[int], slots: List[int],
     flat = np.zeros(max(total, 4), dtype=np.int32)
     for off, p in zip(offsets, pieces):
         flat[off:off + p.size] = p
-    dev = torch.from_numpy(flat).to(device)
-    views = [dev[off:off + p.size] for off, p in zip(offsets, pieces)]
+    return PackedStep(flat, offsets, [p.size for p in pieces], t, r, names,
+                      {g: tables[g].shape[1] for g in names}, page_size, run_lens, cached_np,
+                      np.array(slots, dtype=np.int32), longest)
+
+
+def context_from(packed: PackedStep, dev: torch.Tensor) -> StepContext:
+    """Views of the device copy `dev` of a packed step."""
+    views = [dev[off:off + n] for off, n in zip(packed.offsets, packed.sizes)]
     groups = {}
-    n = len(names)
-    for i, g in enumerate(names):
-        width = tables[g].shape[1]
-        groups[g] = GroupView(views[fixed + i].view(r, width), page_size, width,
-                              token_page=views[fixed + n + i], token_offset=views[fixed + 2 * n])
-    return StepContext(t, r, views[0], views[1], views[2], views[3], views[4], views[5], views[6], groups,
-                       decode_runs=views[7], tile_run=views[8], tile_start=views[9], run_lens_host=run_lens, cached_lens_host=cached_np,
-                       slots_host=np.array(slots, dtype=np.int32))
+    n = len(packed.group_names)
+    for i, g in enumerate(packed.group_names):
+        width = packed.widths[g]
+        groups[g] = GroupView(views[_FIXED_PIECES + i].view(packed.num_requests, width), packed.page_size, width,
+                              token_page=views[_FIXED_PIECES + n + i], token_offset=views[_FIXED_PIECES + 2 * n])
+    return StepContext(packed.num_tokens, packed.num_requests, views[0], views[1], views[2], views[3], views[4],
+                       views[5], views[6], groups, decode_runs=views[7], tile_run=views[8], tile_start=views[9],
+                       longest_decode=views[10], run_lens_host=packed.run_lens, cached_lens_host=packed.cached,
+                       slots_host=packed.slots, longest_decode_host=packed.longest_decode)
+
+
+def build_context(entries: List[StepEntry], cached: List[int], slots: List[int],
+                  tables: Dict[str, np.ndarray], page_size: int, device) -> StepContext:
+    """Pack a step's integers into one buffer, copy it once, and slice it."""
+    packed = pack_step(entries, cached, slots, tables, page_size)
+    return context_from(packed, torch.from_numpy(packed.flat).to(device))

@@ -44,7 +44,7 @@ def build_runner(model_config, source, cfg: EngineConfig) -> ModelRunner:
     needs = model.cache_needs()
     num_pages = size_page_pool(cfg, CacheManager.bytes_per_page(needs, cfg.page_size, cfg.dtype), device)
     cache = CacheManager(needs, cfg.page_size, num_pages, cfg.max_num_seqs, cfg.dtype, device)
-    return ModelRunner(model, cache, ops)
+    return ModelRunner(model, cache, ops, use_graphs=cfg.use_graphs)
 
 
 def runner_from_folder(folder: str, cfg: EngineConfig) -> ModelRunner:

@@ -57,6 +57,10 @@ class DecoderModel:
             elif cid not in written:
                 raise ValueError(f"layer {layer} reads cache {cid} before the call that writes it")
         self.loaded = False
+        parts = [self.embedding, self.embedding.position, self.head] + ([self.head.norm] if self.head.norm else [])
+        for l in self.layers:
+            parts += [l.block, l.mixer, l.feed_forward, l.mixer_norm, l.feed_forward_norm]
+        self.recordable = all(getattr(p, "recordable", False) for p in parts)
 
     # ---------------------------------------------------------------- declarations
 

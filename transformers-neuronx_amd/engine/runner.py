@@ -14,19 +14,58 @@ from typing import Dict, Hashable, List, Optional
 
 import torch
 
+import numpy as np
+
 from ..cache.manager import CacheManager
-from .batch import StepContext, StepEntry, build_context
+from .batch import PackedStep, StepContext, StepEntry, context_from, pack_step
 from .model import DecoderModel
 
 
+class _RecordedStep:
+    """A decode step recorded as a HIP graph: the launches of one step over a fixed number of
+    one-token runs, reading their integers from a device buffer that is rewritten before each replay.
+    The reference keeps one compiled program per (bucket, batch size) and binds its buffers once
+    (decoder.py:2099-2325); this is the counterpart without buckets: what varies between steps is data."""
+
+    def __init__(self, runner: "ModelRunner", packed: PackedStep):
+        dev = runner.model.device
+        self.layout = packed.layout()
+        self.host = torch.empty(packed.flat.size, dtype=torch.int32, pin_memory=True)
+        self.host.numpy()[:] = packed.flat
+        self.static = self.host.to(dev)
+        self.ctx = context_from(packed, self.static)
+        self.ctx.length_bound = runner.max_positions
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):           # once in the open: loads libraries, warms the allocator
+            runner.model.forward(self.ctx, runner.cache.caches)
+        torch.cuda.current_stream(dev).wait_stream(side)
+        torch.cuda.synchronize(dev)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.logits = runner.model.forward(self.ctx, runner.cache.caches)
+
+    def replay(self, packed: PackedStep) -> torch.Tensor:
+        self.host.numpy()[:] = packed.flat
+        self.static.copy_(self.host, non_blocking=True)
+        self.graph.replay()
+        return self.logits
+
+
 class ModelRunner:
-    def __init__(self, model: DecoderModel, cache: CacheManager, ops):
+    def __init__(self, model: DecoderModel, cache: CacheManager, ops, use_graphs: bool = False):
         self.model, self.cache, self.ops = model, cache, ops
         self.vocab = model.spec.vocab_size
         self.max_positions = model.spec.max_positions
+        # decode-only steps are recorded once per batch size and replayed (HIP kernels only)
+        self.use_graphs = use_graphs and getattr(ops, "name", "") == "hip" and model.recordable
+        self._recorded: Dict[tuple, _RecordedStep] = {}
+        self.graph_replays = 0
 
-    def prepare(self, entries: List[StepEntry]) -> StepContext:
-        """Admit new requests, get pages for the step's tokens, lay out the batch."""
+    def prepare(self, entries: List[StepEntry], fixed_width: bool = False) -> PackedStep:
+        """Admit new requests, get pages for the step's tokens, lay out the batch. With `fixed_width`
+        the block tables are as wide as the longest request the model allows, so that every step of
+        the same batch size has the same layout."""
         seen = set()
         for e in entries:
             if e.req in seen:
@@ -50,7 +89,13 @@ class ModelRunner:
         cached = [self.cache.num_tokens(r) for r in reqs]
         slots = [self.cache.slot_of(r) for r in reqs]
         tables = {g: self.cache.block_table(reqs, g) for g in self.cache.groups}
-        return build_context(entries, cached, slots, tables, self.cache.page_size, self.model.device)
+        if fixed_width:
+            full = -(-self.max_positions // self.cache.page_size)
+            for g, t in tables.items():
+                wide = np.full((t.shape[0], full), -1, dtype=np.int32)
+                wide[:, :t.shape[1]] = t
+                tables[g] = wide
+        return pack_step(entries, cached, slots, tables, self.cache.page_size)
 
     @torch.no_grad()
     def step(self, entries: List[StepEntry]) -> Optional[torch.Tensor]:
@@ -58,11 +103,21 @@ class ModelRunner:
         their `want`; None when nothing is wanted (the step still runs)."""
         if not entries:
             return None
-        ctx = self.prepare(entries)
-        logits = self.model.forward(ctx, self.cache.caches)
+        recordable = self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
+        packed = self.prepare(entries, fixed_width=recordable)
+        if recordable:
+            key = packed.layout()
+            rec = self._recorded.get(key)
+            if rec is None:
+                rec = self._recorded[key] = _RecordedStep(self, packed)
+            logits = rec.replay(packed)
+            self.graph_replays += 1
+        else:
+            ctx = context_from(packed, torch.from_numpy(packed.flat).to(self.model.device))
+            logits = self.model.forward(ctx, self.cache.caches)
         for e in entries:
             self.cache.advance(e.req, len(e.tokens))
-        return logits if ctx.logits_rows.numel() else None
+        return logits if any(len(e.want) for e in entries) else None
 
     def finish(self, req: Hashable) -> None:
         """The request is over: its pages and its slot go back."""

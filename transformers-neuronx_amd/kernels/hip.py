@@ -46,7 +46,7 @@ _SIGNATURES = {
                                   _c_void_p],
         "tnx_attention_decode": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                  _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
-                                 _c_int, _c_int, _c_int, _c_void_p],
+                                 _c_int, _c_int, _c_void_p, _c_void_p],
     },
     "sampling": {
         "tnx_ban_tokens": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
@@ -288,7 +288,7 @@ class HipOps:
                        _ptr(out), num_heads, num_kv_heads, head_size, window, _stream())
         n_dec = ctx.decode_runs.numel()
         if n_dec:
-            splits, per_split = self._decode_splits(ctx, n_dec * num_heads, window)
+            splits = self._decode_splits(ctx, n_dec * num_heads, window)
             part_o = part_ml = None
             if splits > 1:
                 part_o = torch.empty(n_dec * num_heads * splits * head_size, dtype=torch.float32, device=q.device)
@@ -296,25 +296,21 @@ class HipOps:
             self._call("attention", "tnx_attention_decode", _ptr(q), _ptr(k_pages), _ptr(v_pages),
                        _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(view.block_table), view.width,
                        view.page_size, num_pages, _ptr(ctx.decode_runs), n_dec, _ptr(out), _ptr(part_o),
-                       _ptr(part_ml), num_heads, num_kv_heads, head_size, window, splits, per_split, _stream())
+                       _ptr(part_ml), num_heads, num_kv_heads, head_size, window, splits, _ptr(ctx.longest_decode),
+                       _stream())
         return out
 
     force_plain_attention = False     # tests set it to run the one-wave-per-query kernel in bfloat16 too
     decode_blocks_wanted = 1024       # the keys of decoding requests are split until about this many blocks run
 
-    def _decode_splits(self, ctx, pairs: int, window: int):
-        """(splits, keys per split) for the decoding runs of a step: enough blocks to fill the chip,
-        no split shorter than 256 keys (one 64-key tile for each of a block's waves)."""
-        key = ("decode_splits", pairs, window)
-        if key not in ctx.plans:
-            single = ctx.run_lens_host == 1
-            longest = int((ctx.cached_lens_host[single] + 1).max())
-            if window:
-                longest = min(longest, window + 64)
-            splits = max(1, min(-(-self.decode_blocks_wanted // pairs), -(-longest // 256)))
-            per_split = -(-(-(-longest // splits)) // 64) * 64
-            ctx.plans[key] = (splits, per_split)
-        return ctx.plans[key]
+    def _decode_splits(self, ctx, pairs: int, window: int) -> int:
+        """How many blocks share the keys of one decoding (request, head): enough blocks to fill the
+        chip, no split shorter than 256 keys (one 64-key tile for each of a block's waves). A step that
+        is recorded for replay is sized for the longest request the engine allows."""
+        longest = ctx.length_bound if ctx.length_bound is not None else ctx.longest_decode_host
+        if window:
+            longest = min(longest, window + 64)
+        return max(1, min(-(-self.decode_blocks_wanted // pairs), -(-longest // 256)))
 
     # ---------------------------------------------------------------- output end
 

@@ -35,7 +35,15 @@ class CacheNeed:
 
 
 class Part:
-    """Base of all parts. `ops` is the kernel backend, `dtype` the compute dtype."""
+    """Base of all parts. `ops` is the kernel backend, `dtype` the compute dtype.
+
+    `recordable` says that a step through this part may be recorded once and replayed: everything it
+    does is a launch on the current stream whose sizes depend on the number of tokens and requests
+    only, and it reads nothing of the step on the host. Parts that loop over requests in Python, or
+    index tensors with host values of the step, leave it False; a model with such a part is never
+    recorded."""
+
+    recordable = False
 
     def param_decls(self, prefix: str) -> List[ParamDecl]:
         return []

@@ -8,6 +8,8 @@ class PreNormBlock(Block):
     (reference: opt/model.py:351-375). The sums are made in float32 by the
     last matrix product of each part."""
 
+    recordable = True
+
     def forward(self, stream: Stream, ctx, cache) -> Stream:
         _, h = self.mixer_norm.forward(stream.x, False, True)
         x = self.mixer.forward(h, ctx, cache, stream.x)
@@ -20,6 +22,8 @@ class PreNormBlock(Block):
 class PostNormBlock(Block):
     """`x = norm(x + mixer(x))`, `x = norm(x + feed_forward(x))`: the norm follows
     each sum, and its output is the stream."""
+
+    recordable = True
 
     reads_compute_copy = True      # the mixer reads the stream itself, in the compute dtype
 

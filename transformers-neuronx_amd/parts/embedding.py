@@ -12,6 +12,8 @@ class TokenEmbedding(Part):
     opt/model.py:162-166; the projection is read by no reference code path,
     opt/config.py:34)."""
 
+    recordable = True
+
     def __init__(self, vocab: int, embed_width: int, width: int, position: PartSpec,
                  table_name: str, projection_name: Optional[str], position_name: str):
         self.vocab, self.embed_width, self.width = vocab, embed_width, width
@@ -46,6 +48,8 @@ class VocabHead(Part):
     which is the token table when the checkpoint holds no head of its own
     (reference: layers/transformer.py:196-208, row selection :298-333; tie
     opt/model.py:204-205). Logits are float32."""
+
+    recordable = True
 
     def __init__(self, vocab: int, embed_width: int, width: int, norm: Optional[PartSpec],
                  weight_name: str, tied_to: Optional[str], projection_name: Optional[str], norm_name: str):

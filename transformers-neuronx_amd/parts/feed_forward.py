@@ -10,6 +10,8 @@ class DenseFeedForward(FeedForward):
     """`act(h W1^T + b1) W2^T + b2`, the activation applied to the float32
     accumulator (reference: hlo.py:550-559; activations.py:20-48)."""
 
+    recordable = True
+
     def __init__(self, width: int, inner: int, activation: str, bias: bool = True,
                  up_name: str = "fc1", down_name: str = "fc2"):
         self.width, self.inner, self.activation, self.has_bias = width, inner, activation, bias

@@ -25,6 +25,8 @@ class Attention(Mixer):
     cache another call of the run order writes.
     """
 
+    recordable = True
+
     def __init__(self, width: int, num_heads: int, head_size: int, num_kv_heads: Optional[int] = None,
                  bias: bool = True, window: Optional[int] = None, scale: Optional[float] = None,
                  own_kv: bool = True, names=("q_proj", "k_proj", "v_proj", "out_proj")):

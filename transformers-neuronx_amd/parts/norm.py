@@ -11,6 +11,8 @@ class LayerNorm(Norm):
     rsqrt(var + eps)`, then weight and bias when `affine`
     (reference: hlo.py:84-105, eps of hlo.py:51 passed in as a parameter)."""
 
+    recordable = True
+
     def __init__(self, width: int, eps: float, affine: bool = True):
         self.width, self.eps, self.affine = width, float(eps), affine
         self.weight = self.bias = None

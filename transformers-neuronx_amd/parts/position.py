@@ -11,6 +11,8 @@ class LearnedPositions(PositionEncoding):
     `position + offset` is read (reference: opt/model.py:232-244, where the
     offset is 2, and decoder.py:562-572)."""
 
+    recordable = True
+
     def __init__(self, width: int, max_positions: int, offset: int = 0):
         self.width, self.max_positions, self.offset = width, max_positions, offset
         self.table = None
@@ -30,6 +32,8 @@ class LearnedPositions(PositionEncoding):
 @register_position("none")
 class NoPositions(PositionEncoding):
     """No encoding at the input: the embedded tokens pass as they are."""
+
+    recordable = True
 
     def __init__(self, **_):
         pass
