@@ -51,6 +51,7 @@ def main():
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    ap.add_argument("--prefill-only", action="store_true", help="measure the prompt step alone (for profiles)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -120,6 +121,11 @@ def main():
             times.append(time.perf_counter() - start)
         return min(times[1:])
 
+    if args.prefill_only:
+        sec_p = prefill(PREFILL_TOKENS)
+        print(json.dumps({"prefill_ms": round(sec_p * 1e3, 3), "tokens": PREFILL_TOKENS,
+                          "frac": round(prefill_flops(raw, PREFILL_TOKENS) / sec_p / PEAK_FLOPS[args.dtype], 4)}))
+        return 0
     value, sec, read = decode(args.batch, args.steps, args.warmup)
     print(f"[bench] decode batch {args.batch}: {value:.1f} tok/s, {sec * 1e3:.2f} ms/step", file=sys.stderr, flush=True)
     achieved = read / sec / 1e9

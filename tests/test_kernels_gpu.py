@@ -307,6 +307,10 @@ def test_bfloat16_attention_kernels_agree(case, window):
     many.decode_blocks_wanted = 1 << 20           # as many splits as the contexts allow
     o_many = many.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)
     torch.testing.assert_close(o_many.float(), o_plain.float(), rtol=2e-2, atol=2e-2)
+    direct = HipOps(torch.bfloat16, DEV)
+    direct.prefill_direct = True                  # the prompt kernel that reads the pages without staging
+    o_direct = direct.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)
+    torch.testing.assert_close(o_direct.float(), o_plain.float(), rtol=2e-2, atol=2e-2)
     one = HipOps(torch.bfloat16, DEV)
     one.decode_blocks_wanted = 1                  # no split at all
     o_one = one.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)

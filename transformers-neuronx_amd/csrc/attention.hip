@@ -361,10 +361,261 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict_
   }
 }
 
+// The same computation with the keys and values of a tile staged through LDS, once for the four waves of a
+// block, and the next tile's global loads in flight while the current one is computed (two LDS buffers, one
+// barrier a tile). Page sizes that are powers of two. K is staged as [key][head_size + 8] and V^T as
+// [head_size][64 + 8] (the padding spreads the rows over the LDS banks).
+template <int NDB>
+__global__ void __launch_bounds__(256)
+attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
+                             const bf16_t* __restrict__ v_pages, const int* __restrict__ run_start,
+                             const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
+                             int page_shift, int num_pages, const int* __restrict__ tile_run,
+                             const int* __restrict__ tile_q0, bf16_t* __restrict__ out, int num_heads, int num_kv,
+                             int head_size, int window) {
+  constexpr int NKS = (NDB + 1) / 2;
+  constexpr int DMAX = 16 * NDB;
+  constexpr int KSTR = DMAX + 8;            // elements per staged key row
+  constexpr int VSTR = 64 + 8;              // elements per staged value row (one head-size element, 64 keys)
+  constexpr int KBUF = 64 * KSTR, VBUF = DMAX * VSTR;
+  constexpr int KCH = (64 * DMAX / 8 + 255) / 256;   // 16-byte chunks a thread stages per tile, keys
+  constexpr int VCH = (DMAX * 8 + 255) / 256;        // and values
+  extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
+  bf16_t* ks_buf = smem;                    // [2][KBUF]
+  bf16_t* vs_buf = smem + 2 * KBUF;         // [2][VBUF]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int run = tile_run[blockIdx.x], h = blockIdx.y;
+  const int kvh = h / (num_heads / num_kv);
+  const int t0 = run_start[run], qlen = run_start[run + 1] - t0, cached = cached_lens[run];
+  const int q0 = tile_q0[blockIdx.x];
+  const int qw0 = q0 + 32 * wave;
+  const bool wave_on = qw0 < qlen;
+  const int nq = num_heads * head_size;
+  const int* tab = table + (size_t)run * table_width;
+  const int total = cached + qlen;
+  const int page_size = 1 << page_shift, pmask = page_size - 1;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int ndb = head_size / 16;
+  const int cpr = head_size / 8;            // chunks per key row
+  const size_t head_stride = (size_t)page_size * head_size;
+
+  bf16x8 qf[2][NKS];
+  int qpos[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int qi = qw0 + 16 * qb + r;
+    qpos[qb] = cached + qi;
+#pragma unroll
+    for (int s = 0; s < NKS; ++s) {
+      const int d0 = 32 * s + 8 * g;
+      qf[qb][s] = (qi < qlen && d0 < head_size) ? *(const bf16x8*)(q + (size_t)(t0 + qi) * nq + h * head_size + d0)
+                                                : zero8;
+    }
+  }
+  // block-wide range of key tiles; each wave computes only the tiles its own queries can see
+  const int blk_last = cached + min(q0 + PREFILL_Q_TILE - 1, qlen - 1);
+  const int blk_lo = window > 0 ? max(0, cached + q0 - window + 1) : 0;
+  const int last_q = cached + min(qw0 + 31, qlen - 1);
+  const int first_q = cached + qw0;
+  const int lo = window > 0 ? max(0, first_q - window + 1) : 0;
+
+  float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
+  f32x4 o[NDB][2];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) o[db][qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  bf16x8 kreg[KCH], vreg[VCH];
+  // Global loads of one tile into registers. Keys beyond the request read the request's last key (a valid
+  // place); they are masked by position below, and their values are zeroed when the tile is staged.
+  auto fetch = [&](int tile0) {
+#pragma unroll
+    for (int j = 0; j < KCH; ++j) {
+      const int c = tid + 256 * j;
+      const int key = min(tile0 + c / cpr, total - 1), dc = c % cpr;
+      const int page = min(max(tab[key >> page_shift], 0), num_pages - 1);
+      kreg[j] = (c < 64 * cpr)
+                    ? *(const bf16x8*)(k_pages + ((size_t)page * num_kv + kvh) * head_stride +
+                                       (size_t)(key & pmask) * head_size + dc * 8)
+                    : zero8;
+    }
+#pragma unroll
+    for (int j = 0; j < VCH; ++j) {
+      const int c = tid + 256 * j;
+      const int d = c >> 3, kc = c & 7;
+      const int key = min(tile0 + 8 * kc, (total - 1) & ~7);
+      const int page = min(max(tab[key >> page_shift], 0), num_pages - 1);
+      vreg[j] = (d < head_size) ? *(const bf16x8*)(v_pages + ((size_t)page * num_kv + kvh) * head_stride +
+                                                   (size_t)d * page_size + (key & pmask))
+                                : zero8;
+    }
+  };
+  auto stage = [&](int buf, int tile0) {
+    bf16_t* kd = ks_buf + buf * KBUF;
+    bf16_t* vd = vs_buf + buf * VBUF;
+#pragma unroll
+    for (int j = 0; j < KCH; ++j) {
+      const int c = tid + 256 * j;
+      if (c < 64 * cpr) *(bf16x8*)(kd + (c / cpr) * KSTR + (c % cpr) * 8) = kreg[j];
+    }
+#pragma unroll
+    for (int j = 0; j < VCH; ++j) {
+      const int c = tid + 256 * j;
+      const int d = c >> 3, kc = c & 7;
+      if (d < head_size) {
+        bf16x8 v = vreg[j];
+        if (tile0 + 8 * kc + 8 > total) {     // keys beyond the request: their values must not be NaN
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (tile0 + 8 * kc + e >= total) v[e] = 0;
+        }
+        *(bf16x8*)(vd + d * VSTR + kc * 8) = v;
+      }
+    }
+  };
+
+  int buf = 0;
+  const int tile_begin = (blk_lo / 64) * 64;
+  fetch(tile_begin);
+  for (int tile0 = tile_begin; tile0 <= blk_last; tile0 += 64, buf ^= 1) {
+    stage(buf, tile0);
+    __syncthreads();
+    if (tile0 + 64 <= blk_last) fetch(tile0 + 64);
+    if (!wave_on || tile0 > last_q || tile0 + 63 < lo) continue;
+    const bf16_t* kd = ks_buf + buf * KBUF;
+    const bf16_t* vd = vs_buf + buf * VBUF;
+
+    f32x4 s[4][2];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+      const bf16_t* krow = kd + (16 * kb + r) * KSTR + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        const bf16x8 kf = (32 * ks + 8 * g < head_size) ? *(const bf16x8*)(krow + 32 * ks) : zero8;
+        a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[0][ks], a0, 0, 0, 0);
+        a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[1][ks], a1, 0, 0, 0);
+      }
+      s[kb][0] = a0;
+      s[kb][1] = a1;
+    }
+    const bool full_tile = tile0 + 63 <= first_q && (window <= 0 || tile0 > last_q - window);
+    if (!full_tile) {
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = tile0 + 16 * kb + 4 * g + i;
+            const bool ok = key <= qpos[qb] && (window <= 0 || key > qpos[qb] - window);
+            if (!ok) s[kb][qb][i] = -INFINITY;
+          }
+    }
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s[kb][qb][i]);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m[qb], mx);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = __expf(m[qb] - m_safe);
+      float sum = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float p = __expf(s[kb][qb][i] - m_safe);
+          s[kb][qb][i] = p;
+          sum += p;
+        }
+      sum += __shfl_xor(sum, 16, 64);
+      sum += __shfl_xor(sum, 32, 64);
+      l[qb] = l[qb] * alpha + sum;
+      m[qb] = m_new;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[db][qb][i] *= alpha;
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      bf16x8 pb[2];
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pb[qb][j] = (bf16_t)s[2 * t + (j >> 2)][qb][j & 3];
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) {
+        if (db >= ndb) continue;
+        const bf16_t* vrow = vd + (16 * db + r) * VSTR + 32 * t + 4 * g;
+        const bf16x4 lo4 = *(const bf16x4*)(vrow);
+        const bf16x4 hi4 = *(const bf16x4*)(vrow + 16);
+        bf16x8 vf;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          vf[i] = lo4[i];
+          vf[4 + i] = hi4[i];
+        }
+        o[db][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[0], o[db][0], 0, 0, 0);
+        o[db][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[1], o[db][1], 0, 0, 0);
+      }
+    }
+  }
+  if (!wave_on) return;
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int qi = qw0 + 16 * qb + r;
+    if (qi >= qlen) continue;
+    const float inv = 1.f / l[qb];
+    bf16_t* orow = out + (size_t)(t0 + qi) * nq + h * head_size;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+      if (db >= ndb) continue;
+      bf16x4 v4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v4[i] = (bf16_t)(o[db][qb][i] * inv);
+      *(bf16x4*)(orow + 16 * db + 4 * g) = v4;
+    }
+  }
+}
+
+template <int NDB>
+static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k_pages,
+                              const bf16_t* v_pages, const int* run_start, const int* cached_lens, const int* table,
+                              int table_width, int page_shift, int num_pages, const int* tile_run,
+                              const int* tile_q0, bf16_t* out, int num_heads, int num_kv, int head_size,
+                              int window) {
+  constexpr int DMAX = 16 * NDB;
+  constexpr size_t bytes = 2 * (size_t)(64 * (DMAX + 8) + DMAX * (64 + 8)) * sizeof(bf16_t);
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<NDB>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) {
+      tnx_set_error("attention_prefill: cannot reserve %zu bytes of LDS: %s", bytes, hipGetErrorString(e));
+      return 2;
+    }
+    configured = true;
+  }
+  attention_prefill_lds_kernel<NDB><<<grid, 256, bytes, stream>>>(q, k_pages, v_pages, run_start, cached_lens, table,
+                                                                 table_width, page_shift, num_pages, tile_run,
+                                                                 tile_q0, out, num_heads, num_kv, head_size, window);
+  return 0;
+}
+
 extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const void* v_pages, const int* run_start,
                                      const int* cached_lens, const int* table, int table_width, int page_size,
                                      int num_pages, const int* tile_run, const int* tile_q0, int num_tiles, void* out,
-                                     int num_heads, int num_kv, int head_size, int window, hipStream_t stream) {
+                                     int num_heads, int num_kv, int head_size, int window, int direct,
+                                     hipStream_t stream) {
   TNX_REQUIRE(num_heads > 0 && num_kv > 0 && num_heads % num_kv == 0, "attention_prefill: bad head counts");
   TNX_REQUIRE(head_size % 16 == 0 && head_size >= 16 && head_size <= 256,
               "attention_prefill: head size %d is not a multiple of 16 in [16, 256]", head_size);
@@ -373,6 +624,26 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
   TNX_REQUIRE(num_heads <= 65535, "attention_prefill: too many heads");
   if (num_tiles <= 0) return 0;
   dim3 grid(num_tiles, num_heads);
+  if ((page_size & (page_size - 1)) == 0 && !direct) {
+    int page_shift = 0;
+    while ((1 << page_shift) < page_size) ++page_shift;
+    int rc;
+#define LAUNCH_LDS(NDB)                                                                                          \
+  rc = launch_prefill_lds<NDB>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages,    \
+                               run_start, cached_lens, table, table_width, page_shift, num_pages, tile_run,      \
+                               tile_q0, (bf16_t*)out, num_heads, num_kv, head_size, window)
+    if (head_size <= 64) {
+      LAUNCH_LDS(4);
+    } else if (head_size <= 128) {
+      LAUNCH_LDS(8);
+    } else {
+      LAUNCH_LDS(16);
+    }
+#undef LAUNCH_LDS
+    if (rc) return rc;
+    TNX_CHECK_LAUNCH("attention_prefill_lds");
+    return 0;
+  }
 #define LAUNCH_PREFILL(NDB)                                                                                        \
   attention_prefill_kernel<NDB><<<grid, 256, 0, stream>>>(                                                         \
       (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, table_width, \

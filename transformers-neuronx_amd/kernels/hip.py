@@ -43,7 +43,7 @@ _SIGNATURES = {
                               _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_attention_prefill": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                   _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
-                                  _c_void_p],
+                                  _c_int, _c_void_p],
         "tnx_attention_decode": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                  _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
                                  _c_int, _c_int, _c_void_p, _c_void_p],
@@ -285,7 +285,7 @@ class HipOps:
             self._call("attention", "tnx_attention_prefill", _ptr(q), _ptr(k_pages), _ptr(v_pages),
                        _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(view.block_table), view.width,
                        view.page_size, num_pages, _ptr(ctx.tile_run), _ptr(ctx.tile_start), ctx.tile_run.numel(),
-                       _ptr(out), num_heads, num_kv_heads, head_size, window, _stream())
+                       _ptr(out), num_heads, num_kv_heads, head_size, window, int(self.prefill_direct), _stream())
         n_dec = ctx.decode_runs.numel()
         if n_dec:
             splits = self._decode_splits(ctx, n_dec * num_heads, window)
@@ -300,6 +300,7 @@ class HipOps:
                        _stream())
         return out
 
+    prefill_direct = False            # tests set it to run the prompt kernel that reads pages without LDS staging
     force_plain_attention = False     # tests set it to run the one-wave-per-query kernel in bfloat16 too
     decode_blocks_wanted = 1024       # the keys of decoding requests are split until about this many blocks run
 
