@@ -366,7 +366,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict_
 // barrier a tile). Page sizes that are powers of two. K is staged as [key][head_size + 8] and V^T as
 // [head_size][64 + 8] (the padding spreads the rows over the LDS banks).
 template <int NDB>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, (NDB <= 8 ? 2 : 1))
 attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                              const bf16_t* __restrict__ v_pages, const int* __restrict__ run_start,
                              const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
@@ -431,59 +431,80 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   bf16x8 kreg[KCH], vreg[VCH];
   // Global loads of one tile into registers. Keys beyond the request read the request's last key (a valid
   // place); they are masked by position below, and their values are zeroed when the tile is staged.
+  // No load here depends on a branch (a thread with no chunk of its own reads the last chunk again), and
+  // the page numbers are fetched for all chunks before the first chunk is.
+  const int k_chunks = 64 * cpr, v_chunks = head_size * 8;
+  int kc_key[KCH], kc_dc[KCH], vc_d[VCH], vc_kc[VCH];
+#pragma unroll
+  for (int j = 0; j < KCH; ++j) {
+    const int c = min(tid + 256 * j, k_chunks - 1);
+    kc_key[j] = c / cpr;
+    kc_dc[j] = c - kc_key[j] * cpr;
+  }
+#pragma unroll
+  for (int j = 0; j < VCH; ++j) {
+    const int c = min(tid + 256 * j, v_chunks - 1);
+    vc_d[j] = c >> 3;
+    vc_kc[j] = c & 7;
+  }
+  // Page numbers are looked up one tile earlier than the data they lead to, so that the data loads of the
+  // next tile can be issued without waiting for a lookup.
+  int kpage[KCH], vpage[VCH];
+  auto lookup = [&](int tile0) {
+#pragma unroll
+    for (int j = 0; j < KCH; ++j) kpage[j] = tab[min(tile0 + kc_key[j], total - 1) >> page_shift];
+#pragma unroll
+    for (int j = 0; j < VCH; ++j) vpage[j] = tab[min(tile0 + 8 * vc_kc[j], (total - 1) & ~7) >> page_shift];
+  };
   auto fetch = [&](int tile0) {
 #pragma unroll
     for (int j = 0; j < KCH; ++j) {
-      const int c = tid + 256 * j;
-      const int key = min(tile0 + c / cpr, total - 1), dc = c % cpr;
-      const int page = min(max(tab[key >> page_shift], 0), num_pages - 1);
-      kreg[j] = (c < 64 * cpr)
-                    ? *(const bf16x8*)(k_pages + ((size_t)page * num_kv + kvh) * head_stride +
-                                       (size_t)(key & pmask) * head_size + dc * 8)
-                    : zero8;
+      const int key = min(tile0 + kc_key[j], total - 1);
+      const int page = min(max(kpage[j], 0), num_pages - 1);
+      kreg[j] = *(const bf16x8*)(k_pages + ((size_t)page * num_kv + kvh) * head_stride +
+                                 (size_t)(key & pmask) * head_size + kc_dc[j] * 8);
     }
 #pragma unroll
     for (int j = 0; j < VCH; ++j) {
-      const int c = tid + 256 * j;
-      const int d = c >> 3, kc = c & 7;
-      const int key = min(tile0 + 8 * kc, (total - 1) & ~7);
-      const int page = min(max(tab[key >> page_shift], 0), num_pages - 1);
-      vreg[j] = (d < head_size) ? *(const bf16x8*)(v_pages + ((size_t)page * num_kv + kvh) * head_stride +
-                                                   (size_t)d * page_size + (key & pmask))
-                                : zero8;
+      const int key = min(tile0 + 8 * vc_kc[j], (total - 1) & ~7);
+      const int page = min(max(vpage[j], 0), num_pages - 1);
+      vreg[j] = *(const bf16x8*)(v_pages + ((size_t)page * num_kv + kvh) * head_stride +
+                                 (size_t)vc_d[j] * page_size + (key & pmask));
     }
   };
   auto stage = [&](int buf, int tile0) {
     bf16_t* kd = ks_buf + buf * KBUF;
     bf16_t* vd = vs_buf + buf * VBUF;
 #pragma unroll
-    for (int j = 0; j < KCH; ++j) {
-      const int c = tid + 256 * j;
-      if (c < 64 * cpr) *(bf16x8*)(kd + (c / cpr) * KSTR + (c % cpr) * 8) = kreg[j];
-    }
+    for (int j = 0; j < KCH; ++j)
+      if (tid + 256 * j < k_chunks) *(bf16x8*)(kd + kc_key[j] * KSTR + kc_dc[j] * 8) = kreg[j];
 #pragma unroll
     for (int j = 0; j < VCH; ++j) {
-      const int c = tid + 256 * j;
-      const int d = c >> 3, kc = c & 7;
-      if (d < head_size) {
+      if (tid + 256 * j < v_chunks) {
         bf16x8 v = vreg[j];
-        if (tile0 + 8 * kc + 8 > total) {     // keys beyond the request: their values must not be NaN
+        const int k0 = tile0 + 8 * vc_kc[j];
+        if (k0 + 8 > total) {                 // keys beyond the request: their values must not be NaN
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if (tile0 + 8 * kc + e >= total) v[e] = 0;
+            if (k0 + e >= total) v[e] = 0;
         }
-        *(bf16x8*)(vd + d * VSTR + kc * 8) = v;
+        *(bf16x8*)(vd + vc_d[j] * VSTR + vc_kc[j] * 8) = v;
       }
     }
   };
 
   int buf = 0;
   const int tile_begin = (blk_lo / 64) * 64;
+  lookup(tile_begin);
   fetch(tile_begin);
+  lookup(tile_begin + 64);          // past the request the lookups repeat its last page: harmless
   for (int tile0 = tile_begin; tile0 <= blk_last; tile0 += 64, buf ^= 1) {
     stage(buf, tile0);
     __syncthreads();
-    if (tile0 + 64 <= blk_last) fetch(tile0 + 64);
+    if (tile0 + 64 <= blk_last) {
+      fetch(tile0 + 64);
+      lookup(tile0 + 128);
+    }
     if (!wave_on || tile0 > last_q || tile0 + 63 < lo) continue;
     const bf16_t* kd = ks_buf + buf * KBUF;
     const bf16_t* vd = vs_buf + buf * VBUF;
