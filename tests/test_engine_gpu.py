@@ -218,3 +218,17 @@ def test_recorded_decode_steps_equal_open_ones(tiny_folders, tiny_folders_bf16, 
         assert torch.equal(open_rows[key], rec_rows[key]), key
         want = expected[rid][p]
         assert float((rec_rows[key] - want).abs().max() / expected[rid].abs().max()) <= TOL[dtype]
+
+
+def test_schedules_with_library_products(tiny_folders_bf16, tmp_path, monkeypatch):
+    """The path long prompts take (vendor library for the plain products, our kernels around them), forced
+    on the tiny model by lowering the row count it starts at."""
+    from transformers_neuronx_amd.kernels.hip import HipOps
+    monkeypatch.setattr(HipOps, "library_rows", 8)
+    folder, cfg, weights = tiny_folders_bf16["A"]
+    requests = _requests(cfg, [17, 100, 128], seed=5)
+    expected = _expected(weights, cfg, requests)
+    for kind, (steps, place) in (("whole", schedules.whole(requests)), ("portions", schedules.portions(requests)),
+                                 ("mixed", schedules.mixed(requests, max_tokens=256, seed=6))):
+        out, _ = _run(folder, "bfloat16", steps, 256, 16, tmp_path, f"lib_{kind}")
+        _compare(out, place, expected, cfg["vocab_size"], "bfloat16")

@@ -73,6 +73,7 @@ GEMM_SHAPES = [(1, 16, 8), (3, 50, 24), (8, 96, 96), (17, 1000, 48), (64, 320, 9
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
 def test_linear(dtype, m, n, k):
     hip, ref = _ops(dtype)
+    hip.library_rows = 0        # our own kernels at every row count (the library path has its own test)
     g = torch.Generator(device=DEV).manual_seed(m * 7 + n * 3 + k)
     x = torch.randn(m, k, device=DEV, generator=g).to(dtype)
     w = (torch.randn(n, k, device=DEV, generator=g) / math.sqrt(k)).to(dtype)
@@ -350,3 +351,26 @@ def test_fused_projection_writes_what_the_two_kernels_write(dtype, heads, kv, hs
     q = hip.qkv_project(h, w[:width].contiguous(), bias[:width].contiguous(), heads, 0, hs, 0.3, ctx, view, None, None)
     q_r = ref.qkv_project(h, w[:width].contiguous(), bias[:width].contiguous(), heads, 0, hs, 0.3, ctx, view, None, None)
     torch.testing.assert_close(q.float(), q_r.float(), **tol)
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 96, 320), (300, 1000, 48), (513, 136, 1024)])
+def test_library_product_and_own_product_agree(m, n, k):
+    """From `library_rows` rows on the plain product goes to the vendor library and our epilogue kernel
+    follows; below it, and always when told so, our own tiled kernel does all of it."""
+    from transformers_neuronx_amd.kernels.hip import HipOps
+    _, ref = _ops(torch.bfloat16)
+    lib, own = HipOps(torch.bfloat16, DEV), HipOps(torch.bfloat16, DEV)
+    own.library_rows = 0
+    g = torch.Generator(device=DEV).manual_seed(m + n)
+    x = torch.randn(m, k, device=DEV, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, device=DEV, generator=g) / math.sqrt(k)).to(torch.bfloat16)
+    bias = torch.randn(n, device=DEV, generator=g)
+    res = torch.randn(m, n, device=DEV, generator=g)
+    for kwargs in (dict(act="relu"), dict(act="gelu"), dict(residual=res, out_f32=True), dict(bias=None)):
+        b = kwargs.pop("bias", bias)
+        want = ref.linear(x, w, b, **kwargs).float()
+        for ops in (lib, own):
+            torch.testing.assert_close(ops.linear(x, w, b, **kwargs).float(), want, rtol=2e-2, atol=2e-2)
+    # the head's float32 output never goes through a bfloat16 product
+    torch.testing.assert_close(lib.linear(x, w, None, out_f32=True), ref.linear(x, w, None, out_f32=True),
+                               rtol=1e-3, atol=1e-3)

@@ -9,6 +9,9 @@
 
 TNX_DEFINE_ERROR_API
 
+// One thread takes 8 consecutive elements of a token's [q | k | v] row: a query chunk goes to the dense
+// query matrix scaled, a key chunk to its page as it is (head-size elements are contiguous there), a value
+// chunk element by element (values lie transposed inside a page).
 template <typename T>
 __global__ void __launch_bounds__(256)
 qkv_write_kernel(const T* __restrict__ qkv, const float* __restrict__ bias, float scale,
@@ -18,29 +21,37 @@ qkv_write_kernel(const T* __restrict__ qkv, const float* __restrict__ bias, floa
   const int t = blockIdx.x;
   const int nq = num_heads * head_size, nk = num_kv * head_size;
   const int total = nq + 2 * nk;
-  int page = -1, off = 0;
-  if (num_kv > 0) {
-    const int pos = positions[t];
-    const int blk = pos / page_size;
-    if (blk < table_width) page = table[token_request[t] * table_width + blk];
-    if (page >= num_pages) page = -1;
-    off = pos % page_size;
+  const int i0 = (blockIdx.y * 256 + threadIdx.x) * 8;
+  if (i0 >= total) return;
+  float v[8];
+  const T* row = qkv + (size_t)t * total + i0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = to_f32(row[j]);
+  if (bias) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] += bias[i0 + j];
   }
-  const T* row = qkv + (size_t)t * total;
-  for (int i = threadIdx.x; i < total; i += 256) {
-    float v = to_f32(row[i]);
-    if (bias) v += bias[i];
-    if (i < nq) {
-      q_out[(size_t)t * nq + i] = from_f32<T>(v * scale);
-    } else if (page >= 0) {
-      if (i < nq + nk) {
-        const int j = i - nq, h = j / head_size, d = j % head_size;
-        k_pages[(((size_t)page * num_kv + h) * page_size + off) * head_size + d] = from_f32<T>(v);
-      } else {
-        const int j = i - nq - nk, h = j / head_size, d = j % head_size;
-        v_pages[(((size_t)page * num_kv + h) * head_size + d) * page_size + off] = from_f32<T>(v);
-      }
-    }
+  if (i0 < nq) {
+    T* dst = q_out + (size_t)t * nq + i0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dst[j] = from_f32<T>(v[j] * scale);
+    return;
+  }
+  const int pos = positions[t];
+  const int blk = pos / page_size, off = pos % page_size;
+  int page = -1;
+  if (blk < table_width) page = table[token_request[t] * table_width + blk];
+  if (page < 0 || page >= num_pages) return;
+  if (i0 < nq + nk) {
+    const int j0 = i0 - nq, h = j0 / head_size, d = j0 % head_size;
+    T* dst = k_pages + (((size_t)page * num_kv + h) * page_size + off) * head_size + d;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dst[j] = from_f32<T>(v[j]);
+  } else {
+    const int j0 = i0 - nq - nk, h = j0 / head_size, d = j0 % head_size;
+    T* dst = v_pages + (((size_t)page * num_kv + h) * head_size + d) * page_size + off;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dst[(size_t)j * page_size] = from_f32<T>(v[j]);
   }
 }
 
@@ -51,12 +62,14 @@ extern "C" int tnx_qkv_write(const void* qkv, int dtype, const float* bias, floa
   TNX_REQUIRE(tokens >= 0 && num_heads > 0 && num_kv >= 0 && head_size > 0, "qkv_write: bad sizes");
   TNX_REQUIRE(page_size > 0 && table_width > 0, "qkv_write: bad page table");
   if (tokens == 0) return 0;
+  TNX_REQUIRE(head_size % 8 == 0, "qkv_write: head size %d is not a multiple of 8", head_size);
+  const dim3 grid(tokens, ((num_heads + 2 * num_kv) * head_size / 8 + 255) / 256);
   if (dtype == TNX_F32)
-    qkv_write_kernel<float><<<tokens, 256, 0, stream>>>((const float*)qkv, bias, scale, positions, token_request,
+    qkv_write_kernel<float><<<grid, 256, 0, stream>>>((const float*)qkv, bias, scale, positions, token_request,
                                                         table, table_width, page_size, num_pages, (float*)q_out,
                                                         (float*)k_pages, (float*)v_pages, num_heads, num_kv, head_size);
   else
-    qkv_write_kernel<bf16_t><<<tokens, 256, 0, stream>>>((const bf16_t*)qkv, bias, scale, positions, token_request,
+    qkv_write_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)qkv, bias, scale, positions, token_request,
                                                          table, table_width, page_size, num_pages, (bf16_t*)q_out,
                                                          (bf16_t*)k_pages, (bf16_t*)v_pages, num_heads, num_kv,
                                                          head_size);

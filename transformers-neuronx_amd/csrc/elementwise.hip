@@ -179,3 +179,54 @@ extern "C" int tnx_layernorm(const float* x, const float* weight, const float* b
   TNX_CHECK_LAUNCH("layernorm");
   return 0;
 }
+
+// What follows a library matrix product: out = act(y + bias) + residual, eight elements a thread.
+// y is bfloat16 [rows, width] (width a multiple of 8), bias and residual float32 and optional, out
+// bfloat16 (may be y itself) or float32 (may be the residual itself).
+__global__ void __launch_bounds__(256)
+epilogue_kernel(const bf16_t* __restrict__ y, const float* __restrict__ bias, int act,
+                const float* residual, void* out, int out_dtype, size_t chunks, int width8) {
+  typedef __attribute__((ext_vector_type(8))) __bf16 b8;
+  typedef __attribute__((ext_vector_type(4))) float f4;
+  const size_t c = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (c >= chunks) return;
+  const int col = (int)(c % width8) * 8;
+  const b8 v = ((const b8*)y)[c];
+  float f[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) f[j] = (float)v[j];
+  if (bias) {
+    const f4 b0 = *(const f4*)(bias + col), b1 = *(const f4*)(bias + col + 4);
+    f[0] += b0.x; f[1] += b0.y; f[2] += b0.z; f[3] += b0.w;
+    f[4] += b1.x; f[5] += b1.y; f[6] += b1.z; f[7] += b1.w;
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) f[j] = apply_act(f[j], act);
+  if (residual) {
+    const f4 r0 = ((const f4*)residual)[2 * c], r1 = ((const f4*)residual)[2 * c + 1];
+    f[0] += r0.x; f[1] += r0.y; f[2] += r0.z; f[3] += r0.w;
+    f[4] += r1.x; f[5] += r1.y; f[6] += r1.z; f[7] += r1.w;
+  }
+  if (out_dtype == TNX_F32) {
+    ((f4*)out)[2 * c] = (f4){f[0], f[1], f[2], f[3]};
+    ((f4*)out)[2 * c + 1] = (f4){f[4], f[5], f[6], f[7]};
+  } else {
+    b8 o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = (bf16_t)f[j];
+    ((b8*)out)[c] = o;
+  }
+}
+
+extern "C" int tnx_epilogue(const void* y, const float* bias, int act, const float* residual, void* out,
+                            int out_dtype, int rows, int width, hipStream_t stream) {
+  TNX_REQUIRE(rows >= 0 && width > 0 && width % 8 == 0, "epilogue: width %d is not a multiple of 8", width);
+  if (rows == 0) return 0;
+  const size_t chunks = (size_t)rows * (width / 8);
+  const size_t blocks = (chunks + 255) / 256;
+  TNX_REQUIRE(blocks < (1ull << 31), "epilogue: too many elements");
+  epilogue_kernel<<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)y, bias, act, residual, out, out_dtype, chunks,
+                                                        width / 8);
+  TNX_CHECK_LAUNCH("epilogue");
+  return 0;
+}

@@ -148,14 +148,29 @@ gemm_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, con
 
   bf16x8 rx[2], rw[2];
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  // No load depends on a branch: rows beyond M or N read the last row, a step beyond K reads the last
+  // whole chunk of the row, and what must count as zero is zeroed after the load.
+  const bf16_t* xsrc[2];
+  const bf16_t* wsrc[2];
+  int kofs[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int c = tid + 256 * j;
+    const int row = c >> 2;
+    kofs[j] = (c & 3) * 8;
+    xsrc[j] = x + (size_t)min(m0 + row, M - 1) * K;
+    wsrc[j] = w + (size_t)min(n0 + row, N - 1) * K;
+  }
   auto fetch = [&](int k0) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int c = tid + 256 * j;
-      const int row = c >> 2, k = k0 + (c & 3) * 8;
+      const int k = k0 + kofs[j];
       const bool k_ok = k + 8 <= K;
-      rx[j] = (k_ok && m0 + row < M) ? *(const bf16x8*)(x + (size_t)(m0 + row) * K + k) : zero;
-      rw[j] = (k_ok && n0 + row < N) ? *(const bf16x8*)(w + (size_t)(n0 + row) * K + k) : zero;
+      const int kc = k_ok ? k : K - 8;
+      const bf16x8 xv = *(const bf16x8*)(xsrc[j] + kc);
+      const bf16x8 wv = *(const bf16x8*)(wsrc[j] + kc);
+      rx[j] = k_ok ? xv : zero;
+      rw[j] = k_ok ? wv : zero;
     }
   };
   fetch(0);

@@ -24,6 +24,7 @@ _SIGNATURES = {
         "tnx_add_positions": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
                               _c_int, _c_int, _c_int, _c_void_p],
         "tnx_cast": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_void_p],
+        "tnx_epilogue": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_layernorm": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
                           _c_void_p],
     },
@@ -197,6 +198,16 @@ class HipOps:
         if residual is not None:
             _want(residual, "residual", torch.float32, (m, n))
         out_dtype = torch.float32 if out_f32 else self.dtype
+        if (self._library_product(m, n, k, w, force_tiled) and (residual is not None or not out_f32)):
+            # Many rows: the plain product goes to the vendor library (hipBLASLt through torch.mm), and one
+            # kernel of ours does what follows it. The float32 head keeps our kernel: its output is not
+            # rounded to bfloat16 on the way.
+            y = torch.mm(self.cast(x, torch.bfloat16), w.t())
+            out = torch.empty(m, n, dtype=out_dtype, device=x.device) if out_f32 else y
+            if bias is not None or residual is not None or (act not in (None, "none")) or out_f32:
+                self._call("elementwise", "tnx_epilogue", _ptr(y), _ptr(bias), _ACT[act], _ptr(residual), _ptr(out),
+                           _code(out_dtype), m, n, _stream())
+            return out
         out = torch.empty(m, n, dtype=out_dtype, device=x.device)
         if w.dtype == torch.float32:
             xa = self.cast(x, torch.float32)
@@ -207,6 +218,12 @@ class HipOps:
             self._call("gemm", "tnx_gemm_bf16", _ptr(xa), _ptr(w), _ptr(bias), _ptr(residual), _ptr(out),
                        _code(out_dtype), _ACT[act], m, n, k, int(force_tiled), _stream())
         return out
+
+    library_rows = 256     # from this many rows on, plain bfloat16 products go to the vendor library; 0: never
+
+    def _library_product(self, m, n, k, w, force_tiled) -> bool:
+        return (self.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and self.library_rows > 0
+                and m >= self.library_rows and not force_tiled and n % 8 == 0 and k % 8 == 0)
 
     # ---------------------------------------------------------------- attention
 
@@ -226,7 +243,8 @@ class HipOps:
                     force_tiled=0):
         """Queries, keys and values of the step's tokens: one matrix product whose epilogue scales the
         queries and stores keys and values in their pages (bfloat16), or product and `qkv_write` apart."""
-        if self.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        if (self.dtype != torch.bfloat16 or w.dtype != torch.bfloat16
+                or self._library_product(ctx.num_tokens, w.shape[0], w.shape[1], w, force_tiled)):
             return self.qkv_write(self.linear(h, w, None), bias, num_heads, num_kv_write, head_size, scale, ctx,
                                   view, k_pages, v_pages)
         t = ctx.num_tokens
