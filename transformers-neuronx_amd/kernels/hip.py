@@ -219,7 +219,9 @@ class HipOps:
                        _code(out_dtype), _ACT[act], m, n, k, int(force_tiled), _stream())
         return out
 
-    library_rows = 256     # from this many rows on, plain bfloat16 products go to the vendor library; 0: never
+    # From this many rows on, plain bfloat16 products go to the vendor library (0: never). Up to 16 rows our
+    # own kernel streams the weight as fast as the library does and fuses what follows the product.
+    library_rows = 17
 
     def _library_product(self, m, n, k, w, force_tiled) -> bool:
         return (self.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and self.library_rows > 0
