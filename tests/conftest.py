@@ -37,7 +37,15 @@ TINY_B = dict(
     max_position_embeddings=256, word_embed_proj_dim=48, do_layer_norm_before=False,
     activation_function="gelu", enable_bias=False, layer_norm_elementwise_affine=False,
     layer_norm_eps=3e-4, init_std=0.05)
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1)}
+# A third one whose sizes reach the paths that need them: head size 64, widths that are multiples of 128
+# (the tile-ordered weight copies of the few-rows product), a vocabulary that is a multiple of 16.
+TINY_C = dict(
+    architectures=["OPTForCausalLM"], model_type="opt",
+    vocab_size=640, hidden_size=128, num_hidden_layers=2, num_attention_heads=2, ffn_dim=256,
+    max_position_embeddings=192, word_embed_proj_dim=128, do_layer_norm_before=True,
+    activation_function="gelu_new", enable_bias=True, layer_norm_elementwise_affine=True,
+    layer_norm_eps=1e-6, init_std=0.04)
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
 
 
 @pytest.fixture(scope="session")

@@ -57,7 +57,7 @@ def _compare(out, place, expected, vocab, dtype):
     return worst
 
 
-CASES = [("A", [5, 17, 31, 100, 128]), ("B", [1, 9, 40, 77, 120, 256])]
+CASES = [("A", [5, 17, 31, 100, 128]), ("B", [1, 9, 40, 77, 120, 256]), ("C", [3, 64, 65, 150, 192])]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

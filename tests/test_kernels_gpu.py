@@ -374,3 +374,53 @@ def test_library_product_and_own_product_agree(m, n, k):
     # the head's float32 output never goes through a bfloat16 product
     torch.testing.assert_close(lib.linear(x, w, None, out_f32=True), ref.linear(x, w, None, out_f32=True),
                                rtol=1e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 64, 128), (8, 4096, 512), (16, 320, 256), (13, 48, 1024), (64, 128, 384)])
+def test_product_from_the_tile_ordered_copy(m, n, k):
+    """The few-rows kernel reading the copy of the weight that is laid out tile after tile."""
+    from transformers_neuronx_amd.kernels.hip import HipOps, tile_order
+    hip, ref = _ops(torch.bfloat16)
+    hip.library_rows = 0
+    g = torch.Generator(device=DEV).manual_seed(m * 31 + n + k)
+    x = torch.randn(m, k, device=DEV, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, device=DEV, generator=g) / math.sqrt(k)).to(torch.bfloat16)
+    bias = torch.randn(n, device=DEV, generator=g)
+    res = torch.randn(m, n, device=DEV, generator=g)
+    pw = hip.prepare_weight(w)
+    assert pw.tiles is not None and pw.tiles.numel() == w.numel()
+    # the copy holds element (n, k) at [n/16][k/128][(k%128)/32][n%16][(k%32)/8][k%8]
+    t = tile_order(w)
+    for nn, kk in ((0, 0), (17, 5), (n - 1, k - 1), (31, 127 % k)):
+        assert t[nn // 16, kk // 128, (kk % 128) // 32, nn % 16, (kk % 32) // 8, kk % 8] == w[nn, kk]
+    for act in (None, "relu", "gelu_new"):
+        torch.testing.assert_close(hip.linear(x, pw, bias, act=act).float(), ref.linear(x, w, bias, act=act).float(),
+                                   rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(hip.linear(x, pw, None, residual=res, out_f32=True),
+                               ref.linear(x, w, None, residual=res, out_f32=True), rtol=1e-3, atol=1e-3)
+    # bit for bit what the same kernel makes of the plain layout: only the addresses differ
+    assert torch.equal(hip.linear(x, pw, bias, out_f32=True), hip.linear(x, w, bias, out_f32=True))
+    assert hip.prepare_weight(w[:, :k - 8].contiguous()).tiles is None       # sizes that have no such copy
+
+
+def test_fused_projection_from_the_tile_ordered_copy():
+    hip, ref = _ops(torch.bfloat16)
+    heads, kv, hs, ps = 4, 2, 32, 16
+    runs, cached = [1, 1, 3], [40, 0, 7]
+    num_pages = 8
+    ctx = _make_step(runs, cached, ps, num_pages, seed=2)
+    view = ctx.groups["full"]
+    width, total = 128, (heads + 2 * kv) * hs
+    g = torch.Generator(device=DEV).manual_seed(4)
+    h = torch.randn(ctx.num_tokens, width, device=DEV, generator=g).to(torch.bfloat16)
+    w = (torch.randn(total, width, device=DEV, generator=g) / 11).to(torch.bfloat16)
+    bias = torch.randn(total, device=DEV, generator=g) * 0.2
+    kp_r = torch.full((num_pages, kv, ps, hs), float("nan"), device=DEV, dtype=torch.bfloat16)
+    vp_r = torch.full((num_pages, kv, hs, ps), float("nan"), device=DEV, dtype=torch.bfloat16)
+    kp, vp = kp_r.clone(), vp_r.clone()
+    q_r = ref.qkv_project(h, w, bias, heads, kv, hs, 0.25, ctx, view, kp_r, vp_r)
+    q = hip.qkv_project(h, hip.prepare_weight(w), bias, heads, kv, hs, 0.25, ctx, view, kp, vp)
+    torch.testing.assert_close(q.float(), q_r.float(), rtol=2e-2, atol=2e-2)
+    assert torch.equal(torch.isnan(kp), torch.isnan(kp_r)) and torch.equal(torch.isnan(vp), torch.isnan(vp_r))
+    torch.testing.assert_close(torch.nan_to_num(kp.float()), torch.nan_to_num(kp_r.float()), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(torch.nan_to_num(vp.float()), torch.nan_to_num(vp_r.float()), rtol=2e-2, atol=2e-2)

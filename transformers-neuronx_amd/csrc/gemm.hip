@@ -228,7 +228,10 @@ gemm_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, con
 // dropped, so the compiler can keep many loads in flight. What is left of K after the last whole step of
 // 128 (K % 128, a multiple of 8) is done by wave 0 with guarded loads. The partial sums of the waves meet
 // in LDS.
-template <int MT, int WAVES, bool QKV>
+// With SHUF the weight is read from a copy laid out for this kernel: [N/16][K/128][4][16 rows][4][8], that is
+// tile after tile in the order the loads take it, so that a block streams one contiguous run of memory and
+// each load of a wave covers 1 KB of it (N a multiple of 16, K of 128).
+template <int MT, int WAVES, bool QKV, bool SHUF>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
                         const float* __restrict__ residual, void* __restrict__ out, int out_dtype, int act, int M,
@@ -237,7 +240,10 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 16;
-  const bf16_t* wrow = w + (size_t)min(n0 + r, N - 1) * K + 8 * g;
+  // element offset of the load of step s at K offset kc: W_STEP * kc + W_LOAD * s from wrow
+  constexpr int W_STEP = SHUF ? 16 : 1, W_LOAD = SHUF ? 512 : 32;
+  const bf16_t* wrow = SHUF ? w + (size_t)blockIdx.x * 16 * K + (r * 4 + g) * 8
+                            : w + (size_t)min(n0 + r, N - 1) * K + 8 * g;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   f32x4 acc[MT];
 #pragma unroll
@@ -257,7 +263,7 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
     auto fetch_w = [&](int slot, int kc) {
       const int k = min(kc, k_last);
 #pragma unroll
-      for (int s = 0; s < 4; ++s) wf[slot][s] = *(const bf16x8*)(wrow + k + 32 * s);
+      for (int s = 0; s < 4; ++s) wf[slot][s] = *(const bf16x8*)(wrow + (size_t)k * W_STEP + W_LOAD * s);
     };
     auto fetch_x = [&](int slot, int kc) {
       const int k = min(kc, k_last);
@@ -296,7 +302,7 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
     for (int s = 0; s < 4; ++s) {
       const int k = k_full + 32 * s + 8 * g;
       const bool ok = k + 8 <= K;
-      const bf16x8 wv = ok ? *(const bf16x8*)(wrow + k_full + 32 * s) : zero;
+      const bf16x8 wv = ok ? *(const bf16x8*)(wrow + (size_t)k_full * W_STEP + W_LOAD * s) : zero;
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
         const bf16x8 xv = ok ? *(const bf16x8*)(xrow[t] + k_full + 32 * s) : zero;
@@ -326,30 +332,42 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
 }
 
 template <int MT, int WAVES>
-static void launch_skinny(const bf16_t* xp, const bf16_t* wp, const float* bias, const float* residual, void* out,
-                          int out_dtype, int act, int M, int N, int K, const QkvScatter* sc, hipStream_t stream) {
-  if (sc)
-    gemm_bf16_skinny_kernel<MT, WAVES, true><<<(N + 15) / 16, WAVES * 64, 0, stream>>>(
-        xp, wp, bias, residual, out, out_dtype, act, M, N, K, *sc);
+static void launch_skinny(const bf16_t* xp, const bf16_t* wp, const bf16_t* ws, const float* bias,
+                          const float* residual, void* out, int out_dtype, int act, int M, int N, int K,
+                          const QkvScatter* sc, hipStream_t stream) {
+  const dim3 grid((N + 15) / 16), block(WAVES * 64);
+  const QkvScatter none{};
+  if (ws && sc)
+    gemm_bf16_skinny_kernel<MT, WAVES, true, true><<<grid, block, 0, stream>>>(xp, ws, bias, residual, out, out_dtype,
+                                                                            act, M, N, K, *sc);
+  else if (ws)
+    gemm_bf16_skinny_kernel<MT, WAVES, false, true><<<grid, block, 0, stream>>>(xp, ws, bias, residual, out,
+                                                                             out_dtype, act, M, N, K, none);
+  else if (sc)
+    gemm_bf16_skinny_kernel<MT, WAVES, true, false><<<grid, block, 0, stream>>>(xp, wp, bias, residual, out,
+                                                                             out_dtype, act, M, N, K, *sc);
   else
-    gemm_bf16_skinny_kernel<MT, WAVES, false><<<(N + 15) / 16, WAVES * 64, 0, stream>>>(
-        xp, wp, bias, residual, out, out_dtype, act, M, N, K, QkvScatter{});
+    gemm_bf16_skinny_kernel<MT, WAVES, false, false><<<grid, block, 0, stream>>>(xp, wp, bias, residual, out,
+                                                                              out_dtype, act, M, N, K, none);
 }
 
-static int gemm_bf16_dispatch(const void* x, const void* w, const float* bias, const float* residual, void* out,
-                              int out_dtype, int act, int M, int N, int K, int force_tiled, const QkvScatter* sc,
-                              hipStream_t stream) {
+static int gemm_bf16_dispatch(const void* x, const void* w, const void* w_tiles, const float* bias,
+                              const float* residual, void* out, int out_dtype, int act, int M, int N, int K,
+                              int force_tiled, const QkvScatter* sc, hipStream_t stream) {
   TNX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   TNX_REQUIRE(K % 8 == 0, "gemm_bf16: the inner size K=%d must be a multiple of 8", K);
   TNX_REQUIRE(((uintptr_t)x | (uintptr_t)w) % 16 == 0, "gemm_bf16: operands must be 16-byte aligned");
   if (M == 0) return 0;
   const bf16_t* xp = (const bf16_t*)x;
   const bf16_t* wp = (const bf16_t*)w;
+  const bf16_t* ws = (const bf16_t*)w_tiles;
+  TNX_REQUIRE(ws == nullptr || (N % 16 == 0 && K % 128 == 0),
+              "gemm_bf16: a tile-ordered weight needs N a multiple of 16 and K of 128, got N=%d K=%d", N, K);
   if (M <= 64 && force_tiled != 1) {
     // Eight waves a block when the sum over K is long and the rows are few (more bytes in flight for each
     // of the few blocks), four otherwise. force_tiled 4 or 8 picks the count, for measurements.
     const int waves = force_tiled == 4 || force_tiled == 8 ? force_tiled : (K >= 8192 && N <= 8192 ? 8 : 4);
-#define SKINNY(MT, WV) launch_skinny<MT, WV>(xp, wp, bias, residual, out, out_dtype, act, M, N, K, sc, stream)
+#define SKINNY(MT, WV) launch_skinny<MT, WV>(xp, wp, ws, bias, residual, out, out_dtype, act, M, N, K, sc, stream)
 #define SKINNY_MT(WV)                     \
   switch ((M + 15) / 16) {                \
     case 1: SKINNY(1, WV); break;         \
@@ -378,14 +396,18 @@ static int gemm_bf16_dispatch(const void* x, const void* w, const float* bias, c
   return 0;
 }
 
-extern "C" int tnx_gemm_bf16(const void* x, const void* w, const float* bias, const float* residual, void* out,
-                             int out_dtype, int act, int M, int N, int K, int force_tiled, hipStream_t stream) {
-  return gemm_bf16_dispatch(x, w, bias, residual, out, out_dtype, act, M, N, K, force_tiled, nullptr, stream);
+// `w_tiles` (optional) is the tile-ordered copy of `w` that the few-rows kernel streams faster.
+extern "C" int tnx_gemm_bf16(const void* x, const void* w, const void* w_tiles, const float* bias,
+                             const float* residual, void* out, int out_dtype, int act, int M, int N, int K,
+                             int force_tiled, hipStream_t stream) {
+  return gemm_bf16_dispatch(x, w, w_tiles, bias, residual, out, out_dtype, act, M, N, K, force_tiled, nullptr,
+                            stream);
 }
 
 // The fused projection of queries, keys and values: `x w^T + bias` with w = [Wq; Wk; Wv] stacked by rows,
 // queries scaled and written densely, keys and values written straight into their cache pages.
-extern "C" int tnx_gemm_bf16_qkv(const void* x, const void* w, const float* bias, int M, int K, const int* token_page,
+extern "C" int tnx_gemm_bf16_qkv(const void* x, const void* w, const void* w_tiles, const float* bias, int M, int K,
+                                 const int* token_page,
                                  const int* token_off, void* q_out, void* k_pages, void* v_pages, float scale,
                                  int num_heads, int num_kv, int head_size, int page_size, int num_pages,
                                  int force_tiled, hipStream_t stream) {
@@ -404,5 +426,6 @@ extern "C" int tnx_gemm_bf16_qkv(const void* x, const void* w, const float* bias
   sc.page_size = page_size;
   sc.num_pages = num_pages;
   const int N = sc.nq + 2 * sc.nk;
-  return gemm_bf16_dispatch(x, w, bias, nullptr, nullptr, TNX_BF16, TNX_ACT_NONE, M, N, K, force_tiled, &sc, stream);
+  return gemm_bf16_dispatch(x, w, w_tiles, bias, nullptr, nullptr, TNX_BF16, TNX_ACT_NONE, M, N, K, force_tiled, &sc,
+                            stream);
 }

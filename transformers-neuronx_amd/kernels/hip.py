@@ -31,11 +31,11 @@ _SIGNATURES = {
     "gemm": {
         "tnx_gemm_f32": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                          _c_int, _c_void_p],
-        "tnx_gemm_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
-                          _c_int, _c_int, _c_void_p],
-        "tnx_gemm_bf16_qkv": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p,
-                              _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                              _c_void_p],
+        "tnx_gemm_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+                          _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_gemm_bf16_qkv": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
+                              _c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int,
+                              _c_int, _c_void_p],
     },
     "attention": {
         "tnx_qkv_write": [_c_void_p, _c_int, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
@@ -56,6 +56,32 @@ _SIGNATURES = {
                        _c_void_p],
     },
 }
+
+
+class PreparedWeight:
+    """A `[out, in]` matrix as the kernels want it: the tensor itself, and beside it (bfloat16, `out` a
+    multiple of 16, `in` of 128) a copy in the order the few-rows kernel streams it,
+    `[out/16][in/128][4][16][4][8]`: each block then reads one contiguous run of memory. The copy doubles
+    the memory of the matrices; it is what decoding reads, the plain tensor is what prompts read."""
+
+    __slots__ = ("tensor", "tiles")
+
+    def __init__(self, tensor: torch.Tensor, tiles: Optional[torch.Tensor]):
+        self.tensor, self.tiles = tensor, tiles
+
+    @property
+    def shape(self):
+        return self.tensor.shape
+
+    @property
+    def dtype(self):
+        return self.tensor.dtype
+
+
+def tile_order(w: torch.Tensor) -> torch.Tensor:
+    """`w[n, k]` -> `[n/16][k/128][s][r][g][e]` with n = 16*nt + r and k = 128*kt + 32*s + 8*g + e."""
+    n, k = w.shape
+    return w.view(n // 16, 16, k // 128, 4, 4, 8).permute(0, 2, 3, 1, 4, 5).contiguous()
 
 
 def library(module: str) -> ctypes.CDLL:
@@ -184,7 +210,20 @@ class HipOps:
 
     # ---------------------------------------------------------------- matrix products
 
+    decode_copies = True    # keep a tile-ordered copy of every matrix for the few-rows kernel
+
+    def prepare_weight(self, w: torch.Tensor) -> PreparedWeight:
+        """Called once per matrix when a part receives its tensors."""
+        tiles = None
+        if (self.decode_copies and self.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 2
+                and w.shape[0] % 16 == 0 and w.shape[1] % 128 == 0):
+            tiles = tile_order(w)
+        return PreparedWeight(w, tiles)
+
     def linear(self, x, w, bias=None, act=None, residual=None, out_f32=False, force_tiled=False):
+        tiles = None
+        if isinstance(w, PreparedWeight):
+            w, tiles = w.tensor, w.tiles
         _want(x, "x")
         _want(w, "w")
         if act not in _ACT:
@@ -215,8 +254,8 @@ class HipOps:
                        _code(out_dtype), _ACT[act], m, n, k, _stream())
         else:
             xa = self.cast(x, torch.bfloat16)
-            self._call("gemm", "tnx_gemm_bf16", _ptr(xa), _ptr(w), _ptr(bias), _ptr(residual), _ptr(out),
-                       _code(out_dtype), _ACT[act], m, n, k, int(force_tiled), _stream())
+            self._call("gemm", "tnx_gemm_bf16", _ptr(xa), _ptr(w), _ptr(tiles), _ptr(bias), _ptr(residual),
+                       _ptr(out), _code(out_dtype), _ACT[act], m, n, k, int(force_tiled), _stream())
         return out
 
     # From this many rows on, plain bfloat16 products go to the vendor library (0: never). Up to 16 rows our
@@ -245,6 +284,9 @@ class HipOps:
                     force_tiled=0):
         """Queries, keys and values of the step's tokens: one matrix product whose epilogue scales the
         queries and stores keys and values in their pages (bfloat16), or product and `qkv_write` apart."""
+        tiles = None
+        if isinstance(w, PreparedWeight):
+            w, tiles = w.tensor, w.tiles
         if (self.dtype != torch.bfloat16 or w.dtype != torch.bfloat16
                 or self._library_product(ctx.num_tokens, w.shape[0], w.shape[1], w, force_tiled)):
             return self.qkv_write(self.linear(h, w, None), bias, num_heads, num_kv_write, head_size, scale, ctx,
@@ -261,7 +303,7 @@ class HipOps:
         _want(view.token_page, "token pages", torch.int32, (t,))
         _want(view.token_offset, "token offsets", torch.int32, (t,))
         q = torch.empty(t, num_heads * head_size, dtype=self.dtype, device=h.device)
-        self._call("gemm", "tnx_gemm_bf16_qkv", _ptr(h), _ptr(w), _ptr(bias), t, h.shape[1],
+        self._call("gemm", "tnx_gemm_bf16_qkv", _ptr(h), _ptr(w), _ptr(tiles), _ptr(bias), t, h.shape[1],
                    _ptr(view.token_page), _ptr(view.token_offset), _ptr(q),
                    _ptr(k_pages) if num_kv_write else None, _ptr(v_pages) if num_kv_write else None, float(scale),
                    num_heads, num_kv_write, head_size, view.page_size, num_pages, int(force_tiled), _stream())

@@ -59,6 +59,10 @@ class ReferenceOps:
 
     # ---------------------------------------------------------------- matrix products
 
+    def prepare_weight(self, w):
+        """Matrices are used as they are here."""
+        return w
+
     @staticmethod
     def activation(y, act):
         if act is None or act == "none":

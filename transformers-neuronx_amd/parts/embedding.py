@@ -30,7 +30,7 @@ class TokenEmbedding(Part):
     def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
         super().load(tensors, prefix, ops, dtype)
         self.table = tensors[self.table_name]
-        self.projection = tensors[self.projection_name] if self.projects else None
+        self.projection = ops.prepare_weight(tensors[self.projection_name]) if self.projects else None
         self.position.load(tensors, self.position_name, ops, dtype)
 
     def forward(self, ctx, want_compute: bool) -> Stream:
@@ -69,8 +69,8 @@ class VocabHead(Part):
 
     def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
         super().load(tensors, prefix, ops, dtype)
-        self.weight = tensors[self.weight_name]
-        self.projection = tensors[self.projection_name] if self.projects else None
+        self.weight = ops.prepare_weight(tensors[self.weight_name])
+        self.projection = ops.prepare_weight(tensors[self.projection_name]) if self.projects else None
         if self.norm is not None:
             self.norm.load(tensors, self.norm_name, ops, dtype)
 

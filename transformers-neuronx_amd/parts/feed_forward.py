@@ -27,8 +27,8 @@ class DenseFeedForward(FeedForward):
 
     def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
         super().load(tensors, prefix, ops, dtype)
-        self.w1 = tensors[f"{prefix}{self.up_name}.weight"]
-        self.w2 = tensors[f"{prefix}{self.down_name}.weight"]
+        self.w1 = ops.prepare_weight(tensors[f"{prefix}{self.up_name}.weight"])
+        self.w2 = ops.prepare_weight(tensors[f"{prefix}{self.down_name}.weight"])
         self.b1 = tensors.get(f"{prefix}{self.up_name}.bias") if self.has_bias else None
         self.b2 = tensors.get(f"{prefix}{self.down_name}.bias") if self.has_bias else None
 

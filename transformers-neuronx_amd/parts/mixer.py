@@ -64,10 +64,10 @@ class Attention(Mixer):
         ins = [qn] + ([kn, vn] if self.own_kv else [])
         # One fused projection: a plain concatenation of the rows (the reference's
         # fused form interleaves per tensor-parallel shard, utils.py:189-242).
-        self.w_qkv = torch.cat([tensors[f"{prefix}{n}.weight"] for n in ins], dim=0).contiguous()
+        self.w_qkv = ops.prepare_weight(torch.cat([tensors[f"{prefix}{n}.weight"] for n in ins], dim=0).contiguous())
         self.b_qkv = (torch.cat([tensors[f"{prefix}{n}.bias"] for n in ins], dim=0).contiguous()
                       if self.has_bias else None)
-        self.w_out = tensors[f"{prefix}{on}.weight"]
+        self.w_out = ops.prepare_weight(tensors[f"{prefix}{on}.weight"])
         self.b_out = tensors[f"{prefix}{on}.bias"] if self.has_bias else None
 
     def forward(self, h, ctx, cache, residual):
