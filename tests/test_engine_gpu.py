@@ -232,3 +232,52 @@ def test_schedules_with_library_products(tiny_folders_bf16, tmp_path, monkeypatc
                                  ("mixed", schedules.mixed(requests, max_tokens=256, seed=6))):
         out, _ = _run(folder, "bfloat16", steps, 256, 16, tmp_path, f"lib_{kind}")
         _compare(out, place, expected, cfg["vocab_size"], "bfloat16")
+
+
+def test_bfloat16_against_float32_at_full_layer_sizes():
+    """Two layers of the sizes of OPT-6.7B (width 4096, 32 heads of 128, inner width 16384, vocabulary
+    50272): the bfloat16 engine against the float32 engine on the same (bfloat16-stored) random weights,
+    under a schedule that takes a long prompt in portions, decodes beside another prompt, and ends with
+    recorded decode steps. The reference's own yardstick for such a pair is `allclose(atol=1.0,
+    rtol=1e-3)` with equal argmax (generation_demo.py:437-443); here the bound is the bfloat16 one of the
+    other tests."""
+    from transformers_neuronx_amd.config import EngineConfig, OPTConfig
+    from transformers_neuronx_amd.engine import DecoderModel, StepEntry
+    from transformers_neuronx_amd.engine.factory import build_runner
+    from transformers_neuronx_amd.opt.spec import opt_spec
+    from transformers_neuronx_amd.weights import TensorDict, random_tensors
+    raw = dict(vocab_size=50272, hidden_size=4096, num_hidden_layers=2, num_attention_heads=32, ffn_dim=16384,
+               max_position_embeddings=2048, init_std=0.02)
+    cfg = OPTConfig.from_dict(raw)
+    spec = opt_spec(cfg)
+    tensors = random_tensors(DecoderModel(spec).param_decls(), spec.init_std, 3, torch.bfloat16, DEV)
+    g = torch.Generator().manual_seed(0)
+    long = torch.randint(3, cfg.vocab_size, (700,), generator=g).tolist()
+    short = torch.randint(3, cfg.vocab_size, (40,), generator=g).tolist()
+
+    def run(dtype):
+        ecfg = EngineConfig(dtype=dtype, page_size=64, max_tokens=1024, max_num_seqs=4)
+        runner = build_runner(cfg, TensorDict(tensors), ecfg)
+        rows = []
+
+        def step(parts):
+            entries, n = [], 0
+            for rid, toks, want in parts:
+                entries.append(StepEntry(rid, toks, want))
+                n += len(want)
+            rows.append(runner.step(entries).float().cpu())
+        step([("a", long[:300], [299])])
+        step([("a", long[300:650], [0, 349])])
+        step([("a", long[650:651], [0]), ("b", short[:30], [29])])        # one token beside a portion
+        for i in range(651, 660):
+            step([("a", long[i:i + 1], [0]), ("b", short[i - 621:i - 620], [0])])   # recorded decode steps
+        return torch.cat(rows)
+
+    low, high = run("bfloat16"), run("float32")
+    scale = float(high.abs().max())
+    err = float((low - high).abs().max()) / scale
+    assert err <= TOL["bfloat16"], err
+    # where float32 has a clear winner bfloat16 names the same token
+    top2 = high.topk(2, dim=-1).values
+    clear = (top2[:, 0] - top2[:, 1]) > 4 * TOL["bfloat16"] * scale
+    assert bool((low.argmax(-1) == high.argmax(-1))[clear].all())
