@@ -364,7 +364,7 @@ class HipOps:
 
     prefill_direct = False            # tests set it to run the prompt kernel that reads pages without LDS staging
     force_plain_attention = False     # tests set it to run the one-wave-per-query kernel in bfloat16 too
-    decode_blocks_wanted = 1024       # the keys of decoding requests are split until about this many blocks run
+    decode_blocks_wanted = 512        # the keys of decoding requests are split until about this many blocks run
 
     def _decode_splits(self, ctx, pairs: int, window: int) -> int:
         """How many blocks share the keys of one decoding (request, head): enough blocks to fill the
