@@ -65,7 +65,7 @@ class LLMEngine:
         t0 = time.perf_counter() if self.record_timings else 0.0
         entries = []
         for run in runs:
-            toks = run.request.tokens[run.start:run.start + run.count]
+            toks = run.request.span(run.start, run.count)
             entries.append(StepEntry(run.request.req_id, toks, [run.count - 1] if run.samples else []))
         logits = self.runner.step(entries)
         sampling = [r for r in runs if r.samples]

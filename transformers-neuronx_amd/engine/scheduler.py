@@ -27,7 +27,7 @@ from ..cache.pages import OutOfPages
 from ..sampling.params import SamplingParams
 
 
-@dataclass
+@dataclass(eq=False)      # a request is itself: lists of requests are searched by identity
 class Request:
     req_id: Hashable
     prompt: List[int]
@@ -47,13 +47,22 @@ class Request:
     def num_tokens(self) -> int:
         return len(self.prompt) + len(self.output)
 
+    def span(self, start: int, count: int) -> List[int]:
+        """Tokens start .. start + count - 1 of prompt and output taken as one sequence."""
+        n = len(self.prompt)
+        if start >= n:
+            return self.output[start - n:start - n + count]
+        if start + count <= n:
+            return self.prompt[start:start + count]
+        return self.prompt[start:] + self.output[:start + count - n]
+
     @property
     def decoding(self) -> bool:
         """All tokens but the newest are stored: the next step brings that one token."""
         return len(self.output) > 0 and self.num_computed == self.num_tokens - 1
 
 
-@dataclass
+@dataclass(eq=False)
 class ScheduledRun:
     request: Request
     start: int                      # first position of the portion
@@ -145,12 +154,14 @@ class Scheduler:
 
     def schedule(self) -> List[ScheduledRun]:
         budget = self.max_num_batched_tokens
+        before_all = self.num_preemptions     # a request can have left `running` only if something was put back
         planned: List[ScheduledRun] = []
         blocked = False                       # pages ran out: admit nothing new this step
         # 1. one token for every decoding request, oldest first
         hold = self.prompts_first and (bool(self.waiting) or any(not r.decoding for r in self.running))
         for req in list(self.running):
-            if hold or req not in self.running or not req.decoding or budget <= 0:
+            if hold or (self.num_preemptions != before_all and req not in self.running) or not req.decoding \
+                    or budget <= 0:
                 continue
             before = self.num_preemptions
             if self._reserve(req, req.num_computed + 1, planned):
@@ -158,10 +169,11 @@ class Scheduler:
                 budget -= 1
             blocked |= self.num_preemptions != before
         # 2. the next portion of every prompt under way
+        planned_ids = {id(p.request) for p in planned}
         for req in list(self.running):
-            if req not in self.running or req.decoding or budget <= 0:
+            if (self.num_preemptions != before_all and req not in self.running) or req.decoding or budget <= 0:
                 continue
-            if any(p.request is req for p in planned):
+            if id(req) in planned_ids:
                 continue
             count = min(req.num_tokens - req.num_computed, self.max_portion, budget)
             before = self.num_preemptions
@@ -188,7 +200,8 @@ class Scheduler:
             planned.append(ScheduledRun(req, req.num_computed, count))
             budget -= count
         # a request put back after it was planned is no longer in `running`
-        return [p for p in planned if p.request in self.running]
+        live = {id(r) for r in self.running}
+        return [p for p in planned if id(p.request) in live]
 
     # ---------------------------------------------------------------- after the step
 
