@@ -224,9 +224,17 @@ def test_attention_finds_a_far_key():
     q = (direction * 10).repeat(heads).reshape(1, heads * hs).to(dtype)
     out = hip.attention(q, heads, heads, hs, ctx, view, kp, vp, None)
     torch.testing.assert_close(out.float(), torch.full_like(out, 5.0).float(), rtol=1e-2, atol=1e-2)
-    # with a window that ends before the far key it is not seen
+    # the window's edge: a query at position `cached` with window w sees keys > cached - w. With
+    # w = cached - far the far key is the first one outside, with one more it is the last one inside.
     out_w = hip.attention(q, heads, heads, hs, ctx, view, kp, vp, cached - far)
     assert out_w.float().abs().max() < 1.0
+    out_in = hip.attention(q, heads, heads, hs, ctx, view, kp, vp, cached - far + 1)
+    torch.testing.assert_close(out_in.float(), torch.full_like(out_in, 5.0).float(), rtol=1e-2, atol=1e-2)
+    plain = type(hip)(dtype, DEV)
+    plain.force_plain_attention = True
+    assert plain.attention(q, heads, heads, hs, ctx, view, kp, vp, cached - far).float().abs().max() < 1.0
+    torch.testing.assert_close(plain.attention(q, heads, heads, hs, ctx, view, kp, vp, cached - far + 1).float(),
+                               torch.full_like(out_in, 5.0).float(), rtol=1e-2, atol=1e-2)
 
 
 def test_attention_refuses_bad_head_size():

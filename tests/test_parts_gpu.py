@@ -159,3 +159,72 @@ def test_a_page_edge_shows(tmp_path):
         qq = ops.qkv_write(torch.cat([q, kq[:, :2 * hs]], 1), None, heads, 1, hs, 1.0, ctx, ctx.groups["full"], kp, vp)
         out = ops.attention(qq, heads, 1, hs, ctx, ctx.groups["full"], kp, vp, None)
         assert abs(float(out[0, 0]) - best) < 1e-3, (target, float(out[0, 0]), best)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("order", ["pre_norm", "post_norm"])
+def test_block_arrangements(dtype, order):
+    """A whole layer through the block part, one request in one step, against the plain block."""
+    from transformers_neuronx_amd.cache.manager import LayerCache
+    from transformers_neuronx_amd.engine.batch import StepEntry, build_context
+    from transformers_neuronx_amd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, PartSpec, Stream)
+    width, heads, hs, inner, n, ps = 64, 2, 32, 160, 23, 16
+    norm = PartSpec("layer_norm", dict(width=width, eps=2e-5, affine=True))
+    mixer = MIXERS.build(PartSpec("attention", dict(width=width, num_heads=heads, head_size=hs)))
+    ffn = FEED_FORWARDS.build(PartSpec("dense", dict(width=width, inner=inner, activation="relu")))
+    n1, n2 = NORMS.build(norm), NORMS.build(norm)
+    block = BLOCKS.build(PartSpec(order), mixer, ffn, n1, n2)
+    named = [(mixer, "model.decoder.layers.0.self_attn."), (ffn, "model.decoder.layers.0."),
+             (n1, "model.decoder.layers.0.self_attn_layer_norm"), (n2, "model.decoder.layers.0.final_layer_norm")]
+    g = torch.Generator(device=DEV).manual_seed(6)
+    t = {}
+    for part, prefix in named:
+        for d in part.param_decls(prefix):
+            v = torch.randn(*d.shape, device=DEV, generator=g) * (0.1 if d.role == "matrix" else 0.3)
+            if d.init == "around_one":
+                v = v + 1
+            t[d.name] = v.to(dtype) if d.role == "matrix" else v
+    ops = _ops(dtype)
+    for part, prefix in named:
+        part.load(t, prefix, ops, dtype)
+    cache = LayerCache(0, "full", True, torch.zeros(3, heads, ps, hs, device=DEV, dtype=dtype),
+                       torch.zeros(3, heads, hs, ps, device=DEV, dtype=dtype))
+    ctx = build_context([StepEntry("a", [0] * n, [])], [0], [0], {"full": np.array([[2, 0]], dtype=np.int32)}, ps, DEV)
+    x = torch.randn(n, width, device=DEV, generator=g)
+    out = block.forward(Stream(x, ops.cast(x, dtype)), ctx, cache)
+    cfg = dict(num_attention_heads=heads, activation_function="relu", do_layer_norm_before=order == "pre_norm",
+               layer_norm_eps=2e-5)
+    want = plain_opt.block(x.cpu(), {k: v.float().cpu() for k, v in t.items()}, cfg, 0)
+    torch.testing.assert_close(out.x.cpu(), want, **_tol(dtype))
+    if order == "post_norm":
+        assert out.compute is not None and out.compute.dtype == dtype
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("projects,normed", [(False, True), (True, False)])
+def test_head_part(dtype, projects, normed):
+    from transformers_neuronx_amd.parts import HEADS, PartSpec, Stream
+    width, embed, vocab = 64, (40 if projects else 64), 333
+    head = HEADS.build(PartSpec("vocab_projection", dict(
+        vocab=vocab, embed_width=embed, width=width,
+        norm=PartSpec("layer_norm", dict(width=width, eps=1e-5, affine=True)) if normed else None,
+        weight_name="lm_head.weight", tied_to="tok", projection_name="proj", norm_name="fn")))
+    decls = {d.name: d for d in head.param_decls()}
+    assert decls["lm_head.weight"].tied_to == "tok" and ("proj" in decls) == projects and ("fn.weight" in decls) == normed
+    g = torch.Generator(device=DEV).manual_seed(8)
+    t = {"lm_head.weight": (torch.randn(vocab, embed, device=DEV, generator=g) / 8).to(dtype),
+         "proj": (torch.randn(embed, width, device=DEV, generator=g) / 8).to(dtype),
+         "fn.weight": torch.randn(width, device=DEV, generator=g) + 1, "fn.bias": torch.randn(width, device=DEV, generator=g)}
+    head.load(t, "", _ops(dtype), dtype)
+    ctx = _ctx([6, 1], [0, 9], 16, 3)
+    ctx.logits_rows = torch.tensor([5, 2, 6], dtype=torch.int32, device=DEV)
+    x = torch.randn(7, width, device=DEV, generator=g)
+    logits = head.forward(Stream(x, None), ctx)
+    rows = x[[5, 2, 6]]
+    if normed:
+        rows = plain_opt.layer_norm(rows, t["fn.weight"], t["fn.bias"], 1e-5)
+    if projects:
+        rows = rows @ t["proj"].float().t()
+    want = rows @ t["lm_head.weight"].float().t()
+    assert logits.dtype == torch.float32 and logits.shape == (3, vocab)
+    torch.testing.assert_close(logits, want, **_tol(dtype))

@@ -177,11 +177,6 @@ class OPTForSampling:
             params.append(p)
         engine.reset()
         ids = [engine.add_request(toks, p) for toks, p in zip(rows, params)]
-        emitted = {i: 0 for i in ids}
-
-        def on_token(out):
-            emitted[out.req_id] += 1
-
         while engine.has_work:
             outs = engine.step()
             if streamer is not None and outs:
