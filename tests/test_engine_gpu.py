@@ -281,3 +281,47 @@ def test_bfloat16_against_float32_at_full_layer_sizes():
     top2 = high.topk(2, dim=-1).values
     clear = (top2[:, 0] - top2[:, 1]) > 4 * TOL["bfloat16"] * scale
     assert bool((low.argmax(-1) == high.argmax(-1))[clear].all())
+
+
+def _odd(v, heads, hs, layers, ffn, proj, pre, act, bias, affine, eps):
+    return dict(architectures=["OPTForCausalLM"], model_type="opt", vocab_size=v, hidden_size=heads * hs,
+                num_hidden_layers=layers, num_attention_heads=heads, ffn_dim=ffn, max_position_embeddings=200,
+                word_embed_proj_dim=proj or heads * hs, do_layer_norm_before=pre, activation_function=act,
+                enable_bias=bias, layer_norm_elementwise_affine=affine, layer_norm_eps=eps, init_std=0.05)
+
+
+# Sizes at the edges of what the kernels take: every head size class (16 .. 256, also ones only the general
+# attention kernel takes), one head and many, widths and vocabularies that are no multiple of 8, 16 or 128,
+# a feed-forward narrower than a tile, an embedding narrower than the model.
+ODD = [
+    _odd(257, 1, 16, 1, 24, None, True, "relu", True, True, 1e-5),
+    _odd(1001, 5, 48, 2, 200, 56, True, "gelu", True, True, 1e-5),
+    _odd(50, 7, 80, 1, 72, None, False, "relu", False, True, 1e-4),
+    _odd(333, 3, 112, 2, 328, 40, True, "gelu_new", True, False, 1e-5),
+    _odd(1234, 2, 144, 1, 520, None, True, "relu", True, True, 1e-5),
+    _odd(777, 1, 256, 1, 264, 24, False, "gelu", True, True, 1e-5),
+    _odd(130, 9, 32, 2, 8, None, True, "relu", True, True, 1e-5),
+    _odd(4099, 6, 64, 1, 1000, None, True, "relu", True, True, 1e-5),
+    _odd(96, 2, 128, 1, 136, None, True, "relu", True, True, 1e-5),
+    _odd(513, 11, 16, 3, 176, 8, True, "relu", False, False, 1e-3),
+]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("index", range(len(ODD)))
+def test_odd_sizes(tmp_path, dtype, index):
+    from safetensors.torch import load_file
+    from transformers_neuronx_amd.config import OPTConfig
+    from transformers_neuronx_amd.weights import write_random_model
+    raw = ODD[index]
+    folder = str(tmp_path / "model")
+    write_random_model(OPTConfig.from_dict(raw), folder, index, dtype=dtype)
+    weights = load_file(os.path.join(folder, "model.safetensors"))
+    requests = _requests(raw, [3, 70, 129, 200], seed=index)
+    expected = _expected(weights, raw, requests)
+    for kind, (steps, place), max_tokens, page_size in [
+        ("singles", schedules.head_then_singles(requests), 256, 16),
+        ("mixed", schedules.mixed(requests, max_tokens=384, seed=index), 384, 64),
+    ]:
+        out, _ = _run(folder, dtype, steps, max_tokens, page_size, tmp_path, kind)
+        _compare(out, place, expected, raw["vocab_size"], dtype)
