@@ -140,6 +140,9 @@ ATTN_CASES = [
     (5, 1, 80, 64, [3, 129, 1], [64, 0, 200]),
     (2, 2, 128, 64, [1, 1, 65], [511, 63, 64]),
     (1, 1, 256, 16, [20, 1], [0, 33]),
+    # several tiles of one run, starting inside a group of 8 positions and inside a page
+    (2, 2, 64, 16, [300, 1, 9], [5, 40, 7]),
+    (2, 1, 128, 64, [131, 2], [61, 126]),
 ]
 
 

@@ -17,7 +17,8 @@ __global__ void __launch_bounds__(256)
 qkv_write_kernel(const T* __restrict__ qkv, const float* __restrict__ bias, float scale,
                  const int* __restrict__ positions, const int* __restrict__ token_request,
                  const int* __restrict__ table, int table_width, int page_size, int num_pages, T* __restrict__ q_out,
-                 T* __restrict__ k_pages, T* __restrict__ v_pages, int num_heads, int num_kv, int head_size) {
+                 T* __restrict__ k_pages, T* __restrict__ v_pages, int num_heads, int num_kv, int head_size,
+                 const int* __restrict__ run_start, int values_of_single_tokens_only) {
   const int t = blockIdx.x;
   const int nq = num_heads * head_size, nk = num_kv * head_size;
   const int total = nq + 2 * nk;
@@ -48,6 +49,10 @@ qkv_write_kernel(const T* __restrict__ qkv, const float* __restrict__ bias, floa
 #pragma unroll
     for (int j = 0; j < 8; ++j) dst[j] = from_f32<T>(v[j]);
   } else {
+    if (values_of_single_tokens_only) {   // the values of longer runs are written by tiles
+      const int r = token_request[t];
+      if (run_start[r + 1] - run_start[r] > 1) return;
+    }
     const int j0 = i0 - nq - nk, h = j0 / head_size, d = j0 % head_size;
     T* dst = v_pages + (((size_t)page * num_kv + h) * head_size + d) * page_size + off;
 #pragma unroll
@@ -55,25 +60,102 @@ qkv_write_kernel(const T* __restrict__ qkv, const float* __restrict__ bias, floa
   }
 }
 
+// The values of a tile of up to 128 consecutive tokens of one run, one kv head a block. Values lie transposed
+// in a page (consecutive positions are neighbours), so the tile goes through LDS: it is read as rows of the
+// product, 16 bytes a thread, and written 8 consecutive positions (16 bytes) a thread. Groups of 8 are
+// aligned to positions, not to the tile; a group that the tile covers in part is written element by element.
+constexpr int VT_TOKENS = 128, VT_DIMS = 64, VT_ROW = VT_DIMS + 8;
+
+__global__ void __launch_bounds__(256)
+value_tiles_kernel(const bf16_t* __restrict__ qkv, const float* __restrict__ bias, const int* __restrict__ run_start,
+                   const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
+                   int page_size, int num_pages, const int* __restrict__ tile_run,
+                   const int* __restrict__ tile_q0, bf16_t* __restrict__ v_pages, int num_heads, int num_kv,
+                   int head_size) {
+  __shared__ __attribute__((aligned(16))) bf16_t sm[VT_TOKENS * VT_ROW];
+  const int run = tile_run[blockIdx.x], q0 = tile_q0[blockIdx.x], kvh = blockIdx.y;
+  const int t0 = run_start[run] + q0;
+  const int n = min(VT_TOKENS, run_start[run + 1] - t0);
+  const int p0 = cached_lens[run] + q0;   // position of the tile's first token
+  const int total = (num_heads + 2 * num_kv) * head_size;
+  const int col0 = (num_heads + num_kv) * head_size + kvh * head_size;
+  const int* tab = table + (size_t)run * table_width;
+  const int groups = (p0 + n - 1) / 8 - p0 / 8 + 1;
+  for (int dc = 0; dc < head_size; dc += VT_DIMS) {
+    const int dims = min(VT_DIMS, head_size - dc);     // a multiple of 8
+    const int chunks = dims / 8;
+    for (int idx = threadIdx.x; idx < n * chunks; idx += 256) {
+      const int i = idx / chunks, c = idx % chunks;
+      bf16x8 v = *(const bf16x8*)(qkv + (size_t)(t0 + i) * total + col0 + dc + c * 8);
+      if (bias) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = (bf16_t)((float)v[j] + bias[col0 + dc + c * 8 + j]);
+      }
+      *(bf16x8*)(sm + i * VT_ROW + c * 8) = v;
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < groups * dims; idx += 256) {
+      const int g = idx / dims, d = idx % dims;
+      const int pos = (p0 / 8 + g) * 8;               // first position of the group
+      const int blk = pos / page_size;
+      const int page = blk < table_width ? tab[blk] : -1;
+      if (page < 0 || page >= num_pages) continue;
+      bf16_t* dst = v_pages + (((size_t)page * num_kv + kvh) * head_size + dc + d) * page_size + pos % page_size;
+      const int i0 = pos - p0;                         // the group's first token within the tile; may be < 0
+      if (i0 >= 0 && i0 + 8 <= n) {
+        bf16x8 v;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = sm[(i0 + j) * VT_ROW + d];
+        *(bf16x8*)dst = v;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (i0 + j >= 0 && i0 + j < n) dst[j] = sm[(i0 + j) * VT_ROW + d];
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// With `num_tiles > 0` (bfloat16 only) the values of the runs that `tile_run` / `tile_q0` cut into tiles of
+// `tile_tokens` tokens are written by tiles, and the token-wise kernel leaves them out.
 extern "C" int tnx_qkv_write(const void* qkv, int dtype, const float* bias, float scale, const int* positions,
                              const int* token_request, const int* table, int table_width, int page_size,
                              int num_pages, void* q_out, void* k_pages, void* v_pages, int tokens, int num_heads,
-                             int num_kv, int head_size, hipStream_t stream) {
+                             int num_kv, int head_size, const int* run_start, const int* cached_lens,
+                             const int* tile_run, const int* tile_q0, int num_tiles, int tile_tokens,
+                             hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && num_heads > 0 && num_kv >= 0 && head_size > 0, "qkv_write: bad sizes");
   TNX_REQUIRE(page_size > 0 && table_width > 0, "qkv_write: bad page table");
   if (tokens == 0) return 0;
   TNX_REQUIRE(head_size % 8 == 0, "qkv_write: head size %d is not a multiple of 8", head_size);
+  const bool by_tiles = num_tiles > 0 && num_kv > 0;
+  if (by_tiles) {
+    TNX_REQUIRE(dtype == TNX_BF16, "qkv_write: values are written by tiles in bfloat16 only");
+    TNX_REQUIRE(tile_tokens > 0 && tile_tokens <= VT_TOKENS, "qkv_write: tiles of %d tokens, at most %d fit",
+                tile_tokens, VT_TOKENS);
+    TNX_REQUIRE(page_size % 8 == 0, "qkv_write: page size %d is not a multiple of 8", page_size);
+    TNX_REQUIRE(run_start && cached_lens && tile_run && tile_q0, "qkv_write: tiles without their tables");
+    TNX_REQUIRE(num_kv <= 65535, "qkv_write: too many heads");
+  }
   const dim3 grid(tokens, ((num_heads + 2 * num_kv) * head_size / 8 + 255) / 256);
   if (dtype == TNX_F32)
     qkv_write_kernel<float><<<grid, 256, 0, stream>>>((const float*)qkv, bias, scale, positions, token_request,
                                                         table, table_width, page_size, num_pages, (float*)q_out,
-                                                        (float*)k_pages, (float*)v_pages, num_heads, num_kv, head_size);
+                                                        (float*)k_pages, (float*)v_pages, num_heads, num_kv, head_size,
+                                                        run_start, 0);
   else
     qkv_write_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)qkv, bias, scale, positions, token_request,
                                                          table, table_width, page_size, num_pages, (bf16_t*)q_out,
                                                          (bf16_t*)k_pages, (bf16_t*)v_pages, num_heads, num_kv,
-                                                         head_size);
+                                                         head_size, run_start, by_tiles ? 1 : 0);
   TNX_CHECK_LAUNCH("qkv_write");
+  if (by_tiles) {
+    value_tiles_kernel<<<dim3(num_tiles, num_kv), 256, 0, stream>>>(
+        (const bf16_t*)qkv, bias, run_start, cached_lens, table, table_width, page_size, num_pages, tile_run, tile_q0,
+        (bf16_t*)v_pages, num_heads, num_kv, head_size);
+    TNX_CHECK_LAUNCH("value_tiles");
+  }
   return 0;
 }
 
@@ -190,9 +272,6 @@ extern "C" int tnx_attention_any(const void* q, int dtype, const void* k_pages, 
 
 // ------------------------------------------------------------------------------------------ bfloat16, prompts
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 #define PREFILL_Q_TILE 128  // queries per block: four waves of 32
 

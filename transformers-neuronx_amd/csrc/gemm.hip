@@ -7,9 +7,6 @@
 
 TNX_DEFINE_ERROR_API
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 __device__ __forceinline__ void epilogue_store(float v, int m, int n, int N, const float* bias, const float* residual,
                                                void* out, int out_dtype, int act) {

@@ -49,6 +49,7 @@ class StepContext:
     decode_runs: torch.Tensor = None     # int32, the runs of one token (each attends with one query)
     tile_run: torch.Tensor = None        # int32, for every tile of QUERY_TILE queries of the longer runs: its run
     tile_start: torch.Tensor = None      # int32, and its first query within the run
+    query_tile: int = QUERY_TILE         # queries of a tile
     longest_decode: torch.Tensor = None  # int32 [1], the most keys a one-token run of this step reads
     longest_decode_host: int = 0
     # When a step is recorded for replay, nothing in its launches may depend on the lengths of this

@@ -39,7 +39,8 @@ _SIGNATURES = {
     },
     "attention": {
         "tnx_qkv_write": [_c_void_p, _c_int, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
-                          _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                          _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p,
+                          _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
         "tnx_attention_any": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                               _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_attention_prefill": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
@@ -140,6 +141,7 @@ class HipOps:
         if self.device.type != "cuda" or not torch.cuda.is_available():
             raise RuntimeError("the HIP kernels need a GPU; none is visible to torch")
         _code(dtype)
+        self._bias_copies = {}
 
     def _call(self, module: str, fn: str, *args):
         lib = library(module)
@@ -238,10 +240,19 @@ class HipOps:
             _want(residual, "residual", torch.float32, (m, n))
         out_dtype = torch.float32 if out_f32 else self.dtype
         if (self._library_product(m, n, k, w, force_tiled) and (residual is not None or not out_f32)):
-            # Many rows: the plain product goes to the vendor library (hipBLASLt through torch.mm), and one
-            # kernel of ours does what follows it. The float32 head keeps our kernel: its output is not
-            # rounded to bfloat16 on the way.
-            y = torch.mm(self.cast(x, torch.bfloat16), w.t())
+            # Many rows: the plain product goes to the vendor library (hipBLASLt through torch), and one
+            # kernel of ours does what follows it. Where the result stays bfloat16 the library adds the bias
+            # (and applies ReLU) before it rounds; with a residual, bias and sum are ours, in float32. The
+            # float32 head keeps our kernel: its output is not rounded to bfloat16 on the way.
+            xa = self.cast(x, torch.bfloat16)
+            if bias is not None and residual is None and not out_f32:
+                b16 = self._bias_bf16(bias)
+                if act == "relu":
+                    return torch._addmm_activation(b16, xa, w.t(), use_gelu=False)
+                y = torch.addmm(b16, xa, w.t())
+                bias = None
+            else:
+                y = torch.mm(xa, w.t())
             out = torch.empty(m, n, dtype=out_dtype, device=x.device) if out_f32 else y
             if bias is not None or residual is not None or (act not in (None, "none")) or out_f32:
                 self._call("elementwise", "tnx_epilogue", _ptr(y), _ptr(bias), _ACT[act], _ptr(residual), _ptr(out),
@@ -261,6 +272,15 @@ class HipOps:
     # From this many rows on, plain bfloat16 products go to the vendor library (0: never). Up to 16 rows our
     # own kernel streams the weight as fast as the library does and fuses what follows the product.
     library_rows = 17
+
+    def _bias_bf16(self, bias):
+        """The bfloat16 copy of a float32 bias that the library's epilogue takes, made once. The original
+        is held with it, so that its address names no other tensor while the copy is kept."""
+        kept = self._bias_copies.get(bias.data_ptr())
+        if kept is None or kept[0] is not bias:
+            kept = (bias, bias.to(torch.bfloat16))
+            self._bias_copies[bias.data_ptr()] = kept
+        return kept[1]
 
     def _library_product(self, m, n, k, w, force_tiled) -> bool:
         return (self.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and self.library_rows > 0
@@ -320,10 +340,15 @@ class HipOps:
             num_pages = self._check_pages(k_pages, v_pages, num_kv_write, head_size, view.page_size)
         _want(view.block_table, "block table", torch.int32, (ctx.num_requests, view.width))
         q = torch.empty(t, num_heads * head_size, dtype=self.dtype, device=qkv.device)
+        # the values of runs of several tokens are written by tiles (transposed through LDS)
+        by_tiles = (self.dtype == torch.bfloat16 and self.value_tiles and num_kv_write
+                    and ctx.tile_run is not None and ctx.tile_run.numel() > 0)
         self._call("attention", "tnx_qkv_write", _ptr(qkv), _code(self.dtype), _ptr(bias), float(scale),
                    _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width, view.page_size,
                    num_pages, _ptr(q), _ptr(k_pages) if num_kv_write else None,
-                   _ptr(v_pages) if num_kv_write else None, t, num_heads, num_kv_write, head_size, _stream())
+                   _ptr(v_pages) if num_kv_write else None, t, num_heads, num_kv_write, head_size,
+                   _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(ctx.tile_run), _ptr(ctx.tile_start),
+                   ctx.tile_run.numel() if by_tiles else 0, ctx.query_tile, _stream())
         return q
 
     def attention(self, q, num_heads, num_kv_heads, head_size, ctx, view, k_pages, v_pages, window=None):
@@ -362,6 +387,7 @@ class HipOps:
                        _stream())
         return out
 
+    value_tiles = True                # tests clear it to write every value token by token
     prefill_direct = False            # tests set it to run the prompt kernel that reads pages without LDS staging
     force_plain_attention = False     # tests set it to run the one-wave-per-query kernel in bfloat16 too
     decode_blocks_wanted = 512        # the keys of decoding requests are split until about this many blocks run
