@@ -293,10 +293,11 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict_
   constexpr int NKS = (NDB + 1) / 2;  // MFMA steps of 32 over the head size
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int run = tile_run[blockIdx.x], h = blockIdx.y;
+  const int tile = blockIdx.x / num_heads, h = blockIdx.x % num_heads;
+  const int run = tile_run[tile];
   const int kvh = h / (num_heads / num_kv);
   const int t0 = run_start[run], qlen = run_start[run + 1] - t0, cached = cached_lens[run];
-  const int qw0 = tile_q0[blockIdx.x] + 32 * wave;
+  const int qw0 = tile_q0[tile] + 32 * wave;
   if (qw0 >= qlen) return;
   const int nq = num_heads * head_size;
   const int* tab = table + (size_t)run * table_width;
@@ -478,10 +479,11 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int run = tile_run[blockIdx.x], h = blockIdx.y;
+  const int tile = blockIdx.x / num_heads, h = blockIdx.x % num_heads;
+  const int run = tile_run[tile];
   const int kvh = h / (num_heads / num_kv);
   const int t0 = run_start[run], qlen = run_start[run + 1] - t0, cached = cached_lens[run];
-  const int q0 = tile_q0[blockIdx.x];
+  const int q0 = tile_q0[tile];
   const int qw0 = q0 + 32 * wave;
   const bool wave_on = qw0 < qlen;
   const int nq = num_heads * head_size;
@@ -734,9 +736,11 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
               "attention_prefill: head size %d is not a multiple of 16 in [16, 256]", head_size);
   TNX_REQUIRE(page_size % 16 == 0 && page_size > 0, "attention_prefill: page size %d is not a multiple of 16",
               page_size);
-  TNX_REQUIRE(num_heads <= 65535, "attention_prefill: too many heads");
   if (num_tiles <= 0) return 0;
-  dim3 grid(num_tiles, num_heads);
+  TNX_REQUIRE((long long)num_tiles * num_heads < (1ll << 31), "attention_prefill: too many tiles");
+  // Blocks are numbered with the head running fastest: the tiles come ordered by falling work, so the blocks
+  // that run longest start first and the short ones fill in behind them.
+  dim3 grid((unsigned)num_tiles * num_heads);
   if ((page_size & (page_size - 1)) == 0 && !direct) {
     int page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;

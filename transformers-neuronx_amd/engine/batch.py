@@ -115,11 +115,15 @@ def pack_step(entries: List[StepEntry], cached: List[int], slots: List[int], tab
     single = run_lens == 1
     decode_runs = np.nonzero(single)[0].astype(np.int32)
     longest = int((cached_np[single] + 1).max()) if single.any() else 0
-    tile_run, tile_start = [], []
+    # Tiles of the longer runs, those that see the most keys first: a kernel that takes them in this order
+    # starts its longest blocks first.
+    tiles = []
     for i in np.nonzero(run_lens > 1)[0]:
         for q0 in range(0, int(run_lens[i]), QUERY_TILE):
-            tile_run.append(i)
-            tile_start.append(q0)
+            tiles.append((-(int(cached_np[i]) + min(q0 + QUERY_TILE, int(run_lens[i]))), int(i), q0))
+    tiles.sort()
+    tile_run = [t[1] for t in tiles]
+    tile_start = [t[2] for t in tiles]
     pieces = [token_ids, positions, token_request, run_start, cached_np, np.array(slots, dtype=np.int32), rows,
               decode_runs, np.array(tile_run, dtype=np.int32), np.array(tile_start, dtype=np.int32),
               np.array([longest], dtype=np.int32)]
