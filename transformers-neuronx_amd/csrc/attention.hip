@@ -274,6 +274,7 @@ extern "C" int tnx_attention_any(const void* q, int dtype, const void* k_pages, 
 
 
 #define PREFILL_Q_TILE 128  // queries per block: four waves of 32
+#define LOG2E 1.4426950408889634f
 
 // Flash-style attention of a run of queries over its request's pages, on MFMA 16x16x32.
 // A wave owns 32 queries (two column blocks of 16) and walks the keys 64 at a time. It computes the
@@ -458,7 +459,10 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict_
 // block, and the next tile's global loads in flight while the current one is computed (two LDS buffers, one
 // barrier a tile). Page sizes that are powers of two. K is staged as [key][head_size + 8] and V^T as
 // [head_size][64 + 8] (the padding spreads the rows over the LDS banks).
-template <int NDB>
+// FAST is the case of a head size of exactly 16 * NDB and pages of 64 keys or more: a tile then lies within
+// one page, whose number is one scalar lookup, every thread's place within the tile is fixed, and no part of
+// the inner loops depends on a size known only at run time.
+template <int NDB, bool FAST>
 __global__ void __launch_bounds__(256, (NDB <= 8 ? 2 : 1))
 attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                              const bf16_t* __restrict__ v_pages, const int* __restrict__ run_start,
@@ -491,6 +495,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   const int total = cached + qlen;
   const int page_size = 1 << page_shift, pmask = page_size - 1;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (FAST) head_size = DMAX;
   const int ndb = head_size / 16;
   const int cpr = head_size / 8;            // chunks per key row
   const size_t head_stride = (size_t)page_size * head_size;
@@ -544,13 +549,36 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   // Page numbers are looked up one tile earlier than the data they lead to, so that the data loads of the
   // next tile can be issued without waiting for a lookup.
   int kpage[KCH], vpage[VCH];
+  int tile_page = 0;                        // FAST: the one page of the tile looked up last
+  int koff[KCH], voff[VCH];                 // FAST: a thread's chunks within the tile's part of the page
+#pragma unroll
+  for (int j = 0; j < KCH; ++j) koff[j] = kc_key[j] * head_size + kc_dc[j] * 8;
+#pragma unroll
+  for (int j = 0; j < VCH; ++j) voff[j] = vc_d[j] * page_size + 8 * vc_kc[j];
   auto lookup = [&](int tile0) {
+    if (FAST) {
+      tile_page = tab[min(tile0, total - 1) >> page_shift];
+      return;
+    }
 #pragma unroll
     for (int j = 0; j < KCH; ++j) kpage[j] = tab[min(tile0 + kc_key[j], total - 1) >> page_shift];
 #pragma unroll
     for (int j = 0; j < VCH; ++j) vpage[j] = tab[min(tile0 + 8 * vc_kc[j], (total - 1) & ~7) >> page_shift];
   };
   auto fetch = [&](int tile0) {
+    if (FAST) {
+      // keys of the page beyond the request are read as they lie: their scores are masked by position and
+      // their values are zeroed when the tile is staged
+      const int page = min(max(tile_page, 0), num_pages - 1);
+      const size_t base = ((size_t)page * num_kv + kvh) * head_stride;
+      const bf16_t* kb = k_pages + base + (size_t)(tile0 & pmask) * head_size;
+      const bf16_t* vb = v_pages + base + (tile0 & pmask);
+#pragma unroll
+      for (int j = 0; j < KCH; ++j) kreg[j] = *(const bf16x8*)(kb + koff[j]);
+#pragma unroll
+      for (int j = 0; j < VCH; ++j) vreg[j] = *(const bf16x8*)(vb + voff[j]);
+      return;
+    }
 #pragma unroll
     for (int j = 0; j < KCH; ++j) {
       const int key = min(tile0 + kc_key[j], total - 1);
@@ -641,24 +669,29 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       const float m_new = fmaxf(m[qb], mx);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = __expf(m[qb] - m_safe);
+      // e^(x - m) as 2^(x log2 e - m log2 e): one multiply-add and the hardware's 2^x
+      const float m_log2 = m_safe * LOG2E;
+      const float alpha = __builtin_amdgcn_exp2f((m[qb] - m_safe) * LOG2E);
       float sum = 0.f;
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float p = __expf(s[kb][qb][i] - m_safe);
+          const float p = __builtin_amdgcn_exp2f(fmaf(s[kb][qb][i], LOG2E, -m_log2));
           s[kb][qb][i] = p;
           sum += p;
         }
       sum += __shfl_xor(sum, 16, 64);
       sum += __shfl_xor(sum, 32, 64);
       l[qb] = l[qb] * alpha + sum;
+      // the sums so far are rescaled only if the maximum of some query of the wave moved
+      if (__builtin_amdgcn_ballot_w64(m_new != m[qb]) != 0) {
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[db][qb][i] *= alpha;
+      }
       m[qb] = m_new;
-#pragma unroll
-      for (int db = 0; db < NDB; ++db)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) o[db][qb][i] *= alpha;
     }
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -702,7 +735,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   }
 }
 
-template <int NDB>
+template <int NDB, bool FAST>
 static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k_pages,
                               const bf16_t* v_pages, const int* run_start, const int* cached_lens, const int* table,
                               int table_width, int page_shift, int num_pages, const int* tile_run,
@@ -712,7 +745,7 @@ static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, co
   constexpr size_t bytes = 2 * (size_t)(64 * (DMAX + 8) + DMAX * (64 + 8)) * sizeof(bf16_t);
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<NDB>,
+    hipError_t e = hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<NDB, FAST>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
     if (e != hipSuccess) {
       tnx_set_error("attention_prefill: cannot reserve %zu bytes of LDS: %s", bytes, hipGetErrorString(e));
@@ -720,7 +753,7 @@ static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, co
     }
     configured = true;
   }
-  attention_prefill_lds_kernel<NDB><<<grid, 256, bytes, stream>>>(q, k_pages, v_pages, run_start, cached_lens, table,
+  attention_prefill_lds_kernel<NDB, FAST><<<grid, 256, bytes, stream>>>(q, k_pages, v_pages, run_start, cached_lens, table,
                                                                  table_width, page_shift, num_pages, tile_run,
                                                                  tile_q0, out, num_heads, num_kv, head_size, window);
   return 0;
@@ -746,9 +779,15 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
     while ((1 << page_shift) < page_size) ++page_shift;
     int rc;
 #define LAUNCH_LDS(NDB)                                                                                          \
-  rc = launch_prefill_lds<NDB>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages,    \
-                               run_start, cached_lens, table, table_width, page_shift, num_pages, tile_run,      \
-                               tile_q0, (bf16_t*)out, num_heads, num_kv, head_size, window)
+  rc = (NDB <= 8 && page_size >= 64 && head_size == 16 * NDB)                                                            \
+           ? launch_prefill_lds<NDB, true>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages,               \
+                                           (const bf16_t*)v_pages, run_start, cached_lens, table, table_width,   \
+                                           page_shift, num_pages, tile_run, tile_q0, (bf16_t*)out, num_heads,    \
+                                           num_kv, head_size, window)                                            \
+           : launch_prefill_lds<NDB, false>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages,              \
+                                            (const bf16_t*)v_pages, run_start, cached_lens, table, table_width,  \
+                                            page_shift, num_pages, tile_run, tile_q0, (bf16_t*)out, num_heads,   \
+                                            num_kv, head_size, window)
     if (head_size <= 64) {
       LAUNCH_LDS(4);
     } else if (head_size <= 128) {
