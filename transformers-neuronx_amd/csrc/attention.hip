@@ -818,7 +818,7 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
 // ------------------------------------------------------------------------------------------ bfloat16, decoding
 
 // One query per request over its pages. The keys of a request are split over `num_splits` blocks; a block's
-// four waves take 64-key tiles in turn. A tile of keys of one head is read as it lies in memory, 16 bytes
+// NW waves (four or eight) take 64-key tiles in turn. A tile of keys of one head is read as it lies in memory, 16 bytes
 // a lane: lane l holds chunk l % CPR (8 head-size elements) of key l / CPR of each group of 64 / CPR keys.
 // The partial dot products are summed over the CPR lanes of a key by a butterfly that halves what each lane
 // keeps at every step, so that in the end every lane holds the score of one key of the tile. Values lie
@@ -827,8 +827,8 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
 // No load depends on a branch: keys beyond the request read a valid place and get weight zero.
 // Partial results (maximum, sum, weighted values, all float32) of waves meet in LDS and those of splits in
 // a workspace that a second kernel merges. The page size is a power of two here.
-template <int CPR>
-__global__ void __launch_bounds__(256, (CPR <= 8 ? 4 : (CPR == 16 ? 2 : 1)))
+template <int CPR, int NW>
+__global__ void __launch_bounds__(64 * NW, (CPR <= 8 ? 16 / NW : (CPR == 16 ? 8 / NW : 1)))
 attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                         const bf16_t* __restrict__ v_pages, const int* __restrict__ run_start,
                         const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
@@ -837,9 +837,9 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                         int window, int num_splits, const int* __restrict__ longest_ptr) {
   constexpr int KPI = 64 / CPR;       // keys per load instruction of a wave
   constexpr int DH = CPR * 8;
-  __shared__ float sm_p[4][64];
-  __shared__ float sm_o[4][DH];
-  __shared__ float sm_m[4], sm_l[4];
+  __shared__ float sm_p[NW][64];
+  __shared__ float sm_o[NW][DH];
+  __shared__ float sm_m[NW], sm_l[NW];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int split = blockIdx.x, h = blockIdx.y, dz = blockIdx.z;
   const int kvh = h / (num_heads / num_kv);
@@ -870,7 +870,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
 #pragma unroll
   for (int i = 0; i < CPR; ++i) acc[i] = 0.f;
 
-  for (int tile0 = k_begin + 64 * wave; tile0 < k_end; tile0 += 256) {
+  for (int tile0 = k_begin + 64 * wave; tile0 < k_end; tile0 += 64 * NW) {
     bf16x8 kv[CPR];
 #pragma unroll
     for (int i = 0; i < CPR; ++i) {
@@ -946,12 +946,14 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     sm_l[wave] = l;
   }
   __syncthreads();
-  for (int d = threadIdx.x; d < DH; d += 256) {
-    float mm = fmaxf(fmaxf(sm_m[0], sm_m[1]), fmaxf(sm_m[2], sm_m[3]));
+  for (int d = threadIdx.x; d < DH; d += 64 * NW) {
+    float mm = sm_m[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) mm = fmaxf(mm, sm_m[w]);
     const float ms = mm == -INFINITY ? 0.f : mm;
     float ll = 0.f, oo = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < NW; ++w) {
       const float f = __expf(sm_m[w] - ms);
       ll += sm_l[w] * f;
       oo += sm_o[w][d] * f;
@@ -994,7 +996,7 @@ extern "C" int tnx_attention_decode(const void* q, const void* k_pages, const vo
                                     const int* cached_lens, const int* table, int table_width, int page_size,
                                     int num_pages, const int* decode_runs, int num_decode, void* out, float* part_o,
                                     float* part_ml, int num_heads, int num_kv, int head_size, int window,
-                                    int num_splits, const int* longest, hipStream_t stream) {
+                                    int num_splits, int waves, const int* longest, hipStream_t stream) {
   TNX_REQUIRE(num_heads > 0 && num_kv > 0 && num_heads % num_kv == 0, "attention_decode: bad head counts");
   TNX_REQUIRE(head_size == 16 || head_size == 32 || head_size == 64 || head_size == 128 || head_size == 256,
               "attention_decode: head size %d is not one of 16, 32, 64, 128, 256", head_size);
@@ -1005,21 +1007,30 @@ extern "C" int tnx_attention_decode(const void* q, const void* k_pages, const vo
   TNX_REQUIRE(num_splits >= 1 && longest != nullptr, "attention_decode: bad split count or no length given");
   TNX_REQUIRE(num_splits == 1 || (part_o && part_ml), "attention_decode: splits need a workspace");
   TNX_REQUIRE(num_heads <= 65535 && num_decode <= 65535, "attention_decode: too many heads or requests");
+  TNX_REQUIRE(waves == 4 || (waves == 8 && head_size <= 128),
+              "attention_decode: blocks have 4 waves, or 8 up to head size 128; not %d at head size %d", waves, head_size);
   if (num_decode <= 0) return 0;
   dim3 grid(num_splits, num_heads, num_decode);
+#define LAUNCH_DECODE_ARGS                                                                                          \
+  (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, table_width,     \
+      page_shift, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window, num_splits,     \
+      longest
 #define LAUNCH_DECODE(CPR)                                                                                         \
-  attention_decode_kernel<CPR><<<grid, 256, 0, stream>>>(                                                          \
-      (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, table_width, \
-      page_shift, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window, num_splits,    \
-      longest)
+  if (waves == 8)                                                                                                  \
+    attention_decode_kernel<CPR, 8><<<grid, 512, 0, stream>>>(LAUNCH_DECODE_ARGS);                                 \
+  else                                                                                                             \
+    attention_decode_kernel<CPR, 4><<<grid, 256, 0, stream>>>(LAUNCH_DECODE_ARGS)
   switch (head_size) {
     case 16: LAUNCH_DECODE(2); break;
     case 32: LAUNCH_DECODE(4); break;
     case 64: LAUNCH_DECODE(8); break;
     case 128: LAUNCH_DECODE(16); break;
-    default: LAUNCH_DECODE(32); break;
+    default:
+      attention_decode_kernel<32, 4><<<grid, 256, 0, stream>>>(LAUNCH_DECODE_ARGS);
+      break;
   }
 #undef LAUNCH_DECODE
+#undef LAUNCH_DECODE_ARGS
   TNX_CHECK_LAUNCH("attention_decode");
   if (num_splits > 1) {
     attention_decode_merge_kernel<<<dim3(num_heads, num_decode), head_size < 64 ? 64 : head_size, 0, stream>>>(

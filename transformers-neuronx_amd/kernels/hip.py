@@ -48,7 +48,7 @@ _SIGNATURES = {
                                   _c_int, _c_void_p],
         "tnx_attention_decode": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                  _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
-                                 _c_int, _c_int, _c_void_p, _c_void_p],
+                                 _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
     },
     "sampling": {
         "tnx_ban_tokens": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
@@ -375,7 +375,7 @@ class HipOps:
                        _ptr(out), num_heads, num_kv_heads, head_size, window, int(self.prefill_direct), _stream())
         n_dec = ctx.decode_runs.numel()
         if n_dec:
-            splits = self._decode_splits(ctx, n_dec * num_heads, window)
+            splits, waves = self._decode_splits(ctx, n_dec * num_heads, window, head_size <= 128)
             part_o = part_ml = None
             if splits > 1:
                 part_o = torch.empty(n_dec * num_heads * splits * head_size, dtype=torch.float32, device=q.device)
@@ -383,23 +383,30 @@ class HipOps:
             self._call("attention", "tnx_attention_decode", _ptr(q), _ptr(k_pages), _ptr(v_pages),
                        _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(view.block_table), view.width,
                        view.page_size, num_pages, _ptr(ctx.decode_runs), n_dec, _ptr(out), _ptr(part_o),
-                       _ptr(part_ml), num_heads, num_kv_heads, head_size, window, splits, _ptr(ctx.longest_decode),
+                       _ptr(part_ml), num_heads, num_kv_heads, head_size, window, splits, waves,
+                       _ptr(ctx.longest_decode),
                        _stream())
         return out
 
     value_tiles = True                # tests clear it to write every value token by token
     prefill_direct = False            # tests set it to run the prompt kernel that reads pages without LDS staging
     force_plain_attention = False     # tests set it to run the one-wave-per-query kernel in bfloat16 too
+    decode_wide_blocks = 1            # blocks of eight waves where four-wave blocks would be split
     decode_blocks_wanted = 512        # the keys of decoding requests are split until about this many blocks run
 
-    def _decode_splits(self, ctx, pairs: int, window: int) -> int:
-        """How many blocks share the keys of one decoding (request, head): enough blocks to fill the
-        chip, no split shorter than 256 keys (one 64-key tile for each of a block's waves). A step that
-        is recorded for replay is sized for the longest request the engine allows."""
+    def _decode_splits(self, ctx, pairs: int, window: int, wide_allowed: bool = True):
+        """(splits, waves): how many blocks share the keys of one decoding (request, head), and how many
+        waves a block has. Enough waves to fill the chip, no wave with less than one 64-key tile. Where
+        blocks of four waves would need an even number of splits, blocks of eight waves take half as many:
+        fewer partial results to merge, none at all with one split. A step that is recorded for replay is
+        sized for the longest request the engine allows."""
         longest = ctx.length_bound if ctx.length_bound is not None else ctx.longest_decode_host
         if window:
             longest = min(longest, window + 64)
-        return max(1, min(-(-self.decode_blocks_wanted // pairs), -(-longest // 256)))
+        splits = max(1, min(-(-self.decode_blocks_wanted // pairs), -(-longest // 256)))
+        if self.decode_wide_blocks and wide_allowed and splits >= 2:
+            return -(-splits // 2), 8
+        return splits, 4
 
     # ---------------------------------------------------------------- output end
 
