@@ -35,14 +35,27 @@ __device__ __forceinline__ float philox_uniform(uint64_t seed, uint64_t counter)
   return (float)(c0 >> 8) * (1.0f / 16777216.0f);
 }
 
-__global__ void __launch_bounds__(256)
+// One block of 1,024 threads a row; four logits a load where the rows allow it.
+__global__ void __launch_bounds__(1024)
 argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int vocab) {
-  __shared__ unsigned long long best[4];
+  __shared__ unsigned long long best[16];
   const float* row = logits + (size_t)blockIdx.x * vocab;
   uint64_t b = 0;
-  for (int i = threadIdx.x; i < vocab; i += 256) {
-    const uint64_t k = order_key(row[i], i);
-    b = k > b ? k : b;
+  if ((vocab & 3) == 0) {
+    const f32x4* row4 = (const f32x4*)row;
+    for (int i = threadIdx.x; i < vocab / 4; i += 1024) {
+      const f32x4 v = row4[i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint64_t k = order_key(v[j], 4 * i + j);
+        b = k > b ? k : b;
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < vocab; i += 1024) {
+      const uint64_t k = order_key(row[i], i);
+      b = k > b ? k : b;
+    }
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
@@ -52,7 +65,7 @@ argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int vocab
   if ((threadIdx.x & 63) == 0) best[threadIdx.x >> 6] = b;
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int w = 1; w < 4; ++w) b = best[w] > b ? best[w] : b;
+    for (int w = 1; w < 16; ++w) b = best[w] > b ? best[w] : b;
     out[blockIdx.x] = (int)(~(uint32_t)b);
   }
 }
@@ -60,7 +73,7 @@ argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int vocab
 extern "C" int tnx_argmax(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
   TNX_REQUIRE(rows >= 0 && vocab > 0, "argmax: bad sizes rows=%d vocab=%d", rows, vocab);
   if (rows == 0) return 0;
-  argmax_kernel<<<rows, 256, 0, stream>>>(logits, out, vocab);
+  argmax_kernel<<<rows, 1024, 0, stream>>>(logits, out, vocab);
   TNX_CHECK_LAUNCH("argmax");
   return 0;
 }
