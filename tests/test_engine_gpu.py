@@ -325,3 +325,45 @@ def test_odd_sizes(tmp_path, dtype, index):
     ]:
         out, _ = _run(folder, dtype, steps, max_tokens, page_size, tmp_path, kind)
         _compare(out, place, expected, raw["vocab_size"], dtype)
+
+
+def test_command_line_dump_and_analyze(tiny_folders, tmp_path, capsys):
+    """`opt_demo run --dump_logits` writes the logits each token was chosen from; `analyze` compares two
+    runs by the reference's yardstick (generation_demo.py:404-443) and fails when they differ."""
+    from transformers_neuronx_amd.config import OPTConfig
+    from transformers_neuronx_amd.opt import demo
+    folder, cfg, weights = tiny_folders["A"]
+    prompt = [5, 17, 3, 200, 9]
+    dirs = {}
+    for amp in ("bf16", "f32"):
+        dirs[amp] = str(tmp_path / f"logits_{amp}")
+        demo.main(["--amp", amp, "run", folder, "--batch_size", "2", "--n_positions", "24", "--prompt_ids",
+                   ",".join(map(str, prompt)), "--top_k", "1", "--dump_logits", dirs[amp],
+                   "--dump_logits_limit", "-1"])
+    steps = sorted(os.listdir(dirs["f32"]), key=lambda f: int(f[:-3]))
+    assert len(steps) == 24 - len(prompt)
+    # the dumped float32 logits are the plain implementation's, token by token, along the greedy path
+    # (top_k 1; the reference's loop never picks the end-of-sequence token, sampling.py:143-144)
+    eos = OPTConfig.from_dict(cfg).eos_token_id
+    seq = list(prompt)
+    for i, name in enumerate(steps):
+        got = torch.load(os.path.join(dirs["f32"], name), weights_only=True)
+        assert got.shape == (2, cfg["vocab_size"])
+        ref = plain_opt.forward_logits(weights, cfg, seq)[-1]
+        torch.testing.assert_close(got[0], ref, rtol=1e-4, atol=1e-4)
+        torch.testing.assert_close(got[1], ref, rtol=1e-4, atol=1e-4)
+        ref = ref.clone()
+        ref[eos] = float("-inf")
+        seq.append(int(ref.argmax()))
+    assert demo.main(["analyze", "-d", dirs["bf16"], dirs["f32"]]) == 0
+    # a spoiled dump is found
+    bad = str(tmp_path / "bad")
+    os.makedirs(bad)
+    for name in steps:
+        t = torch.load(os.path.join(dirs["f32"], name), weights_only=True)
+        if name == "3.pt":
+            t = t.clone()
+            t[0, int(t[0].argmin())] = 1e3
+        torch.save(t, os.path.join(bad, name))
+    assert demo.main(["analyze", "-d", bad, dirs["f32"]]) == 1
+    assert "step 3" in capsys.readouterr().out

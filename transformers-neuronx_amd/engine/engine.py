@@ -36,6 +36,8 @@ class LLMEngine:
         self._ids = itertools.count()
         self.timings: List[dict] = []          # one record per step when `record_timings`
         self.record_timings = False
+        # called with (requests that sample in this step, their logits [n, vocab] float32) before the draw
+        self.logits_hook: Optional[Callable] = None
 
     # ---------------------------------------------------------------- requests
 
@@ -71,6 +73,8 @@ class LLMEngine:
         sampling = [r for r in runs if r.samples]
         tokens: List[Optional[int]] = [None] * len(runs)
         if sampling:
+            if self.logits_hook is not None:
+                self.logits_hook([r.request for r in sampling], logits)
             drawn = self.sampler(logits, [r.request.params for r in sampling],
                                  [len(r.request.output) for r in sampling])
             it = iter(drawn)

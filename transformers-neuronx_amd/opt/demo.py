@@ -3,13 +3,15 @@
     opt_demo [--amp f32|bf16] save DIR --random --config CONFIG.json [--seed N]
     opt_demo [--amp f32|bf16] run DIR [--batch_size 4] [--n_positions 128] [--print_latency]
              [--prompt_len N | --prompt_ids 5,6,7] [--top_k 50] [--top_p 1.0] [--temperature 1.0]
-             [--do_sample] [--max_new_tokens N] [--seed N] [--dump_logits DIR] [--benchmark]
+             [--do_sample] [--max_new_tokens N] [--seed N] [--benchmark]
+             [--dump_logits DIR [--dump_logits_limit N]]
+    opt_demo analyze -d DIR [DIR ...] GOLDEN_DIR
 
 Option names and meanings are the reference's where it has them: gpt_demo.py:37-66
 (`--amp`, `save`, `--random`, `--config`, `run`, `--batch_size`, `--n_positions`,
 `--print_latency`) and generation_demo.py:201-280 (`--prompt_len`: random token ids of
 that length, :267, :492-494; `--top_k`, `--top_p`, `--temperature`, `--do_sample`,
-`--max_new_tokens`, `--dump_logits`, `--benchmark`). Without `--do_sample` `run` does what
+`--max_new_tokens`, `--dump_logits`, `--dump_logits_limit`, `--benchmark`; `analyze -d`, :286-290). Without `--do_sample` `run` does what
 the reference's `run` does: `model.sample(input_ids, sequence_length=n_positions)` with
 top_k 50. There is no tokenizer here (no network to fetch one): prompts are token ids.
 """
@@ -34,6 +36,8 @@ def _parser():
                            "random weight")
     save.add_argument("--config", type=str, default="", help="Path to config.json file")
     save.add_argument("--seed", type=int, default=0)
+    ana = sub.add_parser("analyze")
+    ana.add_argument("-d", "--dirs", nargs="+", required=True, help="folders of dumped logits; the last is the golden one")
     run = sub.add_parser("run")
     run.add_argument("load")
     run.add_argument("--batch_size", type=int, default=4, help="Input batch size")
@@ -49,7 +53,9 @@ def _parser():
     run.add_argument("--max_new_tokens", type=int, default=None)
     run.add_argument("--max_length", type=int, default=None)
     run.add_argument("--seed", type=int, default=15213)
-    run.add_argument("--dump_logits", type=str, default=None, help="folder for the logits of every step")
+    run.add_argument("--dump_logits", type=str, default=None,
+                     help="folder for the logits that each generated token was chosen from: <step>.pt, [batch, vocab]")
+    run.add_argument("--dump_logits_limit", type=int, default=1, help="how many steps to dump; -1 for all")
     run.add_argument("--benchmark", action="store_true")
     run.add_argument("--page_size", type=int, default=64)
     return parser
@@ -91,11 +97,16 @@ def run(args):
     gen = None
     if args.do_sample:
         gen = GenerationConfig(do_sample=True, top_k=args.top_k, top_p=args.top_p, temperature=args.temperature)
+    dumped = []
     if args.dump_logits:
+        # generation_demo.py:694-702 writes the scores of the first `dump_logits_limit` generated tokens
         os.makedirs(args.dump_logits, exist_ok=True)
-        logits = model(input_ids)
-        torch.save(logits.cpu(), os.path.join(args.dump_logits, "0.pt"))
-        model.reset()
+
+        def keep(requests, logits):
+            if args.dump_logits_limit < 0 or len(dumped) < args.dump_logits_limit:
+                order = sorted(range(len(requests)), key=lambda i: requests[i].req_id)
+                dumped.append(logits[order].cpu())
+        model.engine.logits_hook = keep
     if args.print_latency or args.benchmark:
         model.engine.record_timings = True
     print("running model.sample")
@@ -104,6 +115,10 @@ def run(args):
                        top_p=args.top_p, seed=args.seed, generation_config=gen)
     elapsed = time.time() - start
     print("generated_sequence=", out)
+    for i, logits in enumerate(dumped):
+        torch.save(logits, os.path.join(args.dump_logits, f"{i}.pt"))
+    if args.dump_logits:
+        print(f"Dumped the logits of {len(dumped)} steps into {args.dump_logits}")
     if args.print_latency:
         for rec in model.engine.timings:
             print(f"Latency: {math.ceil(rec['seconds'] * 1000)} ms ({rec['tokens']} tokens)")
@@ -120,13 +135,41 @@ def run(args):
         print(json.dumps(report))
 
 
+def analyze(args):
+    """Logits dumped by two or more runs against the last one, the golden one, step by step: the
+    reference's yardstick (generation_demo.py:404-443), `allclose(atol=1.0, rtol=1e-3)` and the same
+    greedy token. Returns the number of steps that fail either."""
+    def load(folder):
+        names = sorted((f for f in os.listdir(folder) if f.endswith(".pt")), key=lambda f: int(f[:-3]))
+        return [torch.load(os.path.join(folder, f), weights_only=True) for f in names]
+    golden_dir, golden = args.dirs[-1], load(args.dirs[-1])
+    failures = 0
+    for folder in args.dirs[:-1]:
+        cand = load(folder)
+        print(f"{folder} vs {golden_dir} (golden): {len(cand)} vs {len(golden)} steps")
+        for i, (a, b) in enumerate(zip(cand, golden)):
+            close = torch.allclose(a, b, atol=1.0, rtol=0.001)
+            same = torch.equal(a.argmax(-1), b.argmax(-1))
+            if not close:
+                print(f"  step {i}: logits differ by up to {float((a - b).abs().max()):.4f}")
+            if not same:
+                print(f"  step {i}: greedy tokens differ: {a.argmax(-1).tolist()} vs {b.argmax(-1).tolist()}")
+            failures += (not close) or (not same)
+            if not same:
+                break                      # later steps follow different tokens
+    print("all steps match" if not failures else f"{failures} steps do not match")
+    return failures
+
+
 def main(argv=None):
     args = _parser().parse_args(argv)
     if args.which == "save":
         save(args)
+    elif args.which == "analyze":
+        return 1 if analyze(args) else 0
     else:
         run(args)
 
 
 if __name__ == "__main__":
-    main()
+    sys.exit(main())

@@ -36,7 +36,7 @@ class OPTForSampling:
             raise ValueError(f"tp_degree={tp_degree}: this engine runs on one GPU")
         if amp is None:
             amp = config.torch_dtype
-        else:
+        elif parse_dtype(amp) != parse_dtype(config.torch_dtype):
             warnings.warn(f"torch_dtype={config.torch_dtype} ignored in favor of amp={amp}")
         n_max = max(n_positions) if isinstance(n_positions, (list, tuple)) else n_positions
         if n_max > config.max_position_embeddings:
