@@ -96,6 +96,57 @@ def test_generation_does_not_depend_on_the_schedule(tiny_folders, name):
     assert alone == together == portions == tight
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_running_ahead_changes_nothing_but_the_call_that_reports(tiny_folders, name):
+    """With `run_ahead` a step is started before the tokens of the step before it are read. Requests that
+    stop at their end-of-sequence token (found out one step late), at their length, that arrive while
+    others run, and that are put back for want of pages generate what they generate without it, and every
+    token is reported once, in order, the last one of a request marked as such."""
+    folder, cfg, weights = tiny_folders[name]
+    prompts = list(_requests(cfg["vocab_size"], [3, 9, 40, 77, 20, 5], 8).values())
+    free = [SamplingParams(max_new_tokens=14, do_sample=False, ignore_eos=True),
+            SamplingParams(max_new_tokens=14, temperature=0.9, seed=4, ignore_eos=True)] * 3
+
+    def generate(run_ahead, params, max_tokens=512, budget=64):
+        runner, ecfg = _runner(folder, max_tokens, max_num_batched_tokens=budget, run_ahead=run_ahead)
+        engine = LLMEngine(runner, ecfg)
+        seen, ends = {}, {}
+        ids = [engine.add_request(p, sp) for p, sp in zip(prompts[:4], params[:4])]
+        calls = 0
+        while engine.has_work:
+            for out in engine.step():
+                assert out.req_id not in ends, "a token after the last one"
+                seen.setdefault(out.req_id, []).append(out.token)
+                if out.finished:
+                    ends[out.req_id] = out.finish_reason
+            calls += 1
+            if calls == 3:                     # two more arrive while the others run
+                ids += [engine.add_request(p, sp) for p, sp in zip(prompts[4:], params[4:])]
+        runner.cache.check()
+        assert not runner.cache.requests
+        outs = [engine.requests[i].output for i in ids]
+        assert [seen[i] for i in ids] == outs and set(ends) == set(ids)
+        assert all(t >= 0 for o in outs for t in o)
+        return outs, [ends[i] for i in ids], engine.scheduler.num_preemptions
+
+    plain, reasons, _ = generate(False, free)
+    assert reasons == ["length"] * 6
+    assert generate(True, free)[:2] == (plain, reasons)
+    # each request now stops at the token it generated fifth, unless that token came earlier already
+    stopping = [SamplingParams(max_new_tokens=14, do_sample=sp.do_sample, temperature=sp.temperature, seed=sp.seed,
+                               eos_token_id=out[4]) for sp, out in zip(free, plain)]
+    want = [out[:out.index(out[4]) + 1] for out in plain]
+    for run_ahead in (False, True):
+        outs, reasons, _ = generate(run_ahead, stopping)
+        assert outs == want and reasons == ["eos"] * 6
+    # and with so few pages that requests are put back and computed again
+    late = [b if i == 3 else a for i, (a, b) in enumerate(zip(free, stopping))]
+    want = [b if i == 3 else a for i, (a, b) in enumerate(zip(plain, want))]
+    for run_ahead in (False, True):
+        outs, reasons, n = generate(run_ahead, late, max_tokens=160, budget=32)
+        assert outs == want and reasons == ["eos" if i == 3 else "length" for i in range(6)] and n > 0
+
+
 def test_sampled_tokens_follow_the_plain_sampler(tiny_folders):
     folder, cfg, weights = tiny_folders["A"]
     prompt = _requests(cfg["vocab_size"], [13], 4)["r0"]

@@ -161,3 +161,39 @@ def test_prompts_first_holds_decoding_until_every_prompt_is_in():
         seen.append([(r.request.req_id, r.start, r.count) for r in runs])
     # a is in after the first step and waits, with one token drawn, until b's prompt is in too
     assert seen == [[("a", 0, 30), ("b", 0, 10)], [("b", 10, 40)], [("b", 50, 10)], [("a", 30, 1), ("b", 60, 1)]]
+
+
+def test_a_step_recorded_before_its_tokens_are_known():
+    """`record` plans on with PENDING tokens, `resolve` fills them in one step late: an end by length is
+    known at once, an end-of-sequence token ends the request when it is read, and the run that the request
+    had in the step started meanwhile gives it nothing."""
+    from transformers_neuronx_amd.engine.scheduler import PENDING
+    s, cache = _sched()
+    s.add(_req("a", 5, new=3, eos_token_id=9))
+    s.add(_req("b", 6, new=8, eos_token_id=9))
+
+    def start():
+        runs = s.schedule()
+        for r in runs:
+            cache.advance(r.request.req_id, r.count)
+        s.record(runs)
+        cache.check()
+        return runs
+
+    first = start()                                  # both prompts; both draw a token
+    a, b = first[0].request, first[1].request
+    assert a.output == [PENDING] and b.output == [PENDING] and a.decoding and b.decoding
+    second = start()                                 # planned with the pending tokens: one token each
+    assert [(r.request.req_id, r.start, r.count, r.out_index) for r in second] == [("a", 5, 1, 1), ("b", 6, 1, 1)]
+    assert a.span(5, 1) == [PENDING]
+    assert s.resolve(first, [4, 9]) == [4, 9]        # b drew its end-of-sequence token in the first step
+    assert b.finished and b.finish_reason == "eos" and b.output == [9] and not cache.has("b")
+    assert a.output == [4, PENDING] and not a.finished
+    third = start()                                  # a alone; its third token ends it by length, at once
+    assert [r.request.req_id for r in third] == ["a"] and a.finished and a.finish_reason == "length"
+    assert not cache.has("a") and not s.has_work
+    assert s.resolve(second, [5, 6]) == [5, None]    # b's token of the second step is dropped
+    assert s.resolve(third, [9]) == [9]              # the last token happens to be the end-of-sequence one
+    assert a.output == [4, 5, 9] and a.finish_reason == "eos" and b.output == [9]
+    assert [r.req_id for r in s.finished] == ["b", "a"]
+    cache.check()

@@ -124,6 +124,8 @@ class EngineConfig:
                      steps go first and prompts fill what is left of the token budget)
     memory_fraction  share of free device memory the page pool may take when it
                      is sized from memory
+    run_ahead        a step is started before the host has read the tokens of the step before it (they
+                     stay on the device for it); generation is the same, tokens are reported one call later
     """
     dtype: torch.dtype = torch.bfloat16
     page_size: int = 64
@@ -137,6 +139,7 @@ class EngineConfig:
     memory_fraction: float = 0.85
     use_graphs: bool = True
     prompts_first: bool = False
+    run_ahead: bool = True
     seed: int = 0
 
     def __post_init__(self):

@@ -3,11 +3,15 @@
 
 TNX_DEFINE_ERROR_API
 
-// out[m, :] = src[idx[m], :], rows of `row_bytes` bytes (a multiple of 4).
+// out[m, :] = src[idx[m], :], rows of `row_bytes` bytes (a multiple of 4). An index -1 - k stands for
+// `indirect[k]`: a row number that an earlier kernel left in device memory (a token that was chosen on the
+// device and has not been read by the host yet).
 __global__ void gather_rows_kernel(const uint32_t* __restrict__ src, const int* __restrict__ idx,
-                                   uint32_t* __restrict__ out, int words, int src_rows) {
+                                   uint32_t* __restrict__ out, int words, int src_rows,
+                                   const int* __restrict__ indirect, int indirect_size) {
   const int m = blockIdx.x;
-  const int r = idx[m];
+  int r = idx[m];
+  if (r < 0 && indirect && -1 - r < indirect_size) r = indirect[-1 - r];
   if (r < 0 || r >= src_rows) return;  // the host checks ids; an id out of range writes nothing
   const uint32_t* s = src + (size_t)r * words;
   uint32_t* o = out + (size_t)m * words;
@@ -15,12 +19,38 @@ __global__ void gather_rows_kernel(const uint32_t* __restrict__ src, const int* 
 }
 
 extern "C" int tnx_gather_rows(const void* src, const int* idx, void* out, int m, int row_bytes, int src_rows,
-                               hipStream_t stream) {
+                               const int* indirect, int indirect_size, hipStream_t stream) {
   TNX_REQUIRE(row_bytes > 0 && row_bytes % 4 == 0, "gather_rows: row of %d bytes is not a multiple of 4", row_bytes);
   TNX_REQUIRE(m >= 0 && src_rows > 0, "gather_rows: bad sizes m=%d rows=%d", m, src_rows);
   if (m == 0) return 0;
-  gather_rows_kernel<<<m, 256, 0, stream>>>((const uint32_t*)src, idx, (uint32_t*)out, row_bytes / 4, src_rows);
+  gather_rows_kernel<<<m, 256, 0, stream>>>((const uint32_t*)src, idx, (uint32_t*)out, row_bytes / 4, src_rows,
+                                            indirect, indirect ? indirect_size : 0);
   TNX_CHECK_LAUNCH("gather_rows");
+  return 0;
+}
+
+// Integers from pinned host memory into device memory by a kernel on the caller's stream: the step's
+// integers arrive without a hand-over between the copy engine's queue and the compute queue.
+__global__ void copy_ints_kernel(const int* __restrict__ src, int* __restrict__ dst, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+
+extern "C" int tnx_copy_ints(const int* src, int* dst, int n, hipStream_t stream) {
+  TNX_REQUIRE(n >= 0 && src && dst, "copy_ints: bad arguments");
+  if (n == 0) return 0;
+  copy_ints_kernel<<<(n + 255) / 256, 256, 0, stream>>>(src, dst, n);
+  TNX_CHECK_LAUNCH("copy_ints");
+  return 0;
+}
+
+// The address under which kernels reach a block of pinned host memory.
+extern "C" int tnx_device_pointer(void* host, void** device) {
+  hipError_t e = hipHostGetDevicePointer(device, host, 0);
+  if (e != hipSuccess) {
+    tnx_set_error("device_pointer: %s", hipGetErrorString(e));
+    return 1;
+  }
   return 0;
 }
 

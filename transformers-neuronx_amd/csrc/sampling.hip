@@ -78,6 +78,29 @@ extern "C" int tnx_argmax(const float* logits, int* out, int rows, int vocab, hi
   return 0;
 }
 
+// kept[slot of the request of row rows[i]] = tokens[i]: the chosen tokens, left where the next step's
+// embedding finds them by the request's slot; and landing[i] = tokens[i] in pinned host memory, where the
+// host reads them once the kernel has ended.
+__global__ void store_tokens_kernel(const int* __restrict__ tokens, const int* __restrict__ rows,
+                                    const int* __restrict__ token_request, const int* __restrict__ slots, int n,
+                                    int* __restrict__ kept, int kept_size, int* __restrict__ landing) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int slot = slots[token_request[rows[i]]];
+  if (slot >= 0 && slot < kept_size) kept[slot] = tokens[i];
+  if (landing) landing[i] = tokens[i];
+}
+
+extern "C" int tnx_store_tokens(const int* tokens, const int* rows, const int* token_request, const int* slots,
+                                int n, int* kept, int kept_size, int* landing, hipStream_t stream) {
+  TNX_REQUIRE(n >= 0 && kept_size > 0, "store_tokens: bad sizes n=%d size=%d", n, kept_size);
+  if (n == 0) return 0;
+  store_tokens_kernel<<<(n + 255) / 256, 256, 0, stream>>>(tokens, rows, token_request, slots, n, kept, kept_size,
+                                                           landing);
+  TNX_CHECK_LAUNCH("store_tokens");
+  return 0;
+}
+
 // logits[row, token[row]] = -inf where token[row] >= 0: a token that must not be chosen.
 __global__ void ban_tokens_kernel(float* __restrict__ logits, const int* __restrict__ token, int rows, int vocab) {
   const int r = blockIdx.x * blockDim.x + threadIdx.x;

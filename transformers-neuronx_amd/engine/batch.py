@@ -51,6 +51,10 @@ class StepContext:
     tile_start: torch.Tensor = None      # int32, and its first query within the run
     query_tile: int = QUERY_TILE         # queries of a tile
     longest_decode: torch.Tensor = None  # int32 [1], the most keys a one-token run of this step reads
+    # int32 [slots]: the token last chosen for the request in each slot, on the device. A token id -1 - s
+    # in `token_ids` stands for `kept_tokens[s]`: a step can be started before the host has read the
+    # tokens that the step before it chose.
+    kept_tokens: Optional[torch.Tensor] = None
     longest_decode_host: int = 0
     # When a step is recorded for replay, nothing in its launches may depend on the lengths of this
     # particular step: `length_bound` then stands in for them where a launch is sized.

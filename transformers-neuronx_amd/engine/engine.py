@@ -14,7 +14,7 @@ from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from .batch import StepEntry
 from .runner import ModelRunner
-from .scheduler import Request, ScheduledRun, Scheduler
+from .scheduler import PENDING, Request, ScheduledRun, Scheduler
 
 
 @dataclass
@@ -25,7 +25,23 @@ class StepOutput:
     finish_reason: Optional[str]
 
 
+@dataclass
+class _StartedStep:
+    """A step whose tokens are chosen on the device and not read yet."""
+    runs: List[ScheduledRun]
+    sampling: List[ScheduledRun]
+    sent: object                         # the tokens on their way to the host (`ops.send_tokens`)
+    started: float
+
+
 class LLMEngine:
+    """With `run_ahead` (the default) a call of `step()` starts one step and returns the tokens of the
+    step before it: the device chooses a step's tokens and keeps them where the next step's embedding
+    finds them, so the host can plan, lay out and start that next step while the device still works,
+    and reads the tokens only afterwards. What a request generates is the same either way; a request
+    that ends at its end-of-sequence token is found out one step late, and the run it has in the step
+    started meanwhile is wasted and dropped."""
+
     def __init__(self, runner: ModelRunner, config: EngineConfig):
         self.runner, self.config = runner, config
         max_len = min(config.max_model_len or runner.max_positions, runner.max_positions)
@@ -38,6 +54,8 @@ class LLMEngine:
         self.record_timings = False
         # called with (requests that sample in this step, their logits [n, vocab] float32) before the draw
         self.logits_hook: Optional[Callable] = None
+        self.run_ahead = bool(getattr(config, "run_ahead", True))
+        self._started: Optional[_StartedStep] = None
 
     # ---------------------------------------------------------------- requests
 
@@ -54,39 +72,69 @@ class LLMEngine:
 
     @property
     def has_work(self) -> bool:
-        return self.scheduler.has_work
+        return self.scheduler.has_work or self._started is not None
 
     # ---------------------------------------------------------------- one step
 
-    @torch.no_grad()
-    def step(self) -> List[StepOutput]:
-        """Schedule, run, sample, record: one batch of portions and decoded tokens."""
+    def _start(self) -> Optional[_StartedStep]:
+        """Plan a step, run it, choose its tokens on the device and record it with the tokens pending."""
         runs = self.scheduler.schedule()
         if not runs:
-            return []
-        t0 = time.perf_counter() if self.record_timings else 0.0
+            return None
+        t0 = time.perf_counter()
         entries = []
         for run in runs:
             toks = run.request.span(run.start, run.count)
+            if toks[-1] == PENDING:
+                # drawn by the step before this one and not read yet: the device has it under the slot
+                toks = toks[:-1] + [-1 - self.runner.cache.slot_of(run.request.req_id)]
             entries.append(StepEntry(run.request.req_id, toks, [run.count - 1] if run.samples else []))
         logits = self.runner.step(entries)
         sampling = [r for r in runs if r.samples]
-        tokens: List[Optional[int]] = [None] * len(runs)
+        sent = None
         if sampling:
+            requests = [r.request for r in sampling]
             if self.logits_hook is not None:
-                self.logits_hook([r.request for r in sampling], logits)
-            drawn = self.sampler(logits, [r.request.params for r in sampling],
-                                 [len(r.request.output) for r in sampling])
-            it = iter(drawn)
-            tokens = [next(it) if r.samples else None for r in runs]
-        self.scheduler.update(runs, tokens)
+                self.logits_hook(requests, logits)
+            drawn = self.sampler.draw(logits, [q.params for q in requests], [len(q.output) for q in requests])
+            sent = self.runner.keep_tokens(drawn)
+        self.scheduler.record(runs)
+        return _StartedStep(runs, sampling, sent, t0)
+
+    def _finish(self, step: _StartedStep) -> List[StepOutput]:
+        """Read the tokens of a started step and give them to their requests."""
+        tokens: List[Optional[int]] = [None] * len(step.runs)
+        if step.sampling:
+            it = iter(self.runner.ops.receive_tokens(step.sent))
+            tokens = [next(it) if r.samples else None for r in step.runs]
+        kept = self.scheduler.resolve(step.runs, tokens)
         if self.record_timings:
             self.runner.ops.synchronize()
-            self.timings.append({"seconds": time.perf_counter() - t0, "tokens": sum(r.count for r in runs),
-                                 "prefill_tokens": sum(r.count for r in runs if r.count > 1 or not r.samples),
-                                 "sampled": len(sampling)})
-        return [StepOutput(r.request.req_id, t, r.request.finished, r.request.finish_reason)
-                for r, t in zip(runs, tokens) if t is not None]
+            self.timings.append({"seconds": time.perf_counter() - step.started,
+                                 "tokens": sum(r.count for r in step.runs),
+                                 "prefill_tokens": sum(r.count for r in step.runs if r.count > 1 or not r.samples),
+                                 "sampled": len(step.sampling)})
+        out = []
+        for r, t in zip(step.runs, kept):
+            if t is not None:
+                q = r.request
+                last = q.finished and r.out_index == len(q.output) - 1
+                out.append(StepOutput(q.req_id, t, last, q.finish_reason if last else None))
+        return out
+
+    @torch.no_grad()
+    def step(self) -> List[StepOutput]:
+        """Schedule, run, sample, record: one batch of portions and decoded tokens. Returns the tokens of
+        the step it ran, or with `run_ahead` those of the step started by the call before."""
+        if not self.run_ahead or self.record_timings:
+            out = self._finish(self._started) if self._started is not None else []
+            self._started = None
+            started = self._start()
+            return out + (self._finish(started) if started is not None else [])
+        started = self._start()
+        out = self._finish(self._started) if self._started is not None else []
+        self._started = started
+        return out
 
     def run(self, on_token: Optional[Callable[[StepOutput], None]] = None) -> None:
         """Step until every request has ended."""
@@ -106,6 +154,7 @@ class LLMEngine:
     def reset(self) -> None:
         """Forget every request and give back all pages (reference: `reset()` zero-fills
         the caches, decoder.py:1957-1969; here nothing needs clearing)."""
+        self._started = None
         self.scheduler.waiting.clear()
         self.scheduler.running.clear()
         self.runner.cache.reset()

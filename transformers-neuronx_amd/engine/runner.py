@@ -30,11 +30,16 @@ class _RecordedStep:
     def __init__(self, runner: "ModelRunner", packed: PackedStep):
         dev = runner.model.device
         self.layout = packed.layout()
-        self.host = torch.empty(packed.flat.size, dtype=torch.int32, pin_memory=True)
-        self.host.numpy()[:] = packed.flat
-        self.static = self.host.to(dev)
+        # Two pinned staging buffers in turn: the copy of one step may still be queued on the device when
+        # the host lays out the next (a step can be started before the one before it has ended).
+        self.ops = runner.ops
+        self.hosts = [runner.ops.pinned_ints(packed.flat.size) for _ in range(2)]
+        self.turn = 0
+        self.hosts[0][0].numpy()[:] = packed.flat
+        self.static = self.hosts[0][0].to(dev)
         self.ctx = context_from(packed, self.static)
         self.ctx.length_bound = runner.max_positions
+        self.ctx.kept_tokens = runner.kept_tokens
         side = torch.cuda.Stream(device=dev)
         side.wait_stream(torch.cuda.current_stream(dev))
         with torch.cuda.stream(side):           # once in the open: loads libraries, warms the allocator
@@ -46,8 +51,10 @@ class _RecordedStep:
             self.logits = runner.model.forward(self.ctx, runner.cache.caches)
 
     def replay(self, packed: PackedStep) -> torch.Tensor:
-        self.host.numpy()[:] = packed.flat
-        self.static.copy_(self.host, non_blocking=True)
+        self.turn ^= 1
+        pinned = self.hosts[self.turn]
+        pinned[0].numpy()[:] = packed.flat
+        self.ops.copy_ints(self.static, pinned)
         self.graph.replay()
         return self.logits
 
@@ -61,6 +68,10 @@ class ModelRunner:
         self.use_graphs = use_graphs and getattr(ops, "name", "") == "hip" and model.recordable
         self._recorded: Dict[tuple, _RecordedStep] = {}
         self.graph_replays = 0
+        # The token last chosen for the request in each slot, kept on the device: a step may name a token
+        # it brings as -1 - slot, and start before the host has read what the step before it chose.
+        self.kept_tokens = torch.zeros(cache.max_seqs, dtype=torch.int32, device=model.device)
+        self._last_ctx: Optional[StepContext] = None
 
     def prepare(self, entries: List[StepEntry], fixed_width: bool = False) -> PackedStep:
         """Admit new requests, get pages for the step's tokens, lay out the batch. With `fixed_width`
@@ -74,7 +85,7 @@ class ModelRunner:
             if len(e.tokens) == 0:
                 raise ValueError(f"request {e.req!r} brings no tokens")
             lo, hi = min(e.tokens), max(e.tokens)
-            if lo < 0 or hi >= self.vocab:
+            if lo < -self.kept_tokens.numel() or hi >= self.vocab:
                 raise ValueError(f"request {e.req!r}: token id {lo if lo < 0 else hi} is outside the vocabulary "
                                  f"of {self.vocab}")
         for e in entries:
@@ -111,13 +122,22 @@ class ModelRunner:
             if rec is None:
                 rec = self._recorded[key] = _RecordedStep(self, packed)
             logits = rec.replay(packed)
+            self._last_ctx = rec.ctx
             self.graph_replays += 1
         else:
             ctx = context_from(packed, torch.from_numpy(packed.flat).to(self.model.device))
+            ctx.kept_tokens = self.kept_tokens
             logits = self.model.forward(ctx, self.cache.caches)
+            self._last_ctx = ctx
         for e in entries:
             self.cache.advance(e.req, len(e.tokens))
         return logits if any(len(e.want) for e in entries) else None
+
+    def keep_tokens(self, tokens: torch.Tensor):
+        """Leave the tokens chosen from the last step's logits (one per wanted row, on the device) where
+        the next step finds them, under the slot of each row's request, and send them to the host.
+        Returns what `ops.receive_tokens` turns into a list."""
+        return self.ops.send_tokens(tokens, self.kept_tokens, self._last_ctx)
 
     def finish(self, req: Hashable) -> None:
         """The request is over: its pages and its slot go back."""

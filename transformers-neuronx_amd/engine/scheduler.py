@@ -17,6 +17,14 @@ Every decision is a function of arrival order, lengths and capacities only:
     lone request that does not fit raises `OutOfPages`;
   * a request ends at its end-of-sequence token (unless told to ignore it), at
     `max_new_tokens`, or at the length limit, and frees its pages in that step.
+
+A step's outcome may be recorded in two halves, so that the next step can be planned and started
+while the device still works on this one: `record` notes what was computed and puts `PENDING` in
+the place of every token that was drawn but not read yet (an end by length is known at once);
+`resolve` fills in the tokens when the host has them and ends requests at their end-of-sequence
+token. A request that is found to have ended this way may already be part of the step that was
+started meanwhile: that run's work is wasted and its token is dropped when it is resolved.
+`update` does both at once.
 """
 from collections import deque
 from dataclasses import dataclass, field
@@ -25,6 +33,9 @@ from typing import Deque, Hashable, List, Optional
 from ..cache.manager import CacheManager
 from ..cache.pages import OutOfPages
 from ..sampling.params import SamplingParams
+
+
+PENDING = -1              # stands in `Request.output` for a token that is drawn but not read yet
 
 
 @dataclass(eq=False)      # a request is itself: lists of requests are searched by identity
@@ -69,6 +80,7 @@ class ScheduledRun:
     count: int                      # tokens in the portion
     samples: bool = False           # the portion ends at the request's newest token: its last logits
                                     # pick the next one
+    out_index: int = -1             # where in the request's output that token goes
 
     def __post_init__(self):
         self.samples = self.start + self.count == self.request.num_tokens
@@ -205,29 +217,68 @@ class Scheduler:
 
     # ---------------------------------------------------------------- after the step
 
-    def update(self, runs: List[ScheduledRun], sampled: List[Optional[int]]) -> List[Request]:
-        """Record what the step computed and the tokens drawn for the runs that
-        sample (`sampled[i]` is None for the others). Returns the requests that ended."""
+    def _end(self, req: Request, reason: str, ended: List[Request]) -> None:
+        req.finish_reason = reason
+        if req.finished:
+            return
+        req.finished = True
+        if req in self.running:
+            self.running.remove(req)
+        elif req in self.waiting:
+            self.waiting.remove(req)
+        if self.cache.has(req.req_id):
+            self.cache.free_request(req.req_id)
+        self.finished.append(req)
+        ended.append(req)
+
+    def record(self, runs: List[ScheduledRun]) -> List[Request]:
+        """What the step computes, before its tokens are known: every run that samples gets `PENDING` as
+        its request's newest token. Requests that reach `max_new_tokens` or the length limit with it end
+        here and free what they hold (their last token is still to be resolved)."""
         ended = []
-        for run, token in zip(runs, sampled):
+        for run in runs:
             req = run.request
             req.num_computed = run.start + run.count
             if not run.samples:
                 continue
+            run.out_index = len(req.output)
+            req.output.append(PENDING)
+            if len(req.output) >= req.params.max_new_tokens:
+                self._end(req, "length", ended)
+            elif req.num_tokens > self.max_model_len:
+                self._end(req, "model_length", ended)
+        return ended
+
+    def resolve(self, runs: List[ScheduledRun], sampled: List[Optional[int]]) -> List[Optional[int]]:
+        """The tokens of a recorded step (`sampled[i]` is None for runs that do not sample). Returns, run
+        by run, the token that the request keeps, or None: for runs that do not sample and for runs of a
+        request that had ended at an earlier token when the step was started."""
+        kept: List[Optional[int]] = []
+        for run, token in zip(runs, sampled):
+            req = run.request
+            if not run.samples:
+                kept.append(None)
+                continue
             if token is None:
                 raise ValueError(f"request {req.req_id!r} needs a token this step")
-            req.output.append(int(token))
+            if run.out_index >= len(req.output):        # the request ended before this token
+                kept.append(None)
+                continue
+            req.output[run.out_index] = int(token)
+            kept.append(int(token))
             p = req.params
             if p.eos_token_id is not None and int(token) == p.eos_token_id and not p.ignore_eos:
-                req.finish_reason = "eos"
-            elif len(req.output) >= p.max_new_tokens:
-                req.finish_reason = "length"
-            elif req.num_tokens > self.max_model_len:
-                req.finish_reason = "model_length"
-            if req.finish_reason:
-                req.finished = True
-                self.running.remove(req)
-                self.cache.free_request(req.req_id)
-                self.finished.append(req)
-                ended.append(req)
-        return ended
+                del req.output[run.out_index + 1:]      # what was drawn after it is dropped
+                self._end(req, "eos", [])
+        return kept
+
+    def update(self, runs: List[ScheduledRun], sampled: List[Optional[int]]) -> List[Request]:
+        """Record what the step computed and the tokens drawn for the runs that
+        sample (`sampled[i]` is None for the others). Returns the requests that ended."""
+        before = len(self.finished)
+        for run, token in zip(runs, sampled):
+            if run.samples and token is None:
+                raise ValueError(f"request {run.request.req_id!r} needs a token this step")
+        self.record(runs)
+        self.resolve(runs, sampled)
+        return self.finished[before:]

@@ -20,7 +20,9 @@ _c_void_p, _c_int, _c_float, _c_ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_flo
 
 _SIGNATURES = {
     "elementwise": {
-        "tnx_gather_rows": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_gather_rows": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_void_p],
+        "tnx_copy_ints": [_c_void_p, _c_void_p, _c_int, _c_void_p],
+        "tnx_device_pointer": [_c_void_p, _c_void_p],
         "tnx_add_positions": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
                               _c_int, _c_int, _c_int, _c_void_p],
         "tnx_cast": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_void_p],
@@ -53,6 +55,8 @@ _SIGNATURES = {
     "sampling": {
         "tnx_ban_tokens": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
         "tnx_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+        "tnx_store_tokens": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p,
+                             _c_void_p],
         "tnx_sample": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                        _c_void_p],
     },
@@ -142,6 +146,7 @@ class HipOps:
             raise RuntimeError("the HIP kernels need a GPU; none is visible to torch")
         _code(dtype)
         self._bias_copies = {}
+        self._landing, self._landing_turn = [None, None], 0
 
     def _call(self, module: str, fn: str, *args):
         lib = library(module)
@@ -151,18 +156,63 @@ class HipOps:
 
     # ---------------------------------------------------------------- input end
 
-    def gather_rows(self, x, rows):
+    def gather_rows(self, x, rows, indirect=None):
+        """`x[rows]`; a row number -1 - k stands for `indirect[k]` (int32, on the device)."""
         _want(x, "x")
         _want(rows, "rows", torch.int32)
         if x.dim() != 2:
             raise ValueError("gather_rows takes a matrix")
+        if indirect is not None:
+            _want(indirect, "indirect rows", torch.int32)
         out = torch.empty(rows.numel(), x.shape[1], dtype=x.dtype, device=x.device)
         self._call("elementwise", "tnx_gather_rows", _ptr(x), _ptr(rows), _ptr(out), rows.numel(),
-                   x.shape[1] * x.element_size(), x.shape[0], _stream())
+                   x.shape[1] * x.element_size(), x.shape[0], _ptr(indirect),
+                   indirect.numel() if indirect is not None else 0, _stream())
         return out
 
-    def embed(self, token_ids, table, dtype=None):
-        return self.gather_rows(table, token_ids)
+    def embed(self, token_ids, table, dtype=None, kept_tokens=None):
+        """Rows of the token table; an id -1 - k is the token kept in `kept_tokens[k]`."""
+        return self.gather_rows(table, token_ids, kept_tokens)
+
+    def pinned_ints(self, n: int):
+        """`n` int32 in pinned host memory, and the address under which kernels reach them."""
+        host = torch.empty(n, dtype=torch.int32, pin_memory=True)
+        address = ctypes.c_void_p()
+        self._call("elementwise", "tnx_device_pointer", ctypes.c_void_p(host.data_ptr()), ctypes.byref(address))
+        return host, address
+
+    def copy_ints(self, dst, pinned) -> None:
+        """`dst[:] = host` for what `pinned_ints` returned, by a kernel on the current stream."""
+        host, address = pinned
+        _want(dst, "dst", torch.int32, (host.numel(),))
+        self._call("elementwise", "tnx_copy_ints", address, _ptr(dst), host.numel(), _stream())
+
+    def send_tokens(self, tokens, kept, ctx):
+        """Leave the chosen tokens for the next step (`kept[slot]`, see `store_tokens`) and write them into
+        pinned host memory by the same kernel. Returns what `receive_tokens` takes."""
+        n = tokens.numel()
+        self._landing_turn ^= 1
+        pinned = self._landing[self._landing_turn]
+        if pinned is None or pinned[0].numel() < n:
+            pinned = self._landing[self._landing_turn] = self.pinned_ints(max(2 * n, 256))
+        self.store_tokens(kept, tokens, ctx, pinned[1])
+        landed = torch.cuda.Event()
+        landed.record()
+        return pinned[0], n, landed
+
+    def receive_tokens(self, sent):
+        host, n, landed = sent
+        landed.synchronize()
+        return host[:n].tolist()
+
+    def store_tokens(self, kept, tokens, ctx, landing=None):
+        """`kept[slot]` = the token chosen for the request in that slot; `tokens[i]` belongs to the
+        request of the step's i-th wanted row. `landing`: an address in pinned host memory that gets
+        the tokens too."""
+        _want(kept, "kept tokens", torch.int32)
+        _want(tokens, "tokens", torch.int32, (ctx.logits_rows.numel(),))
+        self._call("sampling", "tnx_store_tokens", _ptr(tokens), _ptr(ctx.logits_rows), _ptr(ctx.token_request),
+                   _ptr(ctx.slots), tokens.numel(), _ptr(kept), kept.numel(), landing, _stream())
 
     def add_positions(self, src, positions, table, offset, dtype, want_compute):
         _want(src, "src")

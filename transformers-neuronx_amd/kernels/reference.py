@@ -33,8 +33,23 @@ class ReferenceOps:
 
     # ---------------------------------------------------------------- input end
 
-    def embed(self, token_ids, table, dtype=None):
-        return table[token_ids.long()]
+    def embed(self, token_ids, table, dtype=None, kept_tokens=None):
+        """Rows of the token table; an id -1 - k is the token kept in `kept_tokens[k]`."""
+        ids = token_ids.long()
+        if kept_tokens is not None:
+            ids = torch.where(ids < 0, kept_tokens.long()[(-1 - ids).clamp(min=0)], ids)
+        return table[ids]
+
+    def send_tokens(self, tokens, kept, ctx):
+        self.store_tokens(kept, tokens, ctx)
+        return tokens
+
+    def receive_tokens(self, sent):
+        return sent.tolist()
+
+    def store_tokens(self, kept, tokens, ctx):
+        slots = ctx.slots.long()[ctx.token_request.long()[ctx.logits_rows.long()]]
+        kept[slots] = tokens.to(kept.dtype)
 
     def add_positions(self, src, positions, table, offset, dtype, want_compute):
         x = src.float() + table[(positions + offset).long()].float()

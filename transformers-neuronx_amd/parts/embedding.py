@@ -34,7 +34,7 @@ class TokenEmbedding(Part):
         self.position.load(tensors, self.position_name, ops, dtype)
 
     def forward(self, ctx, want_compute: bool) -> Stream:
-        x = self.ops.embed(ctx.token_ids, self.table, self.dtype)
+        x = self.ops.embed(ctx.token_ids, self.table, self.dtype, ctx.kept_tokens)
         if self.projects:
             x = self.ops.linear(x, self.projection, None)
         xf, xc = self.position.at_input(x, ctx.positions, want_compute)

@@ -16,7 +16,11 @@ class Sampler:
         self.ops, self.device = ops, device
 
     def __call__(self, logits: torch.Tensor, params: List[SamplingParams], draws: List[int]) -> List[int]:
-        """`draws[i]` is how many tokens request i has drawn before: the counter of its stream."""
+        return self.draw(logits, params, draws).tolist()
+
+    def draw(self, logits: torch.Tensor, params: List[SamplingParams], draws: List[int]) -> torch.Tensor:
+        """The chosen tokens, int32 on the logits' device; nothing waits for the device here.
+        `draws[i]` is how many tokens request i has drawn before: the counter of its stream."""
         m = logits.shape[0]
         if m != len(params):
             raise ValueError(f"{m} logits rows for {len(params)} requests")
@@ -24,11 +28,11 @@ class Sampler:
         if any(b >= 0 for b in banned):
             self.ops.ban_tokens(logits, torch.tensor(banned, dtype=torch.int32, device=self.device))
         if all(p.greedy for p in params):
-            return self.ops.argmax(logits).tolist()
+            return self.ops.argmax(logits)
         temp = np.array([0.0 if p.greedy else p.temperature for p in params], dtype=np.float32)
         top_k = np.array([p.top_k for p in params], dtype=np.int32)
         top_p = np.array([p.top_p for p in params], dtype=np.float32)
         seeds = np.array([p.seed for p in params], dtype=np.int64)
         counters = np.array(draws, dtype=np.int64)
         dev = lambda a: torch.from_numpy(a).to(self.device)  # noqa: E731
-        return self.ops.sample(logits, dev(temp), dev(top_k), dev(top_p), dev(seeds), dev(counters)).tolist()
+        return self.ops.sample(logits, dev(temp), dev(top_k), dev(top_p), dev(seeds), dev(counters)).to(self.device)
