@@ -360,7 +360,9 @@ static int gemm_bf16_dispatch(const void* x, const void* w, const void* w_tiles,
   const bf16_t* ws = (const bf16_t*)w_tiles;
   TNX_REQUIRE(ws == nullptr || (N % 16 == 0 && K % 128 == 0),
               "gemm_bf16: a tile-ordered weight needs N a multiple of 16 and K of 128, got N=%d K=%d", N, K);
-  if (M <= 64 && force_tiled != 1) {
+  // The few-rows kernel up to 32 rows (beyond that every block reading all of `x` again costs more than the
+  // tiles' detour through LDS: 245 against 151 us for the 50,272 x 4,096 head at 64 rows), or when asked for.
+  if ((M <= 32 || ((force_tiled == 4 || force_tiled == 8) && M <= 64)) && force_tiled != 1) {
     // Eight waves a block when the sum over K is long and the rows are few (more bytes in flight for each
     // of the few blocks), four otherwise. force_tiled 4 or 8 picks the count, for measurements.
     const int waves = force_tiled == 4 || force_tiled == 8 ? force_tiled : (K >= 8192 && N <= 8192 ? 8 : 4);
