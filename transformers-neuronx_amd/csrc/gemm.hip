@@ -105,10 +105,80 @@ gemm_f32_kernel(const float* __restrict__ x, const float* __restrict__ w, const 
   }
 }
 
+// Few rows in float32 (decoding): the product is the weight read once. A wave makes 4 columns of the output
+// for up to MR rows of `x`; its lanes share K four floats at a time, so a row of the weight is read in runs
+// of 1 KB, and the 64 partial sums of every output meet in a butterfly at the end. K is a multiple of 4.
+template <int MR>
+__global__ void __launch_bounds__(256)
+gemm_f32_skinny_kernel(const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias,
+                       const float* __restrict__ residual, void* __restrict__ out, int out_dtype, int act, int M,
+                       int N, int K) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n0 = (blockIdx.x * 4 + wave) * 4;
+  if (n0 >= N) return;
+  const float* wrow[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) wrow[c] = w + (size_t)min(n0 + c, N - 1) * K;
+  const float* xrow[MR];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) xrow[m] = x + (size_t)min(m, M - 1) * K;
+  float acc[4][MR];
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[c][m] = 0.f;
+  const int k_last = K - 4;
+  for (int k0 = 0; k0 < K; k0 += 256) {
+    // lanes beyond K read the last four floats again and add nothing
+    const int k = min(k0 + 4 * lane, k_last);
+    const float keep = k0 + 4 * lane < K ? 1.f : 0.f;
+    f32x4 wv[4], xv[MR];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) wv[c] = *(const f32x4*)(wrow[c] + k);
+#pragma unroll
+    for (int m = 0; m < MR; ++m) xv[m] = *(const f32x4*)(xrow[m] + k);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const f32x4 wk = wv[c] * keep;
+#pragma unroll
+      for (int m = 0; m < MR; ++m) {
+        float a = acc[c][m];
+        a = fmaf(wk[0], xv[m][0], a);
+        a = fmaf(wk[1], xv[m][1], a);
+        a = fmaf(wk[2], xv[m][2], a);
+        a = fmaf(wk[3], xv[m][3], a);
+        acc[c][m] = a;
+      }
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      float a = acc[c][m];
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) a += __shfl_xor(a, o, 64);
+      // every lane has the sum; lane c * MR + m (modulo the wave) writes it
+      if (lane == ((c * MR + m) & 63) && n0 + c < N && m < M)
+        epilogue_store(a, m, n0 + c, N, bias, residual, out, out_dtype, act);
+    }
+}
+
 extern "C" int tnx_gemm_f32(const float* x, const float* w, const float* bias, const float* residual, void* out,
                             int out_dtype, int act, int M, int N, int K, hipStream_t stream) {
   TNX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_f32: bad sizes M=%d N=%d K=%d", M, N, K);
   if (M == 0) return 0;
+  if (M <= 16 && K % 4 == 0 && ((uintptr_t)x | (uintptr_t)w) % 16 == 0) {
+    const dim3 grid((N + 15) / 16);
+    if (M <= 4)
+      gemm_f32_skinny_kernel<4><<<grid, 256, 0, stream>>>(x, w, bias, residual, out, out_dtype, act, M, N, K);
+    else if (M <= 8)
+      gemm_f32_skinny_kernel<8><<<grid, 256, 0, stream>>>(x, w, bias, residual, out, out_dtype, act, M, N, K);
+    else
+      gemm_f32_skinny_kernel<16><<<grid, 256, 0, stream>>>(x, w, bias, residual, out, out_dtype, act, M, N, K);
+    TNX_CHECK_LAUNCH("gemm_f32_skinny");
+    return 0;
+  }
   dim3 grid((N + F32_TILE - 1) / F32_TILE, (M + F32_TILE - 1) / F32_TILE);
   TNX_REQUIRE(grid.y <= 65535, "gemm_f32: M=%d is too large", M);
   gemm_f32_kernel<<<grid, 256, 0, stream>>>(x, w, bias, residual, out, out_dtype, act, M, N, K);
