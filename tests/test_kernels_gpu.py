@@ -143,6 +143,10 @@ ATTN_CASES = [
     # several tiles of one run, starting inside a group of 8 positions and inside a page
     (2, 2, 64, 16, [300, 1, 9], [5, 40, 7]),
     (2, 1, 128, 64, [131, 2], [61, 126]),
+    # long decoding runs at head sizes that are no power of two: several tiles a wave, several splits
+    (3, 3, 80, 64, [1, 1], [700, 1300]),
+    (2, 2, 112, 16, [1, 5], [900, 40]),
+    (2, 1, 96, 32, [1, 1, 1], [300, 5, 64]),
 ]
 
 

@@ -834,9 +834,10 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                         const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
                         int page_shift, int num_pages, const int* __restrict__ decode_runs, bf16_t* __restrict__ out,
                         float* __restrict__ part_o, float* __restrict__ part_ml, int num_heads, int num_kv,
-                        int window, int num_splits, const int* __restrict__ longest_ptr) {
+                        int window, int num_splits, const int* __restrict__ longest_ptr, int head_size) {
   constexpr int KPI = 64 / CPR;       // keys per load instruction of a wave
-  constexpr int DH = CPR * 8;
+  constexpr int DH = CPR * 8;         // the lanes' layout is made for this head size; `head_size` <= DH
+  const int cpr = head_size / 8;      // chunks a key really has: lanes of higher chunks repeat the last one
   __shared__ float sm_p[NW][64];
   __shared__ float sm_o[NW][DH];
   __shared__ float sm_m[NW], sm_l[NW];
@@ -847,7 +848,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
   const int t = run_start[run];
   const int pos = cached_lens[run];   // the query's own position; its key is stored already
   const int* tab = table + (size_t)run * table_width;
-  const int nq = num_heads * DH;
+  const int nq = num_heads * head_size;
   const int page_size = 1 << page_shift, pmask = page_size - 1;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   // The longest range of keys any decoding request of the step reads is given in device memory, so that a
@@ -857,13 +858,14 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
   const int k_begin = (lo / 64) * 64 + split * keys_per_split;
   const int k_end = min(pos + 1, k_begin + keys_per_split);
   const int dchunk = lane % CPR, kgrp = lane / CPR;
-  const size_t head_stride = (size_t)page_size * DH;   // elements of one head of one page
+  const size_t head_stride = (size_t)page_size * head_size;   // elements of one head of one page
+  const int kchunk = min(dchunk, cpr - 1);
 
   float qf[8];
   {
-    const bf16x8 qv = *(const bf16x8*)(q + (size_t)t * nq + h * DH + dchunk * 8);
+    const bf16x8 qv = *(const bf16x8*)(q + (size_t)t * nq + h * head_size + kchunk * 8);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) qf[j] = (float)qv[j];
+    for (int j = 0; j < 8; ++j) qf[j] = dchunk < cpr ? (float)qv[j] : 0.f;
   }
   float m = -INFINITY, l = 0.f;
   float acc[CPR];
@@ -876,8 +878,8 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     for (int i = 0; i < CPR; ++i) {
       const int key = min(tile0 + i * KPI + kgrp, pos);
       const int page = min(max(tab[key >> page_shift], 0), num_pages - 1);
-      kv[i] = *(const bf16x8*)(k_pages + ((size_t)page * num_kv + kvh) * head_stride + (size_t)(key & pmask) * DH +
-                               dchunk * 8);
+      kv[i] = *(const bf16x8*)(k_pages + ((size_t)page * num_kv + kvh) * head_stride +
+                               (size_t)(key & pmask) * head_size + kchunk * 8);
     }
     float part[CPR];
 #pragma unroll
@@ -920,7 +922,8 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     const bf16_t* vbase = v_pages + ((size_t)vpage * num_kv + kvh) * head_stride + (vkey & pmask);
     bf16x8 vv[CPR];
 #pragma unroll
-    for (int i = 0; i < CPR; ++i) vv[i] = *(const bf16x8*)(vbase + (size_t)(i * 8 + (lane >> 3)) * page_size);
+    for (int i = 0; i < CPR; ++i)
+      vv[i] = *(const bf16x8*)(vbase + (size_t)min(i * 8 + (lane >> 3), head_size - 1) * page_size);
     float pv[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) pv[j] = sm_p[wave][kc * 8 + j];
@@ -946,7 +949,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     sm_l[wave] = l;
   }
   __syncthreads();
-  for (int d = threadIdx.x; d < DH; d += 64 * NW) {
+  for (int d = threadIdx.x; d < head_size; d += 64 * NW) {
     float mm = sm_m[0];
 #pragma unroll
     for (int w = 1; w < NW; ++w) mm = fmaxf(mm, sm_m[w]);
@@ -959,10 +962,10 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
       oo += sm_o[w][d] * f;
     }
     if (num_splits == 1) {
-      out[(size_t)t * nq + h * DH + d] = (bf16_t)(oo / ll);
+      out[(size_t)t * nq + h * head_size + d] = (bf16_t)(oo / ll);
     } else {
       const size_t pi = ((size_t)dz * num_heads + h) * num_splits + split;
-      part_o[pi * DH + d] = oo;
+      part_o[pi * head_size + d] = oo;
       if (d == 0) {
         part_ml[pi * 2] = mm;
         part_ml[pi * 2 + 1] = ll;
@@ -998,8 +1001,8 @@ extern "C" int tnx_attention_decode(const void* q, const void* k_pages, const vo
                                     float* part_ml, int num_heads, int num_kv, int head_size, int window,
                                     int num_splits, int waves, const int* longest, hipStream_t stream) {
   TNX_REQUIRE(num_heads > 0 && num_kv > 0 && num_heads % num_kv == 0, "attention_decode: bad head counts");
-  TNX_REQUIRE(head_size == 16 || head_size == 32 || head_size == 64 || head_size == 128 || head_size == 256,
-              "attention_decode: head size %d is not one of 16, 32, 64, 128, 256", head_size);
+  TNX_REQUIRE(head_size % 16 == 0 && head_size >= 16 && head_size <= 256,
+              "attention_decode: head size %d is not a multiple of 16 in [16, 256]", head_size);
   TNX_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0,
               "attention_decode: page size %d is not a power of two from 16 up", page_size);
   int page_shift = 0;
@@ -1014,20 +1017,23 @@ extern "C" int tnx_attention_decode(const void* q, const void* k_pages, const vo
 #define LAUNCH_DECODE_ARGS                                                                                          \
   (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, table_width,     \
       page_shift, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window, num_splits,     \
-      longest
+      longest, head_size
 #define LAUNCH_DECODE(CPR)                                                                                         \
   if (waves == 8)                                                                                                  \
     attention_decode_kernel<CPR, 8><<<grid, 512, 0, stream>>>(LAUNCH_DECODE_ARGS);                                 \
   else                                                                                                             \
     attention_decode_kernel<CPR, 4><<<grid, 256, 0, stream>>>(LAUNCH_DECODE_ARGS)
-  switch (head_size) {
-    case 16: LAUNCH_DECODE(2); break;
-    case 32: LAUNCH_DECODE(4); break;
-    case 64: LAUNCH_DECODE(8); break;
-    case 128: LAUNCH_DECODE(16); break;
-    default:
-      attention_decode_kernel<32, 4><<<grid, 256, 0, stream>>>(LAUNCH_DECODE_ARGS);
-      break;
+  // the lanes' layout is that of the next power of two; a smaller head leaves some lanes idle
+  if (head_size <= 16) {
+    LAUNCH_DECODE(2);
+  } else if (head_size <= 32) {
+    LAUNCH_DECODE(4);
+  } else if (head_size <= 64) {
+    LAUNCH_DECODE(8);
+  } else if (head_size <= 128) {
+    LAUNCH_DECODE(16);
+  } else {
+    attention_decode_kernel<32, 4><<<grid, 256, 0, stream>>>(LAUNCH_DECODE_ARGS);
   }
 #undef LAUNCH_DECODE
 #undef LAUNCH_DECODE_ARGS

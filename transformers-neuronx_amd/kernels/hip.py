@@ -412,7 +412,7 @@ class HipOps:
         window = int(window or 0)
         fast = (self.dtype == torch.bfloat16 and not self.force_plain_attention
                 and (ctx.decode_runs.numel() == 0
-                     or (head_size in (16, 32, 64, 128, 256) and view.page_size & (view.page_size - 1) == 0)))
+                     or view.page_size & (view.page_size - 1) == 0))
         if not fast:
             self._call("attention", "tnx_attention_any", _ptr(q), _code(self.dtype), _ptr(k_pages), _ptr(v_pages),
                        _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width,
