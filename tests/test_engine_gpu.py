@@ -234,9 +234,23 @@ def test_schedules_with_library_products(tiny_folders_bf16, tmp_path, monkeypatc
         _compare(out, place, expected, cfg["vocab_size"], "bfloat16")
 
 
-def test_bfloat16_against_float32_at_full_layer_sizes():
-    """Two layers of the sizes of OPT-6.7B (width 4096, 32 heads of 128, inner width 16384, vocabulary
-    50272): the bfloat16 engine against the float32 engine on the same (bfloat16-stored) random weights,
+FULL_SIZES = {
+    # the layer sizes of three members of the family (reference: the 175B key set, gen_random_pretrained.py:105-140)
+    "6.7b": dict(vocab_size=50272, hidden_size=4096, num_hidden_layers=2, num_attention_heads=32, ffn_dim=16384,
+                 max_position_embeddings=2048, init_std=0.02),
+    # heads of 80: no power of two
+    "2.7b": dict(vocab_size=50272, hidden_size=2560, num_hidden_layers=2, num_attention_heads=32, ffn_dim=10240,
+                 max_position_embeddings=2048, init_std=0.02),
+    # the norm after each half, an embedding narrower than the model
+    "350m": dict(vocab_size=50272, hidden_size=1024, num_hidden_layers=3, num_attention_heads=16, ffn_dim=4096,
+                 max_position_embeddings=2048, word_embed_proj_dim=512, do_layer_norm_before=False, init_std=0.02),
+}
+
+
+@pytest.mark.parametrize("size", list(FULL_SIZES))
+def test_bfloat16_against_float32_at_full_layer_sizes(size):
+    """A few layers of the sizes of OPT-6.7B (width 4096, 32 heads of 128, inner width 16384, vocabulary
+    50272), OPT-2.7B and OPT-350m: the bfloat16 engine against the float32 engine on the same (bfloat16-stored) random weights,
     under a schedule that takes a long prompt in portions, decodes beside another prompt, and ends with
     recorded decode steps. The reference's own yardstick for such a pair is `allclose(atol=1.0,
     rtol=1e-3)` with equal argmax (generation_demo.py:437-443); here the bound is the bfloat16 one of the
@@ -246,9 +260,7 @@ def test_bfloat16_against_float32_at_full_layer_sizes():
     from transformers_neuronx_amd.engine.factory import build_runner
     from transformers_neuronx_amd.opt.spec import opt_spec
     from transformers_neuronx_amd.weights import TensorDict, random_tensors
-    raw = dict(vocab_size=50272, hidden_size=4096, num_hidden_layers=2, num_attention_heads=32, ffn_dim=16384,
-               max_position_embeddings=2048, init_std=0.02)
-    cfg = OPTConfig.from_dict(raw)
+    cfg = OPTConfig.from_dict(FULL_SIZES[size])
     spec = opt_spec(cfg)
     tensors = random_tensors(DecoderModel(spec).param_decls(), spec.init_std, 3, torch.bfloat16, DEV)
     g = torch.Generator().manual_seed(0)
