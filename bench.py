@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine at OPT-6.7B size with random weights.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--model 6.7b|350m|66b] [--mix]
 
 One JSON line: `value` is decoded tokens per second at batch 8 and a 2,048-token context
 (a "step" is one decode step of the whole engine: schedule, model, sampling);
@@ -26,6 +26,12 @@ MODEL = dict(architectures=["OPTForCausalLM"], model_type="opt", vocab_size=5027
              num_hidden_layers=32, num_attention_heads=32, ffn_dim=16384, max_position_embeddings=2048,
              word_embed_proj_dim=4096, do_layer_norm_before=True, activation_function="relu", enable_bias=True,
              layer_norm_elementwise_affine=True, init_std=0.02, torch_dtype="bfloat16")
+# The other sizes BASELINE.json names, for `--model` (the default run and its JSON line stay OPT-6.7B)
+OTHER_MODELS = {
+    "350m": dict(hidden_size=1024, num_hidden_layers=24, num_attention_heads=16, ffn_dim=4096, word_embed_proj_dim=512,
+                 do_layer_norm_before=False),
+    "66b": dict(hidden_size=9216, num_hidden_layers=64, num_attention_heads=72, ffn_dim=36864, word_embed_proj_dim=9216),
+}
 CONTEXT = 2048
 PREFILL_TOKENS = 2048
 PEAK_HBM_GBS = 8000.0                      # MI355X, published
@@ -52,6 +58,12 @@ def main():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--prefill-only", action="store_true", help="measure the prompt step alone (for profiles)")
+    ap.add_argument("--model", default="6.7b", choices=["6.7b"] + sorted(OTHER_MODELS),
+                    help="layer sizes: OPT-6.7B (the measurement of record) or another size BASELINE.json names")
+    ap.add_argument("--mix", action="store_true",
+                    help="instead: 64 requests with prompts of 16 to 1,024 tokens and 256 new tokens each, all "
+                         "queued at once (BASELINE.json's continuous-batching workload); prints its own line")
+    ap.add_argument("--big-batch", type=int, default=64, help="the larger batch of `points` (66b: 32 fits)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -64,12 +76,13 @@ def main():
     from transformers_neuronx_amd.sampling import SamplingParams
 
     raw = dict(MODEL)
+    raw.update(OTHER_MODELS.get(args.model, {}))
     layers_full = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
     cfg = OPTConfig.from_dict(raw)
     dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
-    max_batch = args.batch if args.no_points else max(args.batch, 64)
+    max_batch = args.batch if args.no_points else max(args.batch, args.big_batch)
     ecfg = EngineConfig(dtype=dtype, page_size=64, max_tokens=max_batch * CONTEXT, max_num_seqs=max_batch,
                         max_num_batched_tokens=max(2048, PREFILL_TOKENS), max_model_len=CONTEXT,
                         prompts_first=True)
@@ -121,6 +134,30 @@ def main():
             times.append(time.perf_counter() - start)
         return sorted(times[1:])[2]       # the median of five, after one warm-up
 
+    if args.mix:
+        # every request is there at the start; the scheduler mixes portions of prompts with decoding
+        engine.reset()
+        lengths = torch.randint(16, 1025, (64,), generator=gen).tolist()
+        params = SamplingParams(max_new_tokens=256, do_sample=False, ignore_eos=True)
+        for n in lengths:
+            engine.add_request(torch.randint(3, cfg.vocab_size, (n,), generator=gen).tolist(), params)
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        first, made, steps = {}, 0, 0
+        while engine.has_work:
+            for o in engine.step():
+                first.setdefault(o.req_id, time.perf_counter() - start)
+                made += 1
+            steps += 1
+        torch.cuda.synchronize()
+        sec = time.perf_counter() - start
+        assert made == 64 * 256, made
+        print(json.dumps({"metric": f"OPT-{args.model.upper()} continuous batching: 64 requests, prompts 16-1,024, "
+                                    "256 new tokens each", "value": round(made / sec, 1), "unit": "generated tokens/s",
+                          "seconds": round(sec, 3), "steps": steps, "prompt_tokens": sum(lengths),
+                          "mean_time_to_first_token_ms": round(1e3 * sum(first.values()) / len(first), 2),
+                          "preemptions": engine.scheduler.num_preemptions, "dtype": args.dtype}))
+        return 0
     if args.prefill_only:
         sec_p = prefill(PREFILL_TOKENS)
         print(json.dumps({"prefill_ms": round(sec_p * 1e3, 3), "tokens": PREFILL_TOKENS,
@@ -130,11 +167,11 @@ def main():
     print(f"[bench] decode batch {args.batch}: {value:.1f} tok/s, {sec * 1e3:.2f} ms/step", file=sys.stderr, flush=True)
     achieved = read / sec / 1e9
     out = {
-        "metric": "OPT-6.7B decode tok/s @ batch 1/8/64; prefill tok/s @ 2,048 tokens",
+        "metric": f"OPT-{args.model.upper()} decode tok/s @ batch 1/8/{args.big_batch}; prefill tok/s @ 2,048 tokens",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic (seeded random weights and token ids)",
-        "config": {"model": "OPT-6.7B", "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "none",
+        "config": {"model": "OPT-" + args.model.upper(), "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "none",
                    "layers": cfg.num_hidden_layers, "layers_of_model": layers_full, "hidden_size": cfg.hidden_size,
                    "heads": cfg.num_attention_heads, "head_size": cfg.head_size, "ffn_dim": cfg.ffn_dim,
                    "vocab_size": cfg.vocab_size, "max_positions": cfg.max_position_embeddings,
@@ -151,7 +188,8 @@ def main():
                           "ms": round(sec_p * 1e3, 3), "frac": round(flops / sec_p / PEAK_FLOPS[args.dtype], 4)}
         print(f"[bench] prefill: {out['prefill']}", file=sys.stderr, flush=True)
         points = {}
-        for b, k, w in ((1, min(args.steps, 64), args.warmup), (64, min(args.steps, 32), min(args.warmup, 4))):
+        for b, k, w in ((1, min(args.steps, 64), args.warmup),
+                        (args.big_batch, min(args.steps, 32), min(args.warmup, 4))):
             v, s, _ = decode(b, k, w)
             points[f"decode_b{b}"] = round(v, 2)
             print(f"[bench] decode batch {b}: {v:.1f} tok/s, {s * 1e3:.2f} ms/step", file=sys.stderr, flush=True)

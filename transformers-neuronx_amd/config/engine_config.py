@@ -124,6 +124,9 @@ class EngineConfig:
                      steps go first and prompts fill what is left of the token budget)
     memory_fraction  share of free device memory the page pool may take when it
                      is sized from memory
+    weight_copies    keep a second copy of every matrix in the order the few-rows product streams it
+                     (faster decoding at small batches, twice the memory for matrices); None decides by
+                     what fits beside the cache
     run_ahead        a step is started before the host has read the tokens of the step before it (they
                      stay on the device for it); generation is the same, tokens are reported one call later
     """
@@ -140,6 +143,7 @@ class EngineConfig:
     use_graphs: bool = True
     prompts_first: bool = False
     run_ahead: bool = True
+    weight_copies: Optional[bool] = None
     seed: int = 0
 
     def __post_init__(self):

@@ -34,15 +34,37 @@ def size_page_pool(cfg: EngineConfig, bytes_per_page: int, device: torch.device)
     return 256
 
 
+def _room_for_weight_copies(cfg: EngineConfig, model: DecoderModel, bytes_per_page: int, device) -> bool:
+    """Whether the matrices get a second, tile-ordered copy for the few-rows product (`weight_copies`;
+    left open, they do when matrices twice over and the cache asked for fit 90 % of the device's memory,
+    a quarter of it standing in for a cache sized from what is left)."""
+    if cfg.weight_copies is not None:
+        return bool(cfg.weight_copies)
+    if device.type != "cuda" or cfg.dtype != torch.bfloat16:
+        return False
+    matrices = sum(2 * int(torch.Size(d.shape).numel()) for d in model.param_decls() if d.role in ("matrix", "table"))
+    _, total = torch.cuda.mem_get_info(device)
+    if cfg.num_pages is not None:
+        cache = cfg.num_pages * bytes_per_page
+    elif cfg.max_tokens is not None:
+        cache = -(-cfg.max_tokens // cfg.page_size) * bytes_per_page
+    else:
+        cache = total // 4
+    return 2.2 * matrices + cache <= 0.9 * total
+
+
 def build_runner(model_config, source, cfg: EngineConfig) -> ModelRunner:
     """`model_config` a typed configuration, `source` a `Checkpoint` or `TensorDict`."""
     device = _device_of(cfg)
     arch = resolve(model_config.to_dict())
     model = DecoderModel(arch.build_spec(model_config))
     ops = make_ops(cfg.kernels, cfg.dtype, device)
-    model.load(source, ops, cfg.dtype, device)
     needs = model.cache_needs()
-    num_pages = size_page_pool(cfg, CacheManager.bytes_per_page(needs, cfg.page_size, cfg.dtype), device)
+    bytes_per_page = CacheManager.bytes_per_page(needs, cfg.page_size, cfg.dtype)
+    if hasattr(ops, "decode_copies"):
+        ops.decode_copies = _room_for_weight_copies(cfg, model, bytes_per_page, device)
+    model.load(source, ops, cfg.dtype, device)
+    num_pages = size_page_pool(cfg, bytes_per_page, device)
     cache = CacheManager(needs, cfg.page_size, num_pages, cfg.max_num_seqs, cfg.dtype, device)
     return ModelRunner(model, cache, ops, use_graphs=cfg.use_graphs)
 
