@@ -333,8 +333,14 @@ class HipOps:
         return kept[1]
 
     def _library_product(self, m, n, k, w, force_tiled) -> bool:
-        return (self.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and self.library_rows > 0
-                and m >= self.library_rows and not force_tiled and n % 8 == 0 and k % 8 == 0)
+        if not (self.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and self.library_rows > 0
+                and m >= self.library_rows and not force_tiled and n % 8 == 0 and k % 8 == 0):
+            return False
+        # small matrices at up to 32 rows: one launch of ours (5 to 10 us with its epilogue) beats the
+        # library's product and the epilogue after it (11 to 15 us)
+        return not (m <= 32 and n * k <= self.small_matrix)
+
+    small_matrix = 1 << 23
 
     # ---------------------------------------------------------------- attention
 
