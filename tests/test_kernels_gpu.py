@@ -177,6 +177,14 @@ def _fill_cache_and_compare(dtype, heads, kv, hs, ps, runs, cached, window):
     qkv = torch.randn(ctx.num_tokens, width, device=DEV, generator=g).to(dtype)
     q_h = hip.qkv_write(qkv, bias, heads, kv, hs, scale, ctx, ctx.groups["full"], kp, vp)
     q_r = ref.qkv_write(qkv, bias, heads, kv, hs, scale, ctx, ctx.groups["full"], kp_r, vp_r)
+    if dtype == torch.bfloat16:
+        # values written by tiles (the default for runs of several tokens) and token by token: the same bits
+        tokenwise = type(hip)(dtype, DEV)
+        tokenwise.value_tiles = False
+        kp_t, vp_t = kp_r.clone(), vp_r.clone()      # the reference's pages hold the cached part already
+        kp_t.copy_(kp), vp_t.copy_(vp)
+        tokenwise.qkv_write(qkv, bias, heads, kv, hs, scale, ctx, ctx.groups["full"], kp_t, vp_t)
+        assert torch.equal(torch.nan_to_num(vp_t.float()), torch.nan_to_num(vp.float()))
     tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
     torch.testing.assert_close(q_h.float(), q_r.float(), **tol)
     # what was written is the same, and nothing else was touched (untouched places are still NaN)
@@ -327,6 +335,11 @@ def test_bfloat16_attention_kernels_agree(case, window):
     direct.prefill_direct = True                  # the prompt kernel that reads the pages without staging
     o_direct = direct.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)
     torch.testing.assert_close(o_direct.float(), o_plain.float(), rtol=2e-2, atol=2e-2)
+    narrow = HipOps(torch.bfloat16, DEV)
+    narrow.decode_wide_blocks = 0                 # blocks of four waves only, twice the splits
+    narrow.decode_blocks_wanted = 1 << 20
+    o_narrow = narrow.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)
+    torch.testing.assert_close(o_narrow.float(), o_plain.float(), rtol=2e-2, atol=2e-2)
     one = HipOps(torch.bfloat16, DEV)
     one.decode_blocks_wanted = 1                  # no split at all
     o_one = one.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)
