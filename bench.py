@@ -60,6 +60,8 @@ def main():
     ap.add_argument("--prefill-only", action="store_true", help="measure the prompt step alone (for profiles)")
     ap.add_argument("--model", default="6.7b", choices=["6.7b"] + sorted(OTHER_MODELS),
                     help="layer sizes: OPT-6.7B (the measurement of record) or another size BASELINE.json names")
+    ap.add_argument("--do-sample", action="store_true",
+                    help="decode with temperature 0.8, top-k 50 and top-p 0.95 instead of greedily")
     ap.add_argument("--mix", action="store_true",
                     help="instead: 64 requests with prompts of 16 to 1,024 tokens and 256 new tokens each, all "
                          "queued at once (BASELINE.json's continuous-batching workload); prints its own line")
@@ -101,8 +103,9 @@ def main():
         the full context."""
         engine.reset()
         prompt_len = CONTEXT - (steps + warmup) - 1
-        params = SamplingParams(max_new_tokens=steps + warmup + 1, do_sample=False, ignore_eos=True)
-        for _ in range(batch):
+        for i in range(batch):
+            params = SamplingParams(max_new_tokens=steps + warmup + 1, do_sample=args.do_sample, temperature=0.8,
+                                    top_k=50, top_p=0.95, seed=i, ignore_eos=True)
             engine.add_request(torch.randint(3, cfg.vocab_size, (prompt_len,), generator=gen).tolist(), params)
         while any(not r.decoding for r in engine.requests.values()):
             engine.step()                 # prompts first: nothing decodes until every prompt is in
@@ -170,7 +173,8 @@ def main():
         "metric": f"OPT-{args.model.upper()} decode tok/s @ batch 1/8/{args.big_batch}; prefill tok/s @ 2,048 tokens",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": args.dtype, "data": "synthetic (seeded random weights and token ids)",
+        "dtype": args.dtype, "data": "synthetic (seeded random weights and token ids)"
+                                      + (", sampled (temperature 0.8, top-k 50, top-p 0.95)" if args.do_sample else ""),
         "config": {"model": "OPT-" + args.model.upper(), "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "none",
                    "layers": cfg.num_hidden_layers, "layers_of_model": layers_full, "hidden_size": cfg.hidden_size,
                    "heads": cfg.num_attention_heads, "head_size": cfg.head_size, "ffn_dim": cfg.ffn_dim,

@@ -21,6 +21,37 @@ from .batch import PackedStep, StepContext, StepEntry, context_from, pack_step
 from .model import DecoderModel
 
 
+class _Staging:
+    """Integers from the host to the device without a wait: two pinned buffers in turn, copied by a kernel
+    on the current stream. A pageable copy would hold the host until the device has caught up, and with
+    it the start of the next step. A buffer is written again only when the copy that read it has run."""
+
+    def __init__(self, ops, size: int = 0):
+        self.ops = ops
+        self.buffers = [None, None]
+        self.done = [None, None]
+        self.turn = 0
+        if size:
+            self.buffers = [ops.pinned_ints(size), ops.pinned_ints(size)]
+
+    def send(self, flat: np.ndarray, dst: Optional[torch.Tensor] = None, device=None) -> torch.Tensor:
+        n = flat.size
+        self.turn ^= 1
+        i = self.turn
+        if self.buffers[i] is None or self.buffers[i][0].numel() < n:
+            self.buffers[i] = self.ops.pinned_ints(max(2 * n, 1024))
+        elif self.done[i] is not None:
+            self.done[i].synchronize()
+        self.buffers[i][0].numpy()[:n] = flat
+        if dst is None:
+            dst = torch.empty(n, dtype=torch.int32, device=device)
+        self.ops.copy_ints(dst, self.buffers[i], n)
+        if self.done[i] is None:
+            self.done[i] = torch.cuda.Event()
+        self.done[i].record()
+        return dst
+
+
 class _RecordedStep:
     """A decode step recorded as a HIP graph: the launches of one step over a fixed number of
     one-token runs, reading their integers from a device buffer that is rewritten before each replay.
@@ -30,13 +61,8 @@ class _RecordedStep:
     def __init__(self, runner: "ModelRunner", packed: PackedStep):
         dev = runner.model.device
         self.layout = packed.layout()
-        # Two pinned staging buffers in turn: the copy of one step may still be queued on the device when
-        # the host lays out the next (a step can be started before the one before it has ended).
-        self.ops = runner.ops
-        self.hosts = [runner.ops.pinned_ints(packed.flat.size) for _ in range(2)]
-        self.turn = 0
-        self.hosts[0][0].numpy()[:] = packed.flat
-        self.static = self.hosts[0][0].to(dev)
+        self.staging = _Staging(runner.ops, packed.flat.size)
+        self.static = torch.from_numpy(packed.flat).to(dev)
         self.ctx = context_from(packed, self.static)
         self.ctx.length_bound = runner.max_positions
         self.ctx.kept_tokens = runner.kept_tokens
@@ -51,10 +77,7 @@ class _RecordedStep:
             self.logits = runner.model.forward(self.ctx, runner.cache.caches)
 
     def replay(self, packed: PackedStep) -> torch.Tensor:
-        self.turn ^= 1
-        pinned = self.hosts[self.turn]
-        pinned[0].numpy()[:] = packed.flat
-        self.ops.copy_ints(self.static, pinned)
+        self.staging.send(packed.flat, self.static)
         self.graph.replay()
         return self.logits
 
@@ -72,6 +95,7 @@ class ModelRunner:
         # it brings as -1 - slot, and start before the host has read what the step before it chose.
         self.kept_tokens = torch.zeros(cache.max_seqs, dtype=torch.int32, device=model.device)
         self._last_ctx: Optional[StepContext] = None
+        self._staging = _Staging(ops) if hasattr(ops, "pinned_ints") else None
 
     def prepare(self, entries: List[StepEntry], fixed_width: bool = False) -> PackedStep:
         """Admit new requests, get pages for the step's tokens, lay out the batch. With `fixed_width`
@@ -125,7 +149,11 @@ class ModelRunner:
             self._last_ctx = rec.ctx
             self.graph_replays += 1
         else:
-            ctx = context_from(packed, torch.from_numpy(packed.flat).to(self.model.device))
+            if self._staging is not None:
+                ints = self._staging.send(packed.flat, device=self.model.device)
+            else:
+                ints = torch.from_numpy(packed.flat).to(self.model.device)
+            ctx = context_from(packed, ints)
             ctx.kept_tokens = self.kept_tokens
             logits = self.model.forward(ctx, self.cache.caches)
             self._last_ctx = ctx

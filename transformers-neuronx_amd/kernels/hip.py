@@ -147,6 +147,7 @@ class HipOps:
         _code(dtype)
         self._bias_copies = {}
         self._landing, self._landing_turn = [None, None], 0
+        self._ints, self._ints_done, self._ints_turn = [None, None], [None, None], 0
 
     def _call(self, module: str, fn: str, *args):
         lib = library(module)
@@ -181,11 +182,32 @@ class HipOps:
         self._call("elementwise", "tnx_device_pointer", ctypes.c_void_p(host.data_ptr()), ctypes.byref(address))
         return host, address
 
-    def copy_ints(self, dst, pinned) -> None:
-        """`dst[:] = host` for what `pinned_ints` returned, by a kernel on the current stream."""
+    def copy_ints(self, dst, pinned, n=None) -> None:
+        """`dst[:n] = host[:n]` for what `pinned_ints` returned, by a kernel on the current stream."""
         host, address = pinned
-        _want(dst, "dst", torch.int32, (host.numel(),))
-        self._call("elementwise", "tnx_copy_ints", address, _ptr(dst), host.numel(), _stream())
+        n = host.numel() if n is None else n
+        _want(dst, "dst", torch.int32)
+        if n > host.numel() or n > dst.numel():
+            raise ValueError(f"copy_ints: {n} integers from {host.numel()} into {dst.numel()}")
+        self._call("elementwise", "tnx_copy_ints", address, _ptr(dst), n, _stream())
+
+    def send_ints(self, flat):
+        """A host array of int32 as a device tensor, through pinned memory and a copy kernel (two buffers
+        in turn; one is written again only when the copy that read it has run)."""
+        n = flat.size
+        self._ints_turn ^= 1
+        i = self._ints_turn
+        if self._ints[i] is None or self._ints[i][0].numel() < n:
+            self._ints[i] = self.pinned_ints(max(2 * n, 1024))
+        elif self._ints_done[i] is not None:
+            self._ints_done[i].synchronize()
+        self._ints[i][0].numpy()[:n] = flat
+        dst = torch.empty(n, dtype=torch.int32, device=self.device)
+        self.copy_ints(dst, self._ints[i], n)
+        if self._ints_done[i] is None:
+            self._ints_done[i] = torch.cuda.Event()
+        self._ints_done[i].record()
+        return dst
 
     def send_tokens(self, tokens, kept, ctx):
         """Leave the chosen tokens for the next step (`kept[slot]`, see `store_tokens`) and write them into

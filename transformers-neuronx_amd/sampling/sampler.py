@@ -26,7 +26,10 @@ class Sampler:
             raise ValueError(f"{m} logits rows for {len(params)} requests")
         banned = [p.eos_token_id if (p.ban_eos and p.eos_token_id is not None) else -1 for p in params]
         if any(b >= 0 for b in banned):
-            self.ops.ban_tokens(logits, torch.tensor(banned, dtype=torch.int32, device=self.device))
+            if hasattr(self.ops, "send_ints"):
+                self.ops.ban_tokens(logits, self.ops.send_ints(np.array(banned, dtype=np.int32)))
+            else:
+                self.ops.ban_tokens(logits, torch.tensor(banned, dtype=torch.int32, device=self.device))
         if all(p.greedy for p in params):
             return self.ops.argmax(logits)
         temp = np.array([0.0 if p.greedy else p.temperature for p in params], dtype=np.float32)
@@ -34,5 +37,19 @@ class Sampler:
         top_p = np.array([p.top_p for p in params], dtype=np.float32)
         seeds = np.array([p.seed for p in params], dtype=np.int64)
         counters = np.array(draws, dtype=np.int64)
+        if hasattr(self.ops, "send_ints"):
+            # one block of integers through pinned memory: nothing here waits for the device
+            m2 = m + (m & 1)                                  # the 64-bit pieces start at even places
+            flat = np.zeros(3 * m2 + 4 * m, dtype=np.int32)
+            flat[0:m] = temp.view(np.int32)
+            flat[m2:m2 + m] = top_k
+            flat[2 * m2:2 * m2 + m] = top_p.view(np.int32)
+            flat[3 * m2:3 * m2 + 2 * m] = seeds.view(np.int32)
+            flat[3 * m2 + 2 * m:] = counters.view(np.int32)
+            dev = self.ops.send_ints(flat)
+            return self.ops.sample(logits, dev[0:m].view(torch.float32), dev[m2:m2 + m],
+                                   dev[2 * m2:2 * m2 + m].view(torch.float32),
+                                   dev[3 * m2:3 * m2 + 2 * m].view(torch.int64),
+                                   dev[3 * m2 + 2 * m:].view(torch.int64))
         dev = lambda a: torch.from_numpy(a).to(self.device)  # noqa: E731
         return self.ops.sample(logits, dev(temp), dev(top_k), dev(top_p), dev(seeds), dev(counters)).to(self.device)
