@@ -54,6 +54,11 @@ def test_step_refuses_what_it_cannot_run(tiny_folders):
     runner, _ = _runner(folder, 64)
     with pytest.raises(ValueError, match="vocabulary"):
         runner.step([StepEntry("a", [5, 512], [0])])
+    with pytest.raises(ValueError, match="vocabulary"):
+        runner.step([StepEntry("a", [5, -1], [0])])       # only the engine may name a token kept on the device
+    with pytest.raises(ValueError, match="vocabulary"):
+        LLMEngine(runner, EngineConfig(dtype="float32", kernels="reference", device="cpu")).add_request(
+            [3, -2], SamplingParams(max_new_tokens=2))
     with pytest.raises(ValueError, match="twice"):
         runner.step([StepEntry("a", [5], [0]), StepEntry("a", [6], [0])])
     with pytest.raises(ValueError, match="outside"):

@@ -65,7 +65,10 @@ class LLMEngine:
         rid = req_id if req_id is not None else next(self._ids)
         if rid in self.requests and not self.requests[rid].finished:
             raise ValueError(f"request {rid!r} is already live")
-        req = Request(rid, [int(t) for t in prompt], params)
+        prompt = [int(t) for t in prompt]
+        if prompt and not 0 <= min(prompt) <= max(prompt) < self.runner.vocab:
+            raise ValueError(f"request {rid!r}: a token id of the prompt is outside the vocabulary of {self.runner.vocab}")
+        req = Request(rid, prompt, params)
         self.scheduler.add(req)
         self.requests[rid] = req
         return rid
@@ -89,7 +92,7 @@ class LLMEngine:
                 # drawn by the step before this one and not read yet: the device has it under the slot
                 toks = toks[:-1] + [-1 - self.runner.cache.slot_of(run.request.req_id)]
             entries.append(StepEntry(run.request.req_id, toks, [run.count - 1] if run.samples else []))
-        logits = self.runner.step(entries)
+        logits = self.runner.step(entries, kept_allowed=True)
         sampling = [r for r in runs if r.samples]
         sent = None
         if sampling:

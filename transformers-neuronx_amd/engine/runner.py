@@ -97,10 +97,12 @@ class ModelRunner:
         self._last_ctx: Optional[StepContext] = None
         self._staging = _Staging(ops) if hasattr(ops, "pinned_ints") else None
 
-    def prepare(self, entries: List[StepEntry], fixed_width: bool = False) -> PackedStep:
+    def prepare(self, entries: List[StepEntry], fixed_width: bool = False, kept_allowed: bool = False) -> PackedStep:
         """Admit new requests, get pages for the step's tokens, lay out the batch. With `fixed_width`
         the block tables are as wide as the longest request the model allows, so that every step of
-        the same batch size has the same layout."""
+        the same batch size has the same layout. With `kept_allowed` a token id -1 - slot stands for the
+        token kept on the device for that slot (`keep_tokens`); otherwise every id is a vocabulary entry."""
+        lowest = -self.kept_tokens.numel() if kept_allowed else 0
         seen = set()
         for e in entries:
             if e.req in seen:
@@ -109,7 +111,7 @@ class ModelRunner:
             if len(e.tokens) == 0:
                 raise ValueError(f"request {e.req!r} brings no tokens")
             lo, hi = min(e.tokens), max(e.tokens)
-            if lo < -self.kept_tokens.numel() or hi >= self.vocab:
+            if lo < lowest or hi >= self.vocab:
                 raise ValueError(f"request {e.req!r}: token id {lo if lo < 0 else hi} is outside the vocabulary "
                                  f"of {self.vocab}")
         for e in entries:
@@ -133,13 +135,13 @@ class ModelRunner:
         return pack_step(entries, cached, slots, tables, self.cache.page_size)
 
     @torch.no_grad()
-    def step(self, entries: List[StepEntry]) -> Optional[torch.Tensor]:
+    def step(self, entries: List[StepEntry], kept_allowed: bool = False) -> Optional[torch.Tensor]:
         """Logits float32 `[wanted, vocab]` in the order of the entries and of
         their `want`; None when nothing is wanted (the step still runs)."""
         if not entries:
             return None
         recordable = self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
-        packed = self.prepare(entries, fixed_width=recordable)
+        packed = self.prepare(entries, fixed_width=recordable, kept_allowed=kept_allowed)
         if recordable:
             key = packed.layout()
             rec = self._recorded.get(key)
