@@ -243,3 +243,39 @@ def run_toy_model(ops_kind, dtype, device, tol):
 
 def test_toy_parts_on_the_host():
     run_toy_model("reference", torch.float32, "cpu", 2e-5)
+
+
+def run_toy_routed_model(ops_kind, dtype, device, tol):
+    """A feed-forward that routes tokens to experts and a position encoding of another kind, both defined
+    in the tests, built and stepped under every way of cutting without a change to the framework."""
+    import toy_parts
+    from transformers_neuronx_amd.cache import CacheManager
+    from transformers_neuronx_amd.engine import DecoderModel, ModelRunner
+    from transformers_neuronx_amd.kernels import make_ops
+    from transformers_neuronx_amd.weights import TensorDict, random_tensors
+    spec = toy_parts.toy_spec_routed()
+    model = DecoderModel(spec)
+    assert not model.recordable                                 # toy parts do not claim to be replayable
+    tensors = random_tensors(model.param_decls(), spec.init_std, 5, torch.float32)
+    ops = make_ops(ops_kind, dtype, device)
+    model.load(TensorDict(tensors), ops, dtype, device)
+    runner = ModelRunner(model, CacheManager(model.cache_needs(), 16, 12, 4, dtype, device), ops, use_graphs=True)
+    requests = _requests(211, [70, 33, 100], 9)
+    expected = {rid: toy_parts.toy_routed_plain_logits(tensors, toks) for rid, toks in requests.items()}
+    for steps, place in (schedules.whole(requests), schedules.portions(requests),
+                         schedules.mixed(requests, max_tokens=192, page=16, seed=2, tail=8, max_live=3)):
+        for rec in steps:
+            logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in rec["entries"]])
+            for row in range(logits.shape[0]):
+                rid, pos = place[(rec["step"], row)]
+                want = expected[rid][pos]
+                err = float((logits[row].cpu() - want).abs().max() / want.abs().max())
+                assert err < tol, (rec["step"], rid, pos, err)
+            for rid in rec["end"]:
+                runner.finish(rid)
+            runner.cache.check()
+        assert not runner.cache.requests
+
+
+def test_toy_routed_parts_on_the_host():
+    run_toy_routed_model("reference", torch.float32, "cpu", 2e-5)

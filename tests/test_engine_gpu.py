@@ -156,6 +156,13 @@ def test_toy_parts_on_the_gpu(dtype):
     run_toy_model("hip", dtype, DEV, 2e-5 if dtype == torch.float32 else 3e-2)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_toy_routed_parts_on_the_gpu(dtype):
+    """A routed feed-forward and another position encoding, defined in the tests, on the HIP backend."""
+    from test_engine_cpu import run_toy_routed_model
+    run_toy_routed_model("hip", dtype, DEV, 2e-5 if dtype == torch.float32 else 3e-2)
+
+
 def test_trace_run_as_a_program(tiny_folders, tmp_path):
     import subprocess
     import sys

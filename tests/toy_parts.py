@@ -121,3 +121,114 @@ def toy_plain_logits(w, tokens, width=64, heads=4, window=24, eps=1e-5):
             x = x + attn(h, p, kv=kv_of_first["kv"])
         x = x + ffn(ln(x, p + "norm2"), p)
     return plain_opt.linear(ln(x, "final_norm"), w["head.weight"])
+
+
+# ---------------------------------------------------------------- a routed feed-forward, another position encoding
+
+from transformers_neuronx_amd.parts import FeedForward, PositionEncoding, register_feed_forward, register_position  # noqa: E402
+
+
+@register_feed_forward("toy_routed")
+class ToyRoutedFeedForward(FeedForward):
+    """Every token goes to the one expert its router names: y = p_e * W2_e relu(W1_e h), e = argmax of the
+    router's logits (float32), p_e its softmax probability. Written with torch indexing: a toy."""
+
+    def __init__(self, width: int, inner: int, experts: int):
+        self.width, self.inner, self.experts = width, inner, experts
+
+    def param_decls(self, prefix):
+        d = [ParamDecl(prefix + "router.weight", (self.experts, self.width), "norm")]      # kept in float32
+        for e in range(self.experts):
+            d += [ParamDecl(f"{prefix}experts.{e}.up.weight", (self.inner, self.width)),
+                  ParamDecl(f"{prefix}experts.{e}.down.weight", (self.width, self.inner))]
+        return d
+
+    def load(self, tensors, prefix, ops, dtype):
+        super().load(tensors, prefix, ops, dtype)
+        self.router = tensors[prefix + "router.weight"].float()
+        self.up = [tensors[f"{prefix}experts.{e}.up.weight"] for e in range(self.experts)]
+        self.down = [tensors[f"{prefix}experts.{e}.down.weight"] for e in range(self.experts)]
+
+    def forward(self, h, ctx, residual):
+        probs = torch.softmax(h.float() @ self.router.t(), dim=-1)
+        weight, choice = probs.max(dim=-1)
+        out = residual.clone()
+        for e in range(self.experts):
+            rows = torch.nonzero(choice == e).flatten()
+            if rows.numel():
+                mid = self.ops.linear(h[rows].contiguous(), self.up[e], None, act="relu")
+                y = self.ops.linear(mid, self.down[e], None, out_f32=True)
+                out[rows] += weight[rows, None] * y
+        return out
+
+
+@register_position("toy_sinusoid")
+class ToySinusoid(PositionEncoding):
+    """Fixed sines and cosines of the position, added to the embedded tokens; no parameters."""
+
+    def __init__(self, width: int, base: float):
+        self.width, self.base = width, base
+
+    def at_input(self, x, positions, want_compute):
+        half = self.width // 2
+        freq = self.base ** (-torch.arange(half, device=x.device, dtype=torch.float32) / half)
+        angle = positions.float()[:, None] * freq[None, :]
+        out = x.float() + torch.cat([torch.sin(angle), torch.cos(angle)], dim=-1)
+        return out, (out.to(self.dtype) if want_compute else None)
+
+
+def toy_spec_routed(width=48, heads=3, inner=40, experts=3, vocab=211, positions=140, eps=1e-4, base=50.0):
+    """Two layers: attention with a routed feed-forward (norms after each half), attention with a dense
+    one (norms before); sinusoid positions; no norm before the head."""
+    hs = width // heads
+    norm = PartSpec("layer_norm", dict(width=width, eps=eps, affine=True))
+    attention = PartSpec("attention", dict(width=width, num_heads=heads, head_size=hs))
+    routed = PartSpec("toy_routed", dict(width=width, inner=inner, experts=experts))
+    dense = PartSpec("dense", dict(width=width, inner=2 * inner, activation="relu", bias=False))
+
+    def layer(i, ffn, block):
+        return LayerSpec(prefix=f"layers.{i}.", block=block, mixer=attention, feed_forward=ffn, mixer_norm=norm,
+                         feed_forward_norm=norm, mixer_name="mix.", feed_forward_name="ffn.",
+                         mixer_norm_name="norm1", feed_forward_norm_name="norm2")
+    embedding = PartSpec("token_table", dict(
+        vocab=vocab, embed_width=width, width=width, position=PartSpec("toy_sinusoid", dict(width=width, base=base)),
+        table_name="embed.weight", projection_name=None, position_name="positions"))
+    head = PartSpec("vocab_projection", dict(vocab=vocab, embed_width=width, width=width, norm=None,
+                                             weight_name="head.weight", tied_to="embed.weight",
+                                             projection_name=None, norm_name="final_norm"))
+    return ModelSpec(hidden_size=width, vocab_size=vocab, max_positions=positions, embedding=embedding,
+                     layers=(layer(0, routed, "post_norm"), layer(1, dense, "pre_norm")),
+                     schedule=(LayerCall(0), LayerCall(1)), head=head, init_std=0.1)
+
+
+def toy_routed_plain_logits(w, tokens, width=48, heads=3, experts=3, eps=1e-4, base=50.0):
+    w = {k: v.float() for k, v in w.items()}
+    n, half = len(tokens), width // 2
+    freq = base ** (-torch.arange(half, dtype=torch.float32) / half)
+    angle = torch.arange(n, dtype=torch.float32)[:, None] * freq[None, :]
+    x = w["embed.weight"][torch.tensor(tokens)] + torch.cat([torch.sin(angle), torch.cos(angle)], dim=-1)
+
+    def ln(t, name):
+        return plain_opt.layer_norm(t, w[name + ".weight"], w[name + ".bias"], eps)
+
+    def attn(t, p):
+        q, k, v = (plain_opt.linear(t, w[f"{p}mix.{s}_proj.weight"], w[f"{p}mix.{s}_proj.bias"]) for s in "qkv")
+        c = plain_opt.causal_attention(q, k, v, heads)
+        return plain_opt.linear(c, w[p + "mix.out_proj.weight"], w[p + "mix.out_proj.bias"])
+
+    # layer 0: norms after each half, routed feed-forward
+    p = "layers.0."
+    x = ln(x + attn(x, p), p + "norm1")
+    probs = torch.softmax(x @ w[p + "ffn.router.weight"].t(), dim=-1)
+    y = torch.zeros_like(x)
+    for t in range(n):
+        e = int(probs[t].argmax())
+        mid = torch.relu(plain_opt.linear(x[t:t + 1], w[f"{p}ffn.experts.{e}.up.weight"]))
+        y[t] = probs[t, e] * plain_opt.linear(mid, w[f"{p}ffn.experts.{e}.down.weight"])[0]
+    x = ln(x + y, p + "norm2")
+    # layer 1: norms before each half, dense feed-forward without bias
+    p = "layers.1."
+    x = x + attn(ln(x, p + "norm1"), p)
+    h = torch.relu(plain_opt.linear(ln(x, p + "norm2"), w[p + "ffn.fc1.weight"]))
+    x = x + plain_opt.linear(h, w[p + "ffn.fc2.weight"])
+    return plain_opt.linear(x, w["embed.weight"])
