@@ -58,6 +58,7 @@ def write_random_model(config, folder: str, seed: int, dtype=None) -> str:
     raw["torch_dtype"] = {v: k for k, v in _STORAGE.items()}[dtype]
     with open(os.path.join(folder, "config.json"), "w") as fp:
         json.dump(raw, fp, indent=2)
-    save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(folder, "model.safetensors"),
-              metadata={"format": "pt"})
+    path = os.path.join(folder, "model.safetensors")
+    save_file({k: v.contiguous() for k, v in tensors.items()}, path, metadata={"format": "pt"})
+    os.chmod(path, 0o644)      # the writer leaves it readable by its owner alone; a model folder is for others too
     return folder
