@@ -211,14 +211,14 @@ def filter_top_k_top_p(scores, top_k=None, top_p=None, min_tokens_to_keep=1):
     return values, indices
 
 
-def sample_row(scores, u, top_k=None, top_p=None, temperature=1.0):
+def sample_row(scores, u, top_k=None, top_p=None, temperature=1.0, min_tokens_to_keep=1):
     """sampling.py:337-345: divide by the temperature, filter, softmax over what
     is kept in float (:343), draw one. The draw is by inverse CDF with a given
     uniform `u` in [0, 1) over the kept tokens in ascending order of token id
     (hlo.py:2422-2467 draws by counting `u > cumsum / total` too); the reference's
     host loop uses `torch.multinomial`, whose stream cannot be reproduced, so
     only the distribution is comparable with it."""
-    values, indices = filter_top_k_top_p(scores.float() / temperature, top_k, top_p)
+    values, indices = filter_top_k_top_p(scores.float() / temperature, top_k, top_p, min_tokens_to_keep)
     order = torch.argsort(indices)
     values, indices = values[order], indices[order]
     probs = torch.softmax(values.double(), dim=-1)

@@ -166,6 +166,31 @@ def test_sampled_tokens_follow_the_plain_sampler(tiny_folders):
         toks.append(tok)
 
 
+def test_generation_config_options(tiny_folders):
+    """`GenerationConfig` as the reference's on-device generation reads it (config.py:106-139): a value a
+    batch line, a global top-k above the lines' own, a least number of tokens for top-p, and the constant
+    0.5 in place of random numbers."""
+    from transformers_neuronx_amd import OPTForSampling
+    from transformers_neuronx_amd.config import GenerationConfig
+    folder, cfg, weights = tiny_folders["A"]
+    prompt = _requests(cfg["vocab_size"], [9], 6)["r0"]
+    model = OPTForSampling.from_pretrained(folder, batch_size=3, amp="f32", n_positions=32, kernels="reference",
+                                           device="cpu").load()
+    gen = GenerationConfig(do_sample=True, top_k=[1, 30, 0], top_p=[1.0, 0.02, 0.5], temperature=[1.0, 0.9, 1.4],
+                           top_p_min_tokens=[1, 5, 2], global_top_k=20, deterministic=True, per_batch_line=True,
+                           dynamic=True)
+    out = model.sample(torch.tensor([prompt] * 3), sequence_length=15, generation_config=gen)
+    for b, (k, p, t, least) in enumerate([(1, 1.0, 1.0, 1), (20, 0.02, 0.9, 5), (20, 0.5, 1.4, 2)]):
+        toks = list(prompt)
+        for n in range(6):
+            logits = plain_opt.forward_logits(weights, cfg, toks)[-1]
+            tok = plain_opt.sample_row(logits, 0.5, top_k=k, top_p=p, temperature=t, min_tokens_to_keep=least)
+            assert int(out[b, len(toks)]) == tok, (b, n)
+            toks.append(tok)
+    # the second line is not greedy: five tokens stay and 0.5 falls past the first of them
+    assert out[1].tolist() != out[0].tolist()
+
+
 def test_entry_point_in_the_reference_manner(tiny_folders):
     from transformers_neuronx_amd import OPTForSampling
     folder, cfg, weights = tiny_folders["A"]

@@ -280,6 +280,22 @@ def test_argmax_and_sampling(vocab):
         t_h = hip.sample(logits, temp, top_k, top_p, seeds, counters)
         t_r = ref.sample(logits, temp, top_k, top_p, seeds, counters)
         assert (t_h == t_r).float().mean() >= 0.95, (t_h, t_r)    # a draw on a boundary may round either way
+    # never fewer than `min_keep` tokens, and the constant 0.5 in place of a random number (counter < 0)
+    least = torch.tensor([1, 3, 40, 7] * 6, device=DEV, dtype=torch.int32)
+    tight_p = torch.full((rows,), 0.01, device=DEV)             # top-p alone would keep one token
+    fixed = torch.full((rows,), -1, device=DEV, dtype=torch.int64)
+    t_h = hip.sample(logits, temp, top_k, tight_p, seeds, fixed, least)
+    t_r = ref.sample(logits, temp, top_k, tight_p, seeds, fixed, least)
+    assert (t_h == t_r).float().mean() >= 0.95, (t_h, t_r)
+    for step in range(4):
+        counters = torch.full((rows,), step, device=DEV, dtype=torch.int64)
+        t_h = hip.sample(logits, temp, top_k, tight_p, seeds, counters, least)
+        t_r = ref.sample(logits, temp, top_k, tight_p, seeds, counters, least)
+        assert (t_h == t_r).float().mean() >= 0.95, (t_h, t_r)
+        # a row that keeps 40 tokens does draw others than the best one
+    picks = torch.stack([hip.sample(logits, temp, top_k, tight_p, seeds,
+                                    torch.full((rows,), s, device=DEV, dtype=torch.int64), least) for s in range(12)])
+    assert len(set(picks[:, 2].tolist())) > 1 and len(set(picks[:, 4].tolist())) == 1
 
 
 def test_sampling_distribution():

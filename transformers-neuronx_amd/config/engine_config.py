@@ -75,8 +75,10 @@ class GenerationConfig:
     per_batch_line: bool = False
 
     def __post_init__(self):
-        self.top_p = float(self.top_p)
-        self.temperature = float(self.temperature)
+        # a list gives every batch line its own value (`per_batch_line`)
+        self.top_p = [float(p) for p in self.top_p] if isinstance(self.top_p, (list, tuple)) else float(self.top_p)
+        self.temperature = ([float(t) for t in self.temperature] if isinstance(self.temperature, (list, tuple))
+                            else float(self.temperature))
 
 
 @dataclass

@@ -119,7 +119,8 @@ extern "C" int tnx_ban_tokens(float* logits, const int* token, int rows, int voc
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature, const int* __restrict__ top_k,
               const float* __restrict__ top_p, const long long* __restrict__ seeds,
-              const long long* __restrict__ counters, int* __restrict__ out, int vocab) {
+              const long long* __restrict__ counters, const int* __restrict__ min_keep, int* __restrict__ out,
+              int vocab) {
   __shared__ unsigned int cnt[256];
   __shared__ float mass[256];
   __shared__ float part[SAMPLE_THREADS];
@@ -158,12 +159,10 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
   const float inv_temp = 1.f / temp;
   const float xmax = row[arg] * inv_temp;
 
-  // top-k: the k-th largest key
-  uint64_t floor_key = 0;  // tokens with key >= floor_key are kept
-  const int k = top_k[rowi];
-  if (k > 0 && k < vocab) {
+  // the k-th largest key of the row, by radix selection; every thread of the block calls it together
+  auto kth_largest = [&](unsigned int k) -> uint64_t {
     uint64_t prefix = 0, mask = 0;
-    unsigned int remaining = (unsigned int)k;
+    unsigned int remaining = k;
     for (int pass = 0; pass < 8; ++pass) {
       const int shift = 56 - 8 * pass;
       if (tid < 256) cnt[tid] = 0;
@@ -192,8 +191,15 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
       __syncthreads();
       if (whole_bin) break;  // everything under this prefix is kept: the threshold is the prefix itself
     }
-    floor_key = prefix;
-  }
+    return prefix;
+  };
+
+  // top-k: tokens with key >= floor_key are kept; never fewer than `min_keep` (sampling.py:204-205)
+  uint64_t floor_key = 0;
+  const int keep = min_keep ? max(min_keep[rowi], 1) : 1;
+  int k = top_k[rowi];
+  if (k > 0) k = max(k, keep);
+  if (k > 0 && k < vocab) floor_key = kth_largest((unsigned int)k);
 
   // top-p: the smallest kept key is the last one whose predecessors hold less than p of the mass
   const float p = top_p[rowi];
@@ -250,7 +256,15 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
       __syncthreads();
       if (single) break;
     }
-    floor_key = prefix > floor_key ? prefix : floor_key;
+    uint64_t by_mass = prefix > floor_key ? prefix : floor_key;
+    if (keep > 1) {
+      // at least `keep` tokens stay, the largest ones (sampling.py:232): the floor is no higher than the
+      // keep-th largest key, and no lower than what top-k left
+      const uint64_t nth = keep < vocab ? kth_largest((unsigned int)keep) : 0;
+      const uint64_t least = nth > floor_key ? nth : floor_key;
+      by_mass = by_mass < least ? by_mass : least;
+    }
+    floor_key = by_mass;
   }
 
   // the draw, over the kept tokens in ascending order of token id; thread t owns a contiguous segment
@@ -291,7 +305,8 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     if (lane == 63) sh_total = incl;
   }
   __syncthreads();
-  const float u = philox_uniform((uint64_t)seeds[rowi], (uint64_t)counters[rowi]);
+  // a counter below zero asks for the constant 0.5 the reference calls deterministic (hlo.py:2455-2456)
+  const float u = counters[rowi] < 0 ? 0.5f : philox_uniform((uint64_t)seeds[rowi], (uint64_t)counters[rowi]);
   const float goal = u * sh_total;
   // thread t owns [base_t, base_{t+1}): the scanned values tile the line without gaps
   const float base = part[tid];
@@ -314,11 +329,12 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
 }
 
 extern "C" int tnx_sample(const float* logits, const float* temperature, const int* top_k, const float* top_p,
-                          const long long* seeds, const long long* counters, int* out, int rows, int vocab,
-                          hipStream_t stream) {
+                          const long long* seeds, const long long* counters, const int* min_keep, int* out,
+                          int rows, int vocab, hipStream_t stream) {
   TNX_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
   if (rows == 0) return 0;
-  sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, temperature, top_k, top_p, seeds, counters, out, vocab);
+  sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, temperature, top_k, top_p, seeds, counters, min_keep,
+                                                     out, vocab);
   TNX_CHECK_LAUNCH("sample");
   return 0;
 }

@@ -57,8 +57,8 @@ _SIGNATURES = {
         "tnx_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
         "tnx_store_tokens": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p,
                              _c_void_p],
-        "tnx_sample": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
-                       _c_void_p],
+        "tnx_sample": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
+                       _c_int, _c_void_p],
     },
 }
 
@@ -502,7 +502,8 @@ class HipOps:
         self._call("sampling", "tnx_argmax", _ptr(logits), _ptr(out), logits.shape[0], logits.shape[1], _stream())
         return out
 
-    def sample(self, logits, temperature, top_k, top_p, seeds, counters):
+    def sample(self, logits, temperature, top_k, top_p, seeds, counters, min_keep=None):
+        """See `ReferenceOps.sample`."""
         _want(logits, "logits", torch.float32)
         m = logits.shape[0]
         _want(temperature, "temperature", torch.float32, (m,))
@@ -510,9 +511,11 @@ class HipOps:
         _want(top_p, "top_p", torch.float32, (m,))
         _want(seeds, "seeds", torch.int64, (m,))
         _want(counters, "counters", torch.int64, (m,))
+        if min_keep is not None:
+            _want(min_keep, "min_keep", torch.int32, (m,))
         out = torch.empty(m, dtype=torch.int32, device=logits.device)
         self._call("sampling", "tnx_sample", _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(seeds),
-                   _ptr(counters), _ptr(out), m, logits.shape[1], _stream())
+                   _ptr(counters), _ptr(min_keep), _ptr(out), m, logits.shape[1], _stream())
         return out
 
     def synchronize(self):

@@ -184,13 +184,15 @@ class ReferenceOps:
     def argmax(self, logits):
         return logits.argmax(dim=-1).to(torch.int32)
 
-    def sample(self, logits, temperature, top_k, top_p, seeds, counters):
+    def sample(self, logits, temperature, top_k, top_p, seeds, counters, min_keep=None):
         """One token per row. Row i: logits / temperature[i]; the top_k[i] largest
         are kept (0 keeps all; ties go to the lower token id); of these, in
         descending order, the shortest prefix whose softmax mass reaches
-        top_p[i] (>= 1 keeps all); the draw is by inverse CDF over the kept
+        top_p[i] (>= 1 keeps all); neither keeps fewer than min_keep[i] tokens
+        (1 if not given); the draw is by inverse CDF over the kept
         tokens in ascending order of token id with the uniform number
-        `philox_uniform(seeds[i], counters[i])`. temperature 0 is argmax."""
+        `philox_uniform(seeds[i], counters[i])`, or 0.5 for a counter below zero.
+        temperature 0 is argmax."""
         m, v = logits.shape
         out = torch.empty(m, dtype=torch.int32)
         for i in range(m):
@@ -201,19 +203,23 @@ class ReferenceOps:
                 continue
             row = row / temp
             values, indices = torch.sort(row, descending=True, stable=True)
+            least = max(1, int(min_keep[i])) if min_keep is not None else 1
             k = int(top_k[i])
+            if k > 0:
+                k = max(k, least)
             if 0 < k < v:
                 values, indices = values[:k], indices[:k]
             p = float(top_p[i])
             if p < 1.0:
                 cum = torch.cumsum(torch.softmax(values, -1, dtype=torch.float32), -1)
                 keep = torch.cat([torch.ones(1, dtype=torch.bool), (cum < p)[:-1]])
+                keep[:least] = True
                 values, indices = values[keep], indices[keep]
             order = torch.argsort(indices)
             values, indices = values[order], indices[order]
             w = torch.exp(values - values.max()).double()
             cum = torch.cumsum(w, -1)
-            u = philox_uniform(int(seeds[i]), int(counters[i]))
+            u = 0.5 if int(counters[i]) < 0 else philox_uniform(int(seeds[i]), int(counters[i]))
             pick = int((cum <= u * float(cum[-1])).sum())
             out[i] = int(indices[min(pick, len(indices) - 1)])
         return out.to(logits.device)

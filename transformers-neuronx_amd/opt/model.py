@@ -167,8 +167,17 @@ class OPTForSampling:
         for b, toks in enumerate(rows):
             new = sequence_length - width
             if gen is not None:
-                p = SamplingParams(max_new_tokens=new, do_sample=gen.do_sample, temperature=gen.temperature,
-                                   top_k=gen.top_k, top_p=gen.top_p, seed=seed + b,
+                # config.py:106-139: values may be lists, one entry a batch line (`per_batch_line`); a global
+                # top-k caps every line's own (layers/generation.py:55-56); `dynamic` needs nothing here,
+                # every request carries its own options anyway
+                def line(v):
+                    return v[b] if isinstance(v, (list, tuple)) else v
+                k = int(line(gen.top_k))
+                if gen.global_top_k is not None:
+                    k = min(k, int(gen.global_top_k)) if k > 0 else int(gen.global_top_k)
+                p = SamplingParams(max_new_tokens=new, do_sample=gen.do_sample, temperature=float(line(gen.temperature)),
+                                   top_k=k, top_p=float(line(gen.top_p)), seed=seed + b,
+                                   min_tokens_to_keep=int(line(gen.top_p_min_tokens)), deterministic=gen.deterministic,
                                    eos_token_id=gen.eos_token_id, ignore_eos=gen.eos_token_id is None)
             else:
                 p = SamplingParams(max_new_tokens=new, do_sample=True, temperature=temperature, top_k=top_k,

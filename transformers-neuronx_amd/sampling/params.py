@@ -14,8 +14,11 @@ class SamplingParams:
     top_k        the k largest logits are kept (:151, :210-211); 0 keeps all
     top_p        of those, the shortest prefix in descending order whose softmax mass
                  reaches top_p (:213-249); 1.0 keeps all
+    min_tokens_to_keep  neither filter leaves fewer tokens than this (:204-205, :232;
+                 `top_p_min_tokens` of the `GenerationConfig`)
     seed         the request's own random stream: draw number n of the request uses the
                  counter n, whatever else is in the batch
+    deterministic  every draw uses 0.5 in place of a random number (hlo.py:2455-2456)
     ban_eos      the end-of-sequence token is never chosen (`scores[:, eos] = -inf`,
                  sampling.py:143-144, the OPT loop's behaviour)
     ignore_eos   generation does not stop at the end-of-sequence token
@@ -27,6 +30,8 @@ class SamplingParams:
     top_k: int = 0
     top_p: float = 1.0
     seed: int = 0
+    min_tokens_to_keep: int = 1
+    deterministic: bool = False
     eos_token_id: Optional[int] = None
     ban_eos: bool = False
     ignore_eos: bool = False
@@ -38,6 +43,8 @@ class SamplingParams:
             raise ValueError("top_k has to be a non-negative int (0 keeps all tokens).")
         if not 0.0 < float(self.top_p) <= 1.0:
             raise ValueError("top_p has to be a strictly positive float that less than or equal to 1.0.")
+        if not isinstance(self.min_tokens_to_keep, int) or self.min_tokens_to_keep < 1:
+            raise ValueError("min_tokens_to_keep has to be a positive int.")
         if float(self.temperature) < 0:
             raise ValueError("temperature has to be a non-negative float (0 is greedy).")
 

@@ -36,20 +36,23 @@ class Sampler:
         top_k = np.array([p.top_k for p in params], dtype=np.int32)
         top_p = np.array([p.top_p for p in params], dtype=np.float32)
         seeds = np.array([p.seed for p in params], dtype=np.int64)
-        counters = np.array(draws, dtype=np.int64)
+        counters = np.array([-1 if p.deterministic else n for p, n in zip(params, draws)], dtype=np.int64)
+        least = np.array([p.min_tokens_to_keep for p in params], dtype=np.int32)
         if hasattr(self.ops, "send_ints"):
             # one block of integers through pinned memory: nothing here waits for the device
             m2 = m + (m & 1)                                  # the 64-bit pieces start at even places
-            flat = np.zeros(3 * m2 + 4 * m, dtype=np.int32)
+            flat = np.zeros(3 * m2 + 5 * m, dtype=np.int32)
             flat[0:m] = temp.view(np.int32)
             flat[m2:m2 + m] = top_k
             flat[2 * m2:2 * m2 + m] = top_p.view(np.int32)
             flat[3 * m2:3 * m2 + 2 * m] = seeds.view(np.int32)
-            flat[3 * m2 + 2 * m:] = counters.view(np.int32)
+            flat[3 * m2 + 2 * m:3 * m2 + 4 * m] = counters.view(np.int32)
+            flat[3 * m2 + 4 * m:] = least
             dev = self.ops.send_ints(flat)
             return self.ops.sample(logits, dev[0:m].view(torch.float32), dev[m2:m2 + m],
                                    dev[2 * m2:2 * m2 + m].view(torch.float32),
                                    dev[3 * m2:3 * m2 + 2 * m].view(torch.int64),
-                                   dev[3 * m2 + 2 * m:].view(torch.int64))
+                                   dev[3 * m2 + 2 * m:3 * m2 + 4 * m].view(torch.int64), dev[3 * m2 + 4 * m:])
         dev = lambda a: torch.from_numpy(a).to(self.device)  # noqa: E731
-        return self.ops.sample(logits, dev(temp), dev(top_k), dev(top_p), dev(seeds), dev(counters)).to(self.device)
+        return self.ops.sample(logits, dev(temp), dev(top_k), dev(top_p), dev(seeds), dev(counters),
+                               dev(least)).to(self.device)
