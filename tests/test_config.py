@@ -81,6 +81,17 @@ def test_engine_config():
     assert NeuronConfig(continuous_batching=cb).continuous_batching.num_blocks == 10
     with pytest.raises(ValueError, match="float32"):
         NeuronConfig(cast_logits_dtype="bfloat16")
+    # the reference's other keywords (config.py:206-363): layouts and fusions are taken and change nothing,
+    # what would change the result and has no counterpart is refused, a name it does not have is an error
+    nc = NeuronConfig(attention_layout="BSH", fuse_qkv=True, weight_tiling=True, compilation_worker_count=4,
+                      sequence_parallel_norm=True, output_all_logits=True)
+    assert nc.fuse_qkv and nc.attention_layout == "BSH" and nc.output_all_logits and nc.quant is None
+    for bad in (dict(quant=object()), dict(log_softmax_scores=True), dict(group_query_attention="shard-over-heads"),
+                dict(is_eagle_draft=True), dict(has_pre_attention_norm=False)):
+        with pytest.raises(ValueError, match="no counterpart"):
+            NeuronConfig(**bad)
+    with pytest.raises(TypeError, match="unknown"):
+        NeuronConfig(no_such_switch=1)
 
 
 def test_sequence_length_guard():

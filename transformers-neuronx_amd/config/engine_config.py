@@ -81,30 +81,56 @@ class GenerationConfig:
                             else float(self.temperature))
 
 
-@dataclass
 class NeuronConfig:
-    """The switches of config.py:206-363 that mean something on one GPU.
+    """The reference's bag of switches (config.py:206-363), by its keyword names.
 
-    `continuous_batching` sizes the scheduler and the cache,
-    `on_device_generation` makes `sample` draw with these generation options,
-    `cast_logits_dtype` is always float32 here, `output_all_logits` makes
-    `forward` return the logits of every position. Other keywords of the
-    reference (tensor parallel layouts, quantization, compiler options) are
-    accepted and ignored when they are left at their defaults, and refused with
-    a clear message otherwise."""
-    continuous_batching: Optional[ContinuousBatchingConfig] = None
-    on_device_generation: Optional[GenerationConfig] = None
-    on_device_embedding: bool = True
-    cast_logits_dtype: str = "float32"
-    output_all_logits: bool = False
-    fuse_qkv: bool = True
-    padding_side: str = "left"
+    What means something on one GPU is kept: `continuous_batching` sizes the scheduler and the cache,
+    `on_device_generation` makes `sample` draw with these generation options, `output_all_logits` makes
+    `forward` return the logits of every position, `cast_logits_dtype` is always float32 here,
+    `padding_side` and `on_device_embedding` are recorded. Switches that only choose a layout, a fusion or
+    a way of splitting work over devices are taken and change nothing (the kernels have their own
+    layouts; there is one device). Switches that would change what is computed and have no counterpart
+    here (quantization, sparse attention, grouped queries for OPT, speculative heads, log-softmax scores)
+    are refused unless left at the reference's default."""
 
-    def __post_init__(self):
-        if isinstance(self.continuous_batching, dict):
-            self.continuous_batching = ContinuousBatchingConfig(**self.continuous_batching)
-        if self.cast_logits_dtype != "float32":
+    # keyword -> the reference's default; any value is taken and ignored
+    _NO_EFFECT = dict(attention_layout="HSB", collectives_layout="HSB", cache_layout="SBH", fuse_qkv=False,
+                      fuse_mlp=False, qkv_tiling=False, weight_tiling=False,
+                      mlp_in_weight_tiling_permute_order=[1, 2, 0, 3], mlp_out_weight_tiling_permute_order=[1, 2, 0, 3],
+                      sequence_parallel_norm=False, sequence_parallel_norm_threshold=2048, all_reduce_dtype=None,
+                      attn_output_transposed=False, mlp_out_weight_transpose=False, compilation_worker_count=None,
+                      duplicate_q_weight_sos=False, use_2d_cache_ids=False, lhs_aligned=False)
+    # keyword -> the only value taken
+    _REFUSED = dict(sparse_attn=None, quant=None, kv_cache_quant=None, group_query_attention=None,
+                    bf16_rms_norm=False, log_softmax_scores=False, shard_over_sequence=False,
+                    fused_rmsnorm_qkv=False, fused_rmsnorm_mlp=False, is_eagle_target=False, is_eagle_draft=False,
+                    has_pre_attention_norm=True)
+
+    def __init__(self, *, continuous_batching=None, on_device_generation=None, on_device_embedding: bool = True,
+                 cast_logits_dtype: str = "float32", output_all_logits: bool = False, padding_side: str = "left",
+                 **kwargs):
+        if isinstance(continuous_batching, dict):
+            continuous_batching = ContinuousBatchingConfig(**continuous_batching)
+        if cast_logits_dtype != "float32":
             raise ValueError("logits are returned in float32; cast_logits_dtype must be 'float32'")
+        if padding_side not in ("left", "right"):
+            raise ValueError(f"padding_side must be 'left' or 'right', got {padding_side!r}")
+        self.continuous_batching: Optional[ContinuousBatchingConfig] = continuous_batching
+        self.on_device_generation: Optional[GenerationConfig] = on_device_generation
+        self.on_device_embedding = on_device_embedding
+        self.cast_logits_dtype = cast_logits_dtype
+        self.output_all_logits = output_all_logits
+        self.padding_side = padding_side
+        for name, default in self._NO_EFFECT.items():
+            setattr(self, name, kwargs.pop(name, default))
+        for name, only in self._REFUSED.items():
+            value = kwargs.pop(name, only)
+            if value != only:
+                raise ValueError(f"NeuronConfig({name}={value!r}) has no counterpart in this engine; "
+                                 f"leave it at {only!r}")
+            setattr(self, name, value)
+        if kwargs:
+            raise TypeError(f"NeuronConfig got unknown keywords {sorted(kwargs)}")
 
 
 @dataclass
