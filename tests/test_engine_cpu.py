@@ -191,14 +191,17 @@ def test_generation_config_options(tiny_folders):
     assert out[1].tolist() != out[0].tolist()
 
 
-def test_entry_point_in_the_reference_manner(tiny_folders):
+def test_entry_point_in_the_reference_manner(tiny_folders, tmp_path):
     from transformers_neuronx_amd import OPTForSampling
     folder, cfg, weights = tiny_folders["A"]
     model = OPTForSampling.from_pretrained(folder, batch_size=2, amp="f32", n_positions=48, kernels="reference",
                                            device="cpu", page_size=16)
     with pytest.raises(RuntimeError, match="load"):
         model.sample(torch.tensor([[5, 6]]), 8)
+    assert not model.is_compiled()
+    model.load(str(tmp_path))            # the reference's folder of compiled artifacts: nothing to take from it
     model.to_neuron()
+    assert model.is_compiled()
     ids = torch.tensor([[5, 9, 200, 31], [7, 7, 100, 3]])
     out = model.sample(ids, sequence_length=12, top_k=1)
     assert out.shape == (2, 12) and torch.equal(out[:, :4], ids)
@@ -223,6 +226,11 @@ def test_entry_point_in_the_reference_manner(tiny_folders):
     torch.testing.assert_close(logits[0], plain_opt.forward_logits(weights, cfg, [5, 9])[-1], atol=1e-5, rtol=1e-5)
     model.reset()
     assert not model.engine.runner.cache.requests
+    # other generation options from the next call on (base.py:761-766)
+    from transformers_neuronx_amd.config import GenerationConfig
+    model.update_generation_config(GenerationConfig(do_sample=False))
+    out = model.sample(ids, sequence_length=12)
+    assert out[0].tolist() == plain_opt.greedy(weights, cfg, ids[0].tolist(), 8)
 
 
 def _toy_model(ops_kind, dtype, device):

@@ -148,6 +148,18 @@ def test_greedy_generation_through_the_entry_point(tiny_folders, amp):
     assert set(hip.loaded_libraries()) >= {"elementwise", "gemm", "attention", "sampling"}
 
 
+def test_save_notes_the_built_kernels(tiny_folders, tmp_path):
+    """`save` is the reference's way to keep what was compiled (base.py:39-48); here that is the kernels."""
+    from transformers_neuronx_amd import OPTForSampling
+    model = OPTForSampling.from_pretrained(tiny_folders["A"][0], batch_size=1, amp="bf16", n_positions=32).load()
+    model.save(str(tmp_path / "artifacts"))
+    noted = json.load(open(tmp_path / "artifacts" / "kernels.json"))
+    assert set(noted) == {"elementwise", "gemm", "attention", "sampling"} and all(os.path.exists(p) for p in noted.values())
+    again = OPTForSampling.from_pretrained(tiny_folders["A"][0], batch_size=1, amp="bf16", n_positions=32)
+    again.load(str(tmp_path / "artifacts")).to_neuron()
+    assert again.is_compiled() and again.sample(torch.tensor([[5, 6, 7]]), 6).shape == (1, 6)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_toy_parts_on_the_gpu(dtype):
     """A mixer with state of its own, registered by the test, beside full, windowed and cache-sharing

@@ -9,6 +9,7 @@ compiled and bucketed there (`tp_degree`, `unroll`, `context_length_estimate`)
 has no counterpart on one GPU: those arguments are accepted and, when they ask
 for something that does not exist here (more than one device), refused.
 """
+import os
 import warnings
 from typing import List, Optional, Sequence
 
@@ -86,13 +87,36 @@ class OPTForSampling:
     def load(self, directory: Optional[str] = None) -> "OPTForSampling":
         """Weights to the GPU, the page pool, the engine. (In the reference `load`
         points at precompiled artifacts, base.py:50-52, and `to_neuron` does the
-        work, base.py:77-89; here both names do the one thing there is to do.)"""
-        if directory is not None:
+        work, base.py:77-89; here both names do the one thing there is to do.)
+        `directory`: a model folder to read instead of the one given at construction; a folder without a
+        `config.json` is taken for the reference's folder of compiled artifacts (what `save` writes) and
+        changes nothing, since nothing is compiled ahead but the kernels."""
+        if directory is not None and os.path.exists(os.path.join(directory, "config.json")):
             self._folder = directory
+        if self.engine is not None:
+            return self
         source = self._source if self._source is not None else Checkpoint(self._folder)
         runner = build_runner(self.config, source, self.engine_config)
         self.engine = LLMEngine(runner, self.engine_config)
         return self
+
+    def save(self, directory: str) -> None:
+        """The reference stores its compiled programs here for a later `load` (base.py:39-48). The
+        counterpart of compiling is building the kernels: this builds those not built yet and notes
+        where they lie."""
+        import json
+        from ..kernels import build
+        os.makedirs(directory, exist_ok=True)
+        with open(os.path.join(directory, "kernels.json"), "w") as fp:
+            json.dump({m: build.compile_module(m) for m in build.MODULES}, fp, indent=1)
+
+    def is_compiled(self) -> bool:
+        """base.py:143-151: whether the model is ready to run."""
+        return self.engine is not None
+
+    def update_generation_config(self, generation_config: GenerationConfig) -> None:
+        """base.py:761-766: other generation options from the next `sample` on."""
+        self.neuron_config.on_device_generation = generation_config
 
     to_neuron = load
 
