@@ -100,3 +100,24 @@ def test_sequence_length_guard():
         OPTForSampling(OPTConfig.from_dict(TINY_A), n_positions=129, amp="f32")
     with pytest.raises(ValueError, match="one GPU"):
         OPTForSampling(OPTConfig.from_dict(TINY_A), n_positions=64, amp="f32", tp_degree=2)
+
+
+def test_auto_model_picks_the_class_the_folder_names(tmp_path):
+    """modeling_auto.py:30-47: the class comes from config.json; an unknown model is an AssertionError."""
+    import json
+    from transformers_neuronx_amd import NeuronAutoModelForCausalLM, OPTForSampling
+    from conftest import TINY_A
+    good = tmp_path / "good"
+    good.mkdir()
+    (good / "config.json").write_text(json.dumps(TINY_A))
+    model = NeuronAutoModelForCausalLM.from_pretrained(str(good), batch_size=2, amp="f32", n_positions=64,
+                                                       kernels="reference", device="cpu")
+    assert isinstance(model, OPTForSampling) and model.config.hidden_size == 64
+    by_type = dict(TINY_A, architectures=["SomethingElse"])
+    (good / "config.json").write_text(json.dumps(by_type))
+    assert isinstance(NeuronAutoModelForCausalLM.from_pretrained(str(good), amp="f32", n_positions=64), OPTForSampling)
+    bad = tmp_path / "bad"
+    bad.mkdir()
+    (bad / "config.json").write_text(json.dumps(dict(TINY_A, architectures=["LlamaForCausalLM"], model_type="llama")))
+    with pytest.raises(AssertionError, match="not supported"):
+        NeuronAutoModelForCausalLM.from_pretrained(str(bad))

@@ -10,6 +10,9 @@ def __getattr__(name):
     if name in ("OPTForSampling", "OPTForGreedySearch"):
         from .opt import model
         return getattr(model, name)
+    if name == "NeuronAutoModelForCausalLM":
+        from .modeling_auto import NeuronAutoModelForCausalLM
+        return NeuronAutoModelForCausalLM
     if name == "LLMEngine":
         from .engine.engine import LLMEngine
         return LLMEngine
