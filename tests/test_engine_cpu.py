@@ -226,6 +226,24 @@ def test_entry_point_in_the_reference_manner(tiny_folders, tmp_path):
     torch.testing.assert_close(logits[0], plain_opt.forward_logits(weights, cfg, [5, 9])[-1], atol=1e-5, rtol=1e-5)
     model.reset()
     assert not model.engine.runner.cache.requests
+    # a streamer gets one token of every row at a time and is told the end (sampling.py:159-160, :172-173),
+    # also when the rows' prompts differ in length and enter the cache in different steps
+    class Collect:
+        def __init__(self):
+            self.columns, self.ended = [], False
+
+        def put(self, tokens):
+            assert tokens.shape == (2, 1) and not self.ended
+            self.columns.append(tokens)
+
+        def end(self):
+            self.ended = True
+    model.engine.scheduler.max_num_batched_tokens = 3          # the two prompts cannot share a step
+    collect = Collect()
+    out = model.sample(padded, sequence_length=9, start_ids=torch.tensor([2, 0]), top_k=1, streamer=collect)
+    model.engine.scheduler.max_num_batched_tokens = 2048
+    assert collect.ended and torch.equal(torch.cat(collect.columns, dim=1), out[:, 4:])
+    assert out[0, 4:].tolist() == plain_opt.greedy(weights, cfg, [5, 9], 5)[2:]
     # other generation options from the next call on (base.py:761-766)
     from transformers_neuronx_amd.config import GenerationConfig
     model.update_generation_config(GenerationConfig(do_sample=False))

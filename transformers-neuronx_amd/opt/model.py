@@ -210,10 +210,21 @@ class OPTForSampling:
             params.append(p)
         engine.reset()
         ids = [engine.add_request(toks, p) for toks, p in zip(rows, params)]
+        column = 0              # generated tokens already handed to the streamer, the same for every row
         while engine.has_work:
-            outs = engine.step()
-            if streamer is not None and outs:
-                streamer.put(torch.tensor([[o.token] for o in outs]))
+            engine.step()
+            if streamer is None:
+                continue
+            # sampling.py:159-160 hands over one token of every row at a time, `[batch, 1]`: the next column
+            # goes out when every row has it or has ended (a row that ended repeats its last token's filler)
+            reqs = [engine.requests[i] for i in ids]
+            while column < sequence_length - width and all(
+                    (len(q.output) > column and q.output[column] >= 0) or (q.finished and len(q.output) <= column)
+                    for q in reqs):
+                streamer.put(torch.tensor([[q.output[column] if len(q.output) > column else
+                                            (p.eos_token_id if p.eos_token_id is not None else 0)]
+                                           for q, p in zip(reqs, params)], dtype=prompts.dtype))
+                column += 1
         if streamer is not None:
             streamer.end()
         result = torch.empty(len(rows), sequence_length, dtype=prompts.dtype)
