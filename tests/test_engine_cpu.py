@@ -166,6 +166,35 @@ def test_sampled_tokens_follow_the_plain_sampler(tiny_folders):
         toks.append(tok)
 
 
+def test_forward_by_sequence_ids(tiny_folders):
+    """With `continuous_batching` in the NeuronConfig `forward` is driven the way the reference's serving
+    integration drives it (base.py:575-637): prompts go in one at a time under their `seq_ids`, then the
+    sequences decode together, in any order, and a sequence id is used again for a new prompt."""
+    from transformers_neuronx_amd import OPTForSampling
+    from transformers_neuronx_amd.config import ContinuousBatchingConfig, NeuronConfig
+    folder, cfg, weights = tiny_folders["B"]
+    nc = NeuronConfig(continuous_batching=ContinuousBatchingConfig(max_num_seqs=3, max_model_len=64), padding_side="right")
+    model = OPTForSampling.from_pretrained(folder, batch_size=3, amp="f32", n_positions=64, neuron_config=nc,
+                                           kernels="reference", device="cpu", page_size=16).load()
+    a, b = _requests(cfg["vocab_size"], [11, 4], 12).values()
+
+    def last(tokens):
+        return plain_opt.forward_logits(weights, cfg, tokens)[-1]
+    la = model(torch.tensor([a]), torch.arange(11).unsqueeze(0), torch.tensor([2]))
+    lb = model(torch.tensor([b]), torch.arange(4).unsqueeze(0), torch.tensor([0]))
+    torch.testing.assert_close(la[0], last(a), atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(lb[0], last(b), atol=1e-5, rtol=1e-5)
+    both = model(torch.tensor([[7], [9]]), torch.tensor([[4], [11]]), torch.tensor([0, 2]))      # b first, then a
+    torch.testing.assert_close(both[0], last(b + [7]), atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(both[1], last(a + [9]), atol=1e-5, rtol=1e-5)
+    with pytest.raises(ValueError, match="holds"):
+        model(torch.tensor([[5]]), torch.tensor([[9]]), torch.tensor([0]))
+    again = model(torch.tensor([a[:6]]), torch.arange(6).unsqueeze(0), torch.tensor([0]))          # row 0 anew
+    torch.testing.assert_close(again[0], last(a[:6]), atol=1e-5, rtol=1e-5)
+    only_a = model(torch.tensor([[3]]), torch.tensor([[12]]), torch.tensor([2]))                   # row 2 went on
+    torch.testing.assert_close(only_a[0], last(a + [9, 3]), atol=1e-5, rtol=1e-5)
+
+
 def test_generation_config_options(tiny_folders):
     """`GenerationConfig` as the reference's on-device generation reads it (config.py:106-139): a value a
     batch line, a global top-k above the lines' own, a least number of tokens for top-p, and the constant

@@ -146,6 +146,8 @@ class OPTForSampling:
         to `start_ids` lose their padding here instead of masking it)."""
         engine = self._need_engine()
         runner = engine.runner
+        if self.neuron_config.continuous_batching is not None and cache_ids is not None and start_ids is not None:
+            return self._forward_sequences(input_ids, cache_ids, start_ids)
         rows = self._rows(input_ids, start_ids)
         if cache_ids is None:
             for b in range(len(rows)):
@@ -164,6 +166,35 @@ class OPTForSampling:
         if every:
             return logits.view(len(rows), -1, logits.shape[-1])
         return logits
+
+    def _forward_sequences(self, input_ids, cache_ids, seq_ids) -> torch.Tensor:
+        """The form a continuous-batching driver uses (base.py:500-600, :630-637): `seq_ids` (given as
+        `start_ids`) name the cache rows, `cache_ids [n, tokens]` the positions the tokens take. A row
+        whose positions begin at 0 starts a new sequence in that row; otherwise the tokens go on from
+        where the row is. Rows not named keep what they hold. Logits come back in the order given."""
+        runner = self.engine.runner
+        ids = torch.as_tensor(input_ids)
+        pos = torch.as_tensor(cache_ids)
+        if ids.dim() == 1:
+            ids = ids.unsqueeze(0)
+        if pos.dim() == 1:
+            pos = pos.unsqueeze(0).expand(ids.shape[0], -1)
+        seqs = [int(s) for s in torch.as_tensor(seq_ids).flatten()]
+        if len(seqs) != ids.shape[0] or pos.shape != ids.shape:
+            raise ValueError(f"{ids.shape[0]} rows of tokens, positions of shape {tuple(pos.shape)}, {len(seqs)} seq_ids")
+        every = self.neuron_config.output_all_logits
+        entries = []
+        for i, seq in enumerate(seqs):
+            key, first = ("seq", seq), int(pos[i, 0])
+            if first == 0:
+                runner.finish(key)
+            have = runner.cache.num_tokens(key) if runner.cache.has(key) else 0
+            if first != have:
+                raise ValueError(f"cache_ids start at {first}, but sequence {seq} holds {have} tokens")
+            toks = ids[i].tolist()
+            entries.append(StepEntry(key, toks, list(range(len(toks))) if every else [len(toks) - 1]))
+        logits = runner.step(entries)
+        return logits.view(len(seqs), -1, logits.shape[-1]) if every else logits
 
     __call__ = forward
 
