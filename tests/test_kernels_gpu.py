@@ -96,6 +96,12 @@ def test_linear(dtype, m, n, k):
         y_t = hip.linear(x, w, bias, act="relu", residual=res, out_f32=True, force_tiled=True)
         y_r = ref.linear(x, w, bias, act="relu", residual=res, out_f32=True)
         torch.testing.assert_close(y_t, y_r, **tol32)
+        if m <= 32:
+            # the few-rows kernel with two weight tiles a block, from the row-major weight and from the tile-ordered copy
+            y_2 = hip.linear(x, w, bias, act="relu", residual=res, out_f32=True, force_tiled=2)
+            torch.testing.assert_close(y_2, y_r, **tol32)
+            y_2 = hip.linear(x, hip.prepare_weight(w), bias, act="relu", residual=res, out_f32=True, force_tiled=2)
+            torch.testing.assert_close(y_2, y_r, **tol32)
 
 
 def test_linear_float32_matrix_in_bfloat16_engine():
@@ -378,7 +384,7 @@ def test_fused_projection_writes_what_the_two_kernels_write(dtype, heads, kv, hs
     w = (torch.randn(total, width, device=DEV, generator=g) / math.sqrt(width)).to(dtype)
     bias = torch.randn(total, device=DEV, generator=g) * 0.2
     tol = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
-    variants = [0] if dtype == torch.float32 else [0, 1]
+    variants = [0] if dtype == torch.float32 else [0, 1, 2]      # 2: two weight tiles a block
     for b in (bias, None):
         kp_r = torch.full((num_pages, kv, ps, hs), float("nan"), device=DEV, dtype=dtype)
         vp_r = torch.full((num_pages, kv, hs, ps), float("nan"), device=DEV, dtype=dtype)

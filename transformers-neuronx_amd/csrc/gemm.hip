@@ -287,7 +287,9 @@ gemm_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, con
 
 // ------------------------------------------------------------------------------------------ bfloat16, few rows
 
-// One block of WAVES waves makes 16 columns of the output (16 rows of `w`) for all M <= 16 * MT rows of `x`.
+// One block of WAVES waves makes 16 * RT columns of the output (RT tiles of 16 rows of `w`) for all
+// M <= 16 * MT rows of `x`; with RT = 2 every fragment of `x` serves two products, which pays for wide
+// matrices (N >= 16,384: 29.2 -> 27.2 us at 8 rows, 34.1 -> 29.6 at 16) and costs blocks for narrow ones.
 // The waves share the K axis in steps of 128; inside a step each of the four loads of a wave covers 64
 // contiguous bytes of each of its 16 weight rows (the four lane groups side by side), and `x` is read the
 // same way. The weight is fetched two steps ahead of its use, `x` one step. No load in the main loop
@@ -298,23 +300,28 @@ gemm_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, con
 // With SHUF the weight is read from a copy laid out for this kernel: [N/16][K/128][4][16 rows][4][8], that is
 // tile after tile in the order the loads take it, so that a block streams one contiguous run of memory and
 // each load of a wave covers 1 KB of it (N a multiple of 16, K of 128).
-template <int MT, int WAVES, bool QKV, bool SHUF>
+template <int MT, int WAVES, bool QKV, bool SHUF, int RT>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
                         const float* __restrict__ residual, void* __restrict__ out, int out_dtype, int act, int M,
                         int N, int K, QkvScatter sc) {
-  __shared__ float red[WAVES][MT][4][64];
+  __shared__ float red[WAVES][MT][RT][4][64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * 16 * RT;     // RT tiles of 16 weight rows a block; tile j begins at n0 + 16 j
   // element offset of the load of step s at K offset kc: W_STEP * kc + W_LOAD * s from wrow
   constexpr int W_STEP = SHUF ? 16 : 1, W_LOAD = SHUF ? 512 : 32;
-  const bf16_t* wrow = SHUF ? w + (size_t)blockIdx.x * 16 * K + (r * 4 + g) * 8
-                            : w + (size_t)min(n0 + r, N - 1) * K + 8 * g;
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  f32x4 acc[MT];
+  const bf16_t* wrow[RT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < RT; ++j)
+    wrow[j] = SHUF ? w + (size_t)min((int)blockIdx.x * RT + j, N / 16 - 1) * 16 * K + (r * 4 + g) * 8
+                   : w + (size_t)min(n0 + 16 * j + r, N - 1) * K + 8 * g;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  f32x4 acc[MT][RT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int j = 0; j < RT; ++j) acc[t][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
   const bf16_t* xrow[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) xrow[t] = x + (size_t)min(t * 16 + r, M - 1) * K + 8 * g;
@@ -326,11 +333,13 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
     // ahead and `x` one step ahead; the scheduling barriers keep the fetches of later steps in front of
     // the products of the current one, so a product waits only for its own operands.
     const int kb0 = wave * 128;
-    bf16x8 wf[3][4], xf[2][MT][4];
+    bf16x8 wf[3][RT][4], xf[2][MT][4];
     auto fetch_w = [&](int slot, int kc) {
       const int k = min(kc, k_last);
 #pragma unroll
-      for (int s = 0; s < 4; ++s) wf[slot][s] = *(const bf16x8*)(wrow + (size_t)k * W_STEP + W_LOAD * s);
+      for (int j = 0; j < RT; ++j)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) wf[slot][j][s] = *(const bf16x8*)(wrow[j] + (size_t)k * W_STEP + W_LOAD * s);
     };
     auto fetch_x = [&](int slot, int kc) {
       const int k = min(kc, k_last);
@@ -344,7 +353,9 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
       for (int t = 0; t < MT; ++t)
 #pragma unroll
         for (int s = 0; s < 4; ++s)
-          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[wslot][s], xf[xslot][t][s], acc[t], 0, 0, 0);
+#pragma unroll
+          for (int j = 0; j < RT; ++j)
+            acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[wslot][j][s], xf[xslot][t][s], acc[t][j], 0, 0, 0);
     };
     fetch_x(0, kb0);
     fetch_w(0, kb0);
@@ -369,26 +380,31 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
     for (int s = 0; s < 4; ++s) {
       const int k = k_full + 32 * s + 8 * g;
       const bool ok = k + 8 <= K;
-      const bf16x8 wv = ok ? *(const bf16x8*)(wrow + (size_t)k_full * W_STEP + W_LOAD * s) : zero;
 #pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        const bf16x8 xv = ok ? *(const bf16x8*)(xrow[t] + k_full + 32 * s) : zero;
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, xv, acc[t], 0, 0, 0);
+      for (int j = 0; j < RT; ++j) {
+        const bf16x8 wv = ok ? *(const bf16x8*)(wrow[j] + (size_t)k_full * W_STEP + W_LOAD * s) : zero;
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          const bf16x8 xv = ok ? *(const bf16x8*)(xrow[t] + k_full + 32 * s) : zero;
+          acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, xv, acc[t][j], 0, 0, 0);
+        }
       }
     }
   }
 #pragma unroll
   for (int t = 0; t < MT; ++t)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) red[wave][t][i][lane] = acc[t][i];
+    for (int j = 0; j < RT; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave][t][j][i][lane] = acc[t][j][i];
   __syncthreads();
-  // acc[t][i] of lane l is output column n0 + 4*(l/16) + i, row 16*t + l%16.
-  for (int idx = tid; idx < MT * 256; idx += WAVES * 64) {
-    const int t = idx >> 8, i = (idx >> 6) & 3, l = idx & 63;
+  // acc[t][j][i] of lane l is output column n0 + 16*j + 4*(l/16) + i, row 16*t + l%16.
+  for (int idx = tid; idx < MT * RT * 256; idx += WAVES * 64) {
+    const int l = idx & 63, i = (idx >> 6) & 3, j = (idx >> 8) % RT, t = idx / (256 * RT);
     float v = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < WAVES; ++wv) v += red[wv][t][i][l];
-    const int n = n0 + 4 * (l >> 4) + i, m = t * 16 + (l & 15);
+    for (int wv = 0; wv < WAVES; ++wv) v += red[wv][t][j][i][l];
+    const int n = n0 + 16 * j + 4 * (l >> 4) + i, m = t * 16 + (l & 15);
     if (n < N && m < M) {
       if (QKV)
         qkv_store(v, m, n, bias, sc);
@@ -398,24 +414,24 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
   }
 }
 
-template <int MT, int WAVES>
+template <int MT, int WAVES, int RT>
 static void launch_skinny(const bf16_t* xp, const bf16_t* wp, const bf16_t* ws, const float* bias,
                           const float* residual, void* out, int out_dtype, int act, int M, int N, int K,
                           const QkvScatter* sc, hipStream_t stream) {
-  const dim3 grid((N + 15) / 16), block(WAVES * 64);
+  const dim3 grid((N + 16 * RT - 1) / (16 * RT)), block(WAVES * 64);
   const QkvScatter none{};
   if (ws && sc)
-    gemm_bf16_skinny_kernel<MT, WAVES, true, true><<<grid, block, 0, stream>>>(xp, ws, bias, residual, out, out_dtype,
-                                                                            act, M, N, K, *sc);
+    gemm_bf16_skinny_kernel<MT, WAVES, true, true, RT><<<grid, block, 0, stream>>>(xp, ws, bias, residual, out,
+                                                                                out_dtype, act, M, N, K, *sc);
   else if (ws)
-    gemm_bf16_skinny_kernel<MT, WAVES, false, true><<<grid, block, 0, stream>>>(xp, ws, bias, residual, out,
-                                                                             out_dtype, act, M, N, K, none);
+    gemm_bf16_skinny_kernel<MT, WAVES, false, true, RT><<<grid, block, 0, stream>>>(xp, ws, bias, residual, out,
+                                                                                 out_dtype, act, M, N, K, none);
   else if (sc)
-    gemm_bf16_skinny_kernel<MT, WAVES, true, false><<<grid, block, 0, stream>>>(xp, wp, bias, residual, out,
-                                                                             out_dtype, act, M, N, K, *sc);
+    gemm_bf16_skinny_kernel<MT, WAVES, true, false, RT><<<grid, block, 0, stream>>>(xp, wp, bias, residual, out,
+                                                                                 out_dtype, act, M, N, K, *sc);
   else
-    gemm_bf16_skinny_kernel<MT, WAVES, false, false><<<grid, block, 0, stream>>>(xp, wp, bias, residual, out,
-                                                                              out_dtype, act, M, N, K, none);
+    gemm_bf16_skinny_kernel<MT, WAVES, false, false, RT><<<grid, block, 0, stream>>>(xp, wp, bias, residual, out,
+                                                                                  out_dtype, act, M, N, K, none);
 }
 
 static int gemm_bf16_dispatch(const void* x, const void* w, const void* w_tiles, const float* bias,
@@ -434,17 +450,24 @@ static int gemm_bf16_dispatch(const void* x, const void* w, const void* w_tiles,
   // tiles' detour through LDS: 245 against 151 us for the 50,272 x 4,096 head at 64 rows), or when asked for.
   if ((M <= 32 || ((force_tiled == 4 || force_tiled == 8) && M <= 64)) && force_tiled != 1) {
     // Eight waves a block when the sum over K is long and the rows are few (more bytes in flight for each
-    // of the few blocks), four otherwise. force_tiled 4 or 8 picks the count, for measurements.
+    // of the few blocks), four otherwise; two weight tiles a block for wide matrices. force_tiled 4 or 8
+    // picks the wave count and 2 the two tiles, for measurements and tests.
     const int waves = force_tiled == 4 || force_tiled == 8 ? force_tiled : (K >= 8192 && N <= 8192 ? 8 : 4);
-#define SKINNY(MT, WV) launch_skinny<MT, WV>(xp, wp, ws, bias, residual, out, out_dtype, act, M, N, K, sc, stream)
-#define SKINNY_MT(WV)                     \
-  switch ((M + 15) / 16) {                \
-    case 1: SKINNY(1, WV); break;         \
-    case 2: SKINNY(2, WV); break;         \
-    case 3: SKINNY(3, WV); break;         \
-    default: SKINNY(4, WV); break;        \
+    const bool two_tiles = force_tiled == 2 || (force_tiled == 0 && waves == 4 && N >= 16384 && M <= 32);
+#define SKINNY(MT, WV, RT) \
+  launch_skinny<MT, WV, RT>(xp, wp, ws, bias, residual, out, out_dtype, act, M, N, K, sc, stream)
+#define SKINNY_MT(WV)                        \
+  switch ((M + 15) / 16) {                   \
+    case 1: SKINNY(1, WV, 1); break;         \
+    case 2: SKINNY(2, WV, 1); break;         \
+    case 3: SKINNY(3, WV, 1); break;         \
+    default: SKINNY(4, WV, 1); break;        \
   }
-    if (waves == 8) {
+    if (two_tiles && M <= 16) {
+      SKINNY(1, 4, 2);
+    } else if (two_tiles && M <= 32) {
+      SKINNY(2, 4, 2);
+    } else if (waves == 8) {
       SKINNY_MT(8);
     } else {
       SKINNY_MT(4);
