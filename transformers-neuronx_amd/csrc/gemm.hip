@@ -449,10 +449,10 @@ static int gemm_bf16_dispatch(const void* x, const void* w, const void* w_tiles,
   // The few-rows kernel up to 32 rows (beyond that every block reading all of `x` again costs more than the
   // tiles' detour through LDS: 245 against 151 us for the 50,272 x 4,096 head at 64 rows), or when asked for.
   if ((M <= 32 || ((force_tiled == 4 || force_tiled == 8) && M <= 64)) && force_tiled != 1) {
-    // Eight waves a block when the sum over K is long and the rows are few (more bytes in flight for each
-    // of the few blocks), four otherwise; two weight tiles a block for wide matrices. force_tiled 4 or 8
-    // picks the wave count and 2 the two tiles, for measurements and tests.
-    const int waves = force_tiled == 4 || force_tiled == 8 ? force_tiled : (K >= 8192 && N <= 8192 ? 8 : 4);
+    // Four waves a block; eight when the blocks are fewer than the compute units and the sum over K is long
+    // enough to share (more bytes in flight for each of the few blocks). Two weight tiles a block for wide
+    // matrices. force_tiled 4 or 8 picks the wave count and 2 the two tiles, for measurements and tests.
+    const int waves = force_tiled == 4 || force_tiled == 8 ? force_tiled : (N < 4096 && K >= 2048 ? 8 : 4);
     const bool two_tiles = force_tiled == 2 || (force_tiled == 0 && waves == 4 && N >= 16384 && M <= 32);
 #define SKINNY(MT, WV, RT) \
   launch_skinny<MT, WV, RT>(xp, wp, ws, bias, residual, out, out_dtype, act, M, N, K, sc, stream)
