@@ -357,6 +357,11 @@ def test_bfloat16_attention_kernels_agree(case, window):
     direct.prefill_direct = True                  # the prompt kernel that reads the pages without staging
     o_direct = direct.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)
     torch.testing.assert_close(o_direct.float(), o_plain.float(), rtol=2e-2, atol=2e-2)
+    for sets in (2, 3):                           # the staged prompt kernel with one set of waves a block, and two
+        forced = HipOps(torch.bfloat16, DEV)
+        forced.prefill_direct = sets
+        o_forced = forced.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)
+        torch.testing.assert_close(o_forced.float(), o_plain.float(), rtol=2e-2, atol=2e-2)
     narrow = HipOps(torch.bfloat16, DEV)
     narrow.decode_wide_blocks = 0                 # blocks of four waves only, twice the splits
     narrow.decode_blocks_wanted = 1 << 20

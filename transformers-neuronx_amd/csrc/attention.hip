@@ -276,6 +276,24 @@ extern "C" int tnx_attention_any(const void* q, int dtype, const void* k_pages, 
 #define PREFILL_Q_TILE 128  // queries per block: four waves of 32
 #define LOG2E 1.4426950408889634f
 
+// Maximum and sum over the four rows of 16 lanes of a wave (lanes l, l ^ 16, l ^ 32, l ^ 48), the same bits in
+// all four: gfx950's lane swaps exchange halves and rows of two registers in the vector unit, where a
+// shuffle would go through LDS and make the wave wait for it.
+__device__ inline float rows_max(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned v = __float_as_uint(fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])));
+  const auto b = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ inline float rows_sum(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned v = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
+  const auto b = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // Flash-style attention of a run of queries over its request's pages, on MFMA 16x16x32.
 // A wave owns 32 queries (two column blocks of 16) and walks the keys 64 at a time. It computes the
 // transposed scores S^T = K Q^T, so that the accumulator layout (lane = query, four consecutive keys per
@@ -462,8 +480,13 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict_
 // FAST is the case of a head size of exactly 16 * NDB and pages of 64 keys or more: a tile then lies within
 // one page, whose number is one scalar lookup, every thread's place within the tile is fixed, and no part of
 // the inner loops depends on a size known only at run time.
-template <int NDB, bool FAST>
-__global__ void __launch_bounds__(256, (NDB <= 8 ? 2 : 1))
+// With GROUPS = 2 a block has two such sets of four waves for the same 128 queries: the first takes the
+// first half of the key tiles and the second the rest, each through LDS buffers of its own, and their
+// partial results (maximum, sum, weighted values, float32) meet in LDS at the end. The tile of the last
+// queries of a long prompt, which sees the most keys, then takes half as long, and it is that tile which the
+// launch waits for.
+template <int NDB, bool FAST, int GROUPS>
+__global__ void __launch_bounds__(256 * GROUPS, (NDB <= 8 && GROUPS == 1 ? 2 : 1))
 attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                              const bf16_t* __restrict__ v_pages, const int* __restrict__ run_start,
                              const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
@@ -478,10 +501,11 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   constexpr int KCH = (64 * DMAX / 8 + 255) / 256;   // 16-byte chunks a thread stages per tile, keys
   constexpr int VCH = (DMAX * 8 + 255) / 256;        // and values
   extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
-  bf16_t* ks_buf = smem;                    // [2][KBUF]
-  bf16_t* vs_buf = smem + 2 * KBUF;         // [2][VBUF]
+  const int grp = GROUPS == 1 ? 0 : threadIdx.x >> 8;      // which set of four waves
+  bf16_t* ks_buf = smem + grp * 2 * (KBUF + VBUF);          // [2][KBUF]
+  bf16_t* vs_buf = ks_buf + 2 * KBUF;                       // [2][VBUF]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;   // within the set
   const int r = lane & 15, g = lane >> 4;
   const int tile = blockIdx.x / num_heads, h = blockIdx.x % num_heads;
   const int run = tile_run[tile];
@@ -616,34 +640,57 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   };
 
   int buf = 0;
-  const int tile_begin = (blk_lo / 64) * 64;
-  lookup(tile_begin);
+  // the block's key tiles, in equal shares for its sets of waves; every set passes the same number of
+  // barriers, a set whose share is shorter (or empty) idles at the end
+  const int blk_begin = (blk_lo / 64) * 64;
+  const int share = ((blk_last - blk_begin) / 64 + GROUPS) / GROUPS;      // tiles a set, rounded up
+  const int tile_begin = blk_begin + grp * share * 64;
+  const int tile_last = min(blk_last, tile_begin + share * 64 - 1);         // the last key of this set
+  lookup(tile_begin);               // past the request the lookups repeat its last page: harmless
   fetch(tile_begin);
-  lookup(tile_begin + 64);          // past the request the lookups repeat its last page: harmless
-  for (int tile0 = tile_begin; tile0 <= blk_last; tile0 += 64, buf ^= 1) {
-    stage(buf, tile0);
+  lookup(tile_begin + 64);
+  for (int it = 0, tile0 = tile_begin; it < share; ++it, tile0 += 64, buf ^= 1) {
+    const bool live = tile0 <= tile_last;
+    if (live) stage(buf, tile0);
     __syncthreads();
-    if (tile0 + 64 <= blk_last) {
+    if (tile0 + 64 <= tile_last) {
       fetch(tile0 + 64);
       lookup(tile0 + 128);
     }
-    if (!wave_on || tile0 > last_q || tile0 + 63 < lo) continue;
+    if (!live || !wave_on || tile0 > last_q || tile0 + 63 < lo) continue;
     const bf16_t* kd = ks_buf + buf * KBUF;
     const bf16_t* vd = vs_buf + buf * VBUF;
 
+    // the keys of 16 rows are read from LDS while the products of the 16 rows before them run (where the
+    // registers allow a second set of them: head sizes up to 128)
+    constexpr int KA = NDB <= 8 ? 2 : 1;
     f32x4 s[4][2];
-#pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
-      f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+    bf16x8 kf[KA][NKS];
+    auto read_keys = [&](int kb, bf16x8* dst) {
       const bf16_t* krow = kd + (16 * kb + r) * KSTR + 8 * g;
 #pragma unroll
+      for (int ks = 0; ks < NKS; ++ks)
+        dst[ks] = (32 * ks + 8 * g < head_size) ? *(const bf16x8*)(krow + 32 * ks) : zero8;
+    };
+    if (KA == 2) read_keys(0, kf[0]);
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      if (KA == 2) {
+        if (kb < 3) read_keys(kb + 1, kf[(kb + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);    // the reads stay ahead of the products, as written
+      } else {
+        read_keys(kb, kf[0]);
+      }
+      const bf16x8* kc = kf[KA == 2 ? kb & 1 : 0];
+      f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
-        const bf16x8 kf = (32 * ks + 8 * g < head_size) ? *(const bf16x8*)(krow + 32 * ks) : zero8;
-        a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[0][ks], a0, 0, 0, 0);
-        a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[1][ks], a1, 0, 0, 0);
+        a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kc[ks], qf[0][ks], a0, 0, 0, 0);
+        a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kc[ks], qf[1][ks], a1, 0, 0, 0);
       }
       s[kb][0] = a0;
       s[kb][1] = a1;
+      if (KA == 2) __builtin_amdgcn_sched_barrier(0);
     }
     const bool full_tile = tile0 + 63 <= first_q && (window <= 0 || tile0 > last_q - window);
     if (!full_tile) {
@@ -665,8 +712,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
       for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s[kb][qb][i]);
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = rows_max(mx);
       const float m_new = fmaxf(m[qb], mx);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
       // e^(x - m) as 2^(x log2 e - m log2 e): one multiply-add and the hardware's 2^x
@@ -681,8 +727,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
           s[kb][qb][i] = p;
           sum += p;
         }
-      sum += __shfl_xor(sum, 16, 64);
-      sum += __shfl_xor(sum, 32, 64);
+      sum = rows_sum(sum);
       l[qb] = l[qb] * alpha + sum;
       // the sums so far are rescaled only if the maximum of some query of the wave moved
       if (__builtin_amdgcn_ballot_w64(m_new != m[qb]) != 0) {
@@ -700,9 +745,8 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
       for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
         for (int j = 0; j < 8; ++j) pb[qb][j] = (bf16_t)s[2 * t + (j >> 2)][qb][j & 3];
-#pragma unroll
-      for (int db = 0; db < NDB; ++db) {
-        if (db >= ndb) continue;
+      // the values of 16 head-size elements are read while the products of the 16 before them run
+      auto read_values = [&](int db) {
         const bf16_t* vrow = vd + (16 * db + r) * VSTR + 32 * t + 4 * g;
         const bf16x4 lo4 = *(const bf16x4*)(vrow);
         const bf16x4 hi4 = *(const bf16x4*)(vrow + 16);
@@ -712,8 +756,56 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
           vf[i] = lo4[i];
           vf[4 + i] = hi4[i];
         }
-        o[db][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[0], o[db][0], 0, 0, 0);
-        o[db][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[1], o[db][1], 0, 0, 0);
+        return vf;
+      };
+      bf16x8 vf[3];
+      vf[0] = read_values(0);
+      vf[1] = read_values(min(1, NDB - 1));
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) {
+        if (db + 2 < NDB) vf[(db + 2) % 3] = read_values(db + 2);
+        __builtin_amdgcn_sched_barrier(0);    // the reads stay ahead of the products, as written
+        if (db < ndb) {
+          o[db][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db % 3], pb[0], o[db][0], 0, 0, 0);
+          o[db][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db % 3], pb[1], o[db][1], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+  if (GROUPS == 2) {
+    // the second set leaves what it has in LDS (every lane its own words, lanes side by side), the first adds it
+    float* po = (float*)smem;                                   // [4 waves][NDB][2][4][64]
+    float* pml = po + 4 * NDB * 2 * 4 * 64;                     // [4 waves][2][2][64]
+    __syncthreads();                                            // the staged tiles are done with
+    if (grp == 1 && wave_on) {
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) {
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) po[(((wave * NDB + db) * 2 + qb) * 4 + i) * 64 + lane] = o[db][qb][i];
+        pml[((wave * 2 + qb) * 2 + 0) * 64 + lane] = m[qb];
+        pml[((wave * 2 + qb) * 2 + 1) * 64 + lane] = l[qb];
+      }
+    }
+    __syncthreads();
+    if (grp == 1) return;
+    if (wave_on) {
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) {
+        const float m1 = pml[((wave * 2 + qb) * 2 + 0) * 64 + lane];
+        const float l1 = pml[((wave * 2 + qb) * 2 + 1) * 64 + lane];
+        const float m_all = fmaxf(m[qb], m1);
+        const float m_safe = m_all == -INFINITY ? 0.f : m_all;
+        const float a0 = __builtin_amdgcn_exp2f((m[qb] - m_safe) * LOG2E);
+        const float a1 = __builtin_amdgcn_exp2f((m1 - m_safe) * LOG2E);
+        l[qb] = l[qb] * a0 + l1 * a1;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            o[db][qb][i] = o[db][qb][i] * a0 + po[(((wave * NDB + db) * 2 + qb) * 4 + i) * 64 + lane] * a1;
       }
     }
   }
@@ -735,17 +827,19 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   }
 }
 
-template <int NDB, bool FAST>
+template <int NDB, bool FAST, int GROUPS>
 static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k_pages,
                               const bf16_t* v_pages, const int* run_start, const int* cached_lens, const int* table,
                               int table_width, int page_shift, int num_pages, const int* tile_run,
                               const int* tile_q0, bf16_t* out, int num_heads, int num_kv, int head_size,
                               int window) {
   constexpr int DMAX = 16 * NDB;
-  constexpr size_t bytes = 2 * (size_t)(64 * (DMAX + 8) + DMAX * (64 + 8)) * sizeof(bf16_t);
+  constexpr size_t bytes = GROUPS * 2 * (size_t)(64 * (DMAX + 8) + DMAX * (64 + 8)) * sizeof(bf16_t);
+  static_assert(GROUPS == 1 || bytes >= (4 * NDB * 2 * 4 * 64 + 4 * 2 * 2 * 64) * sizeof(float),
+                "the partial results of the second set of waves must fit the staging buffers");
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<NDB, FAST>,
+    hipError_t e = hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<NDB, FAST, GROUPS>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
     if (e != hipSuccess) {
       tnx_set_error("attention_prefill: cannot reserve %zu bytes of LDS: %s", bytes, hipGetErrorString(e));
@@ -753,7 +847,7 @@ static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, co
     }
     configured = true;
   }
-  attention_prefill_lds_kernel<NDB, FAST><<<grid, 256, bytes, stream>>>(q, k_pages, v_pages, run_start, cached_lens, table,
+  attention_prefill_lds_kernel<NDB, FAST, GROUPS><<<grid, 256 * GROUPS, bytes, stream>>>(q, k_pages, v_pages, run_start, cached_lens, table,
                                                                  table_width, page_shift, num_pages, tile_run,
                                                                  tile_q0, out, num_heads, num_kv, head_size, window);
   return 0;
@@ -774,20 +868,23 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
   // Blocks are numbered with the head running fastest: the tiles come ordered by falling work, so the blocks
   // that run longest start first and the short ones fill in behind them.
   dim3 grid((unsigned)num_tiles * num_heads);
-  if ((page_size & (page_size - 1)) == 0 && !direct) {
+  if ((page_size & (page_size - 1)) == 0 && direct != 1) {
+    const int sets = direct == 2 ? 1 : 2;       // `direct` 2: one set of waves a block; 0 or 3: two
     int page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
     int rc;
+#define LDS_ARGS                                                                                                 \
+  grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, \
+      table_width, page_shift, num_pages, tile_run, tile_q0, (bf16_t*)out, num_heads, num_kv, head_size, window
 #define LAUNCH_LDS(NDB)                                                                                          \
-  rc = (NDB <= 8 && page_size >= 64 && head_size == 16 * NDB)                                                            \
-           ? launch_prefill_lds<NDB, true>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages,               \
-                                           (const bf16_t*)v_pages, run_start, cached_lens, table, table_width,   \
-                                           page_shift, num_pages, tile_run, tile_q0, (bf16_t*)out, num_heads,    \
-                                           num_kv, head_size, window)                                            \
-           : launch_prefill_lds<NDB, false>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages,              \
-                                            (const bf16_t*)v_pages, run_start, cached_lens, table, table_width,  \
-                                            page_shift, num_pages, tile_run, tile_q0, (bf16_t*)out, num_heads,   \
-                                            num_kv, head_size, window)
+  {                                                                                                              \
+    constexpr int G = NDB <= 8 ? 2 : 1;     /* two sets of waves where LDS holds the buffers of both */          \
+    const bool fast = NDB <= 8 && page_size >= 64 && head_size == 16 * NDB;                                      \
+    if (sets == 1)                                                                                               \
+      rc = fast ? launch_prefill_lds<NDB, true, 1>(LDS_ARGS) : launch_prefill_lds<NDB, false, 1>(LDS_ARGS);      \
+    else                                                                                                         \
+      rc = fast ? launch_prefill_lds<NDB, true, G>(LDS_ARGS) : launch_prefill_lds<NDB, false, G>(LDS_ARGS);      \
+  }
     if (head_size <= 64) {
       LAUNCH_LDS(4);
     } else if (head_size <= 128) {
@@ -796,6 +893,7 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
       LAUNCH_LDS(16);
     }
 #undef LAUNCH_LDS
+#undef LDS_ARGS
     if (rc) return rc;
     TNX_CHECK_LAUNCH("attention_prefill_lds");
     return 0;

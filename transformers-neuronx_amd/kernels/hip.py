@@ -8,6 +8,7 @@ if that fails the call fails: there is no other path.
 import ctypes
 from typing import Dict, Optional
 
+import numpy as np
 import torch
 
 from . import build
@@ -145,6 +146,7 @@ class HipOps:
         if self.device.type != "cuda" or not torch.cuda.is_available():
             raise RuntimeError("the HIP kernels need a GPU; none is visible to torch")
         _code(dtype)
+        self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         self._bias_copies = {}
         self._landing, self._landing_turn = [None, None], 0
         self._ints, self._ints_done, self._ints_turn = [None, None], [None, None], 0
@@ -450,7 +452,8 @@ class HipOps:
             self._call("attention", "tnx_attention_prefill", _ptr(q), _ptr(k_pages), _ptr(v_pages),
                        _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(view.block_table), view.width,
                        view.page_size, num_pages, _ptr(ctx.tile_run), _ptr(ctx.tile_start), ctx.tile_run.numel(),
-                       _ptr(out), num_heads, num_kv_heads, head_size, window, int(self.prefill_direct), _stream())
+                       _ptr(out), num_heads, num_kv_heads, head_size, window,
+                       int(self.prefill_direct) or self._prefill_sets(ctx, num_heads, window), _stream())
         n_dec = ctx.decode_runs.numel()
         if n_dec:
             splits, waves = self._decode_splits(ctx, n_dec * num_heads, window, head_size <= 128)
@@ -466,8 +469,35 @@ class HipOps:
                        _stream())
         return out
 
+    def _prefill_sets(self, ctx, num_heads, window) -> int:
+        """How the staged prompt kernel runs this step: 0, two sets of four waves a block that halve a tile's
+        keys between them, or 2, one set. One set lets two blocks share a compute unit and overlap each other's
+        waits; two sets halve the time of the tile that sees the most keys, which the launch waits for when the
+        blocks are few or uneven. The choice compares the two estimates below, in the time one 64-key step
+        of a block takes (measured at head size 128: 2.6 us for a block alone on its unit, 3.9 us for two that
+        share it, 4.1 us for a block of two sets, 7 us for a second round of blocks)."""
+        plan = ctx.plans.get(("prefill_sets", window))
+        if plan is None:
+            lens, cached = ctx.run_lens_host, ctx.cached_lens_host
+            steps = []
+            for i in np.nonzero(lens > 1)[0]:
+                for q0 in range(0, int(lens[i]), ctx.query_tile):
+                    last = int(cached[i]) + min(q0 + ctx.query_tile, int(lens[i]))      # keys the tile's last query sees
+                    first = max(0, int(cached[i]) + q0 - window + 1) // 64 if window > 0 else 0
+                    steps.append(-(-last // 64) - first)
+            steps = np.array(steps)
+            halves = (steps + 1) // 2
+            units = self.compute_units
+            one = max(steps.max() * 2.6, steps.sum() * num_heads / units * 1.95)
+            two = max(halves.max() * 4.1, halves.sum() * num_heads / units * 4.1)
+            if len(steps) * num_heads > units:
+                two += 7.0
+            plan = ctx.plans[("prefill_sets", window)] = 0 if two < one else 2
+        return plan
+
     value_tiles = True                # tests clear it to write every value token by token
-    prefill_direct = False            # tests set it to run the prompt kernel that reads pages without LDS staging
+    prefill_direct = False            # tests set it: True, the prompt kernel that reads pages without LDS staging;
+                                      # 2, the staged one with one set of four waves a block; 3, with two
     force_plain_attention = False     # tests set it to run the one-wave-per-query kernel in bfloat16 too
     decode_wide_blocks = 1            # blocks of eight waves where four-wave blocks would be split
     decode_blocks_wanted = 512        # the keys of decoding requests are split until about this many blocks run
