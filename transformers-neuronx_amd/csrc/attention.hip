@@ -276,23 +276,6 @@ extern "C" int tnx_attention_any(const void* q, int dtype, const void* k_pages, 
 #define PREFILL_Q_TILE 128  // queries per block: four waves of 32
 #define LOG2E 1.4426950408889634f
 
-// Maximum and sum over the four rows of 16 lanes of a wave (lanes l, l ^ 16, l ^ 32, l ^ 48), the same bits in
-// all four: gfx950's lane swaps exchange halves and rows of two registers in the vector unit, where a
-// shuffle would go through LDS and make the wave wait for it.
-__device__ inline float rows_max(float x) {
-  const unsigned u = __float_as_uint(x);
-  const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  const unsigned v = __float_as_uint(fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])));
-  const auto b = __builtin_amdgcn_permlane16_swap(v, v, false, false);
-  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
-}
-__device__ inline float rows_sum(float x) {
-  const unsigned u = __float_as_uint(x);
-  const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  const unsigned v = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
-  const auto b = __builtin_amdgcn_permlane16_swap(v, v, false, false);
-  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
-}
 
 // Flash-style attention of a run of queries over its request's pages, on MFMA 16x16x32.
 // A wave owns 32 queries (two column blocks of 16) and walks the keys 64 at a time. It computes the
@@ -391,8 +374,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict_
       for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s[kb][qb][i]);
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = rows_max(mx);
       const float m_new = fmaxf(m[qb], mx);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
       const float alpha = __expf(m[qb] - m_safe);
@@ -405,8 +387,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict_
           s[kb][qb][i] = p;
           sum += p;
         }
-      sum += __shfl_xor(sum, 16, 64);
-      sum += __shfl_xor(sum, 32, 64);
+      sum = rows_sum(sum);
       l[qb] = l[qb] * alpha + sum;
       m[qb] = m_new;
 #pragma unroll

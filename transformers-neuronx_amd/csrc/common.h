@@ -72,15 +72,73 @@ __device__ __forceinline__ void store_any(void* p, int dtype, size_t i, float v)
     ((bf16_t*)p)[i] = (bf16_t)v;
 }
 
+// Exchanges between the lanes of a wave without LDS. Within a row of 16 lanes the vector unit's data-parallel
+// controls reach lane ^ 1 and lane ^ 2 (quad permutations), 7 - lane within 8 (the other quad), 15 - lane
+// (the other half of the row) and lane ^ 8 (a rotation by 8); between rows, gfx950's lane swaps exchange rows
+// and halves of two registers. A shuffle would go through LDS and make the wave wait for it.
+#define TNX_DPP_XOR1 0xB1         // quad_perm [1, 0, 3, 2]
+#define TNX_DPP_XOR2 0x4E         // quad_perm [2, 3, 0, 1]
+#define TNX_DPP_HALF_MIRROR 0x141 // lane -> 7 - lane within each 8
+#define TNX_DPP_MIRROR 0x140      // lane -> 15 - lane within each 16
+#define TNX_DPP_XOR8 0x128        // row_ror:8
+template <int CTRL>
+__device__ __forceinline__ float lane_dpp(float v) {
+  const int i = __builtin_bit_cast(int, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(i, i, CTRL, 0xf, 0xf, false));
+}
+// The swaps give back both registers as a pair; its halves are taken into scalars before anything else is
+// done with them (a bit cast applied to an element of the pair reads the first element, whichever is named).
+__device__ __forceinline__ void swap_rows(unsigned u, unsigned& first, unsigned& second) {
+  const auto p = __builtin_amdgcn_permlane16_swap(u, u, false, false);   // rows [r0 r0 r2 r2] and [r1 r1 r3 r3]
+  first = p[0];
+  second = p[1];
+}
+__device__ __forceinline__ void swap_halves(unsigned u, unsigned& first, unsigned& second) {
+  const auto p = __builtin_amdgcn_permlane32_swap(u, u, false, false);   // halves [lo lo] and [hi hi]
+  first = p[0];
+  second = p[1];
+}
+// the value of lane ^ 16, and of lane ^ 32
+__device__ __forceinline__ float lane_xor16(float v) {
+  unsigned a, b;
+  swap_rows(__float_as_uint(v), a, b);
+  return __uint_as_float((threadIdx.x & 16) ? a : b);
+}
+__device__ __forceinline__ float lane_xor32(float v) {
+  unsigned a, b;
+  swap_halves(__float_as_uint(v), a, b);
+  return __uint_as_float((threadIdx.x & 32) ? a : b);
+}
+// Maximum and sum over the four rows of 16 lanes of a wave (lanes l, l ^ 16, l ^ 32, l ^ 48), the same bits in
+// all four.
+__device__ __forceinline__ float rows_max(float x) {
+  unsigned a, b;
+  swap_halves(__float_as_uint(x), a, b);
+  x = fmaxf(__uint_as_float(a), __uint_as_float(b));
+  swap_rows(__float_as_uint(x), a, b);
+  return fmaxf(__uint_as_float(a), __uint_as_float(b));
+}
+__device__ __forceinline__ float rows_sum(float x) {
+  unsigned a, b;
+  swap_halves(__float_as_uint(x), a, b);
+  x = __uint_as_float(a) + __uint_as_float(b);
+  swap_rows(__float_as_uint(x), a, b);
+  return __uint_as_float(a) + __uint_as_float(b);
+}
+// Sum and maximum over the 64 lanes of a wave, the same bits in every lane.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
+  v += lane_dpp<TNX_DPP_XOR1>(v);
+  v += lane_dpp<TNX_DPP_XOR2>(v);
+  v += lane_dpp<TNX_DPP_HALF_MIRROR>(v);
+  v += lane_dpp<TNX_DPP_MIRROR>(v);
+  return rows_sum(v);
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
+  v = fmaxf(v, lane_dpp<TNX_DPP_XOR1>(v));
+  v = fmaxf(v, lane_dpp<TNX_DPP_XOR2>(v));
+  v = fmaxf(v, lane_dpp<TNX_DPP_HALF_MIRROR>(v));
+  v = fmaxf(v, lane_dpp<TNX_DPP_MIRROR>(v));
+  return rows_max(v);
 }
 
 // Sum over a block of `NW` waves; every thread gets the result. `scratch` holds NW floats.

@@ -155,9 +155,7 @@ gemm_f32_skinny_kernel(const float* __restrict__ x, const float* __restrict__ w,
   for (int c = 0; c < 4; ++c)
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
-      float a = acc[c][m];
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) a += __shfl_xor(a, o, 64);
+      const float a = wave_sum(acc[c][m]);
       // every lane has the sum; lane c * MR + m (modulo the wave) writes it
       if (lane == ((c * MR + m) & 63) && n0 + c < N && m < M)
         epilogue_store(a, m, n0 + c, N, bias, residual, out, out_dtype, act);
