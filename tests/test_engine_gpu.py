@@ -9,6 +9,7 @@ import torch
 
 import plain_opt
 import schedules
+from conftest import TINY_A
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -123,11 +124,19 @@ def test_pages_are_used_again_without_leaking(tiny_folders, tmp_path):
 
 
 @pytest.mark.parametrize("amp", ["f32", "bf16"])
-def test_greedy_generation_through_the_entry_point(tiny_folders, amp):
+def test_greedy_generation_through_the_entry_point(tiny_folders, amp, tmp_path):
+    from safetensors.torch import load_file
     from transformers_neuronx_amd import OPTForSampling
+    from transformers_neuronx_amd.config import OPTConfig
     from transformers_neuronx_amd.kernels import hip
-    for name in ("A", "B"):
-        folder, cfg, weights = tiny_folders[name]
+    from transformers_neuronx_amd.weights import write_random_model
+    # with weights as narrow as A's the greedy path repeats one token; a third model has A's sizes and
+    # weights ten times as wide, so that its tokens differ from one another
+    wide = str(tmp_path / "wide")
+    write_random_model(OPTConfig.from_dict(dict(TINY_A, init_std=0.2)), wide, 11, dtype="float32")
+    cases = [tiny_folders["A"], tiny_folders["B"],
+             (wide, json.load(open(os.path.join(wide, "config.json"))), load_file(os.path.join(wide, "model.safetensors")))]
+    for case, (folder, cfg, weights) in enumerate(cases):
         model = OPTForSampling.from_pretrained(folder, batch_size=3, amp=amp, n_positions=64, page_size=16,
                                                num_pages=9, max_num_batched_tokens=24).load()
         ids = torch.randint(3, cfg["vocab_size"], (3, 11), generator=torch.Generator().manual_seed(2))
@@ -136,6 +145,7 @@ def test_greedy_generation_through_the_entry_point(tiny_folders, amp):
         if amp == "f32":
             for b in range(3):
                 assert out[b].tolist() == plain_opt.greedy(weights, cfg, ids[b].tolist(), 29)
+                assert case != 2 or len(set(out[b, 11:].tolist())) > 8
         else:
             # bfloat16 may part from the float32 choice where two logits are close: every chosen token
             # must be within the rounding of the best one under the plain implementation
