@@ -431,9 +431,12 @@ def test_library_product_and_own_product_agree(m, n, k):
                                rtol=1e-3, atol=1e-3)
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 64, 128), (8, 4096, 512), (16, 320, 256), (13, 48, 1024), (64, 128, 384)])
+@pytest.mark.parametrize("m,n,k", [(1, 64, 128), (8, 4096, 512), (16, 320, 256), (13, 48, 1024), (64, 128, 384),
+                                   (8, 8192, 256), (3, 12304, 384), (20, 16400, 128), (1, 50272, 640)])
 def test_product_from_the_tile_ordered_copy(m, n, k):
-    """The few-rows kernel reading the copy of the weight that is laid out tile after tile."""
+    """The few-rows kernel reading the copy of the weight that is laid out tile after tile. The last four
+    matrices have hundreds of tiles: a wave that has no step of its own (K of three steps for four waves), two
+    tiles a block with an odd number of tiles, a vocabulary-sized matrix."""
     from transformers_neuronx_amd.kernels.hip import HipOps, tile_order
     hip, ref = _ops(torch.bfloat16)
     hip.library_rows = 0
