@@ -73,14 +73,13 @@ __device__ __forceinline__ void store_any(void* p, int dtype, size_t i, float v)
 }
 
 // Exchanges between the lanes of a wave without LDS. Within a row of 16 lanes the vector unit's data-parallel
-// controls reach lane ^ 1 and lane ^ 2 (quad permutations), 7 - lane within 8 (the other quad), 15 - lane
-// (the other half of the row) and lane ^ 8 (a rotation by 8); between rows, gfx950's lane swaps exchange rows
-// and halves of two registers. A shuffle would go through LDS and make the wave wait for it.
+// controls reach lane ^ 1 and lane ^ 2 (quad permutations), 7 - lane within 8 (the other quad) and 15 - lane
+// (the other half of the row); between rows, gfx950's lane swaps exchange rows and halves of two registers.
+// A shuffle would go through LDS and make the wave wait for it.
 #define TNX_DPP_XOR1 0xB1         // quad_perm [1, 0, 3, 2]
 #define TNX_DPP_XOR2 0x4E         // quad_perm [2, 3, 0, 1]
 #define TNX_DPP_HALF_MIRROR 0x141 // lane -> 7 - lane within each 8
 #define TNX_DPP_MIRROR 0x140      // lane -> 15 - lane within each 16
-#define TNX_DPP_XOR8 0x128        // row_ror:8
 template <int CTRL>
 __device__ __forceinline__ float lane_dpp(float v) {
   const int i = __builtin_bit_cast(int, v);
@@ -97,17 +96,6 @@ __device__ __forceinline__ void swap_halves(unsigned u, unsigned& first, unsigne
   const auto p = __builtin_amdgcn_permlane32_swap(u, u, false, false);   // halves [lo lo] and [hi hi]
   first = p[0];
   second = p[1];
-}
-// the value of lane ^ 16, and of lane ^ 32
-__device__ __forceinline__ float lane_xor16(float v) {
-  unsigned a, b;
-  swap_rows(__float_as_uint(v), a, b);
-  return __uint_as_float((threadIdx.x & 16) ? a : b);
-}
-__device__ __forceinline__ float lane_xor32(float v) {
-  unsigned a, b;
-  swap_halves(__float_as_uint(v), a, b);
-  return __uint_as_float((threadIdx.x & 32) ? a : b);
 }
 // Maximum and sum over the four rows of 16 lanes of a wave (lanes l, l ^ 16, l ^ 32, l ^ 48), the same bits in
 // all four.
