@@ -204,13 +204,19 @@ def test_trace_run_as_a_program(tiny_folders, tmp_path):
         _compare(str(out), place, expected, cfg["vocab_size"], dtype)
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_recorded_decode_steps_equal_open_ones(tiny_folders, tiny_folders_bf16, dtype):
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16 library"])
+def test_recorded_decode_steps_equal_open_ones(tiny_folders, tiny_folders_bf16, dtype, monkeypatch):
     """Decode steps replayed from a recording give the logits of steps launched in the open, replay after
-    replay, with prompt steps and other batch sizes in between."""
+    replay, with prompt steps and other batch sizes in between. The third case sends every product of two rows
+    and more to the vendor library, as batches of 17 and more do: its calls are recorded and replayed too."""
     from transformers_neuronx_amd.config import EngineConfig
     from transformers_neuronx_amd.engine import StepEntry
     from transformers_neuronx_amd.engine.factory import runner_from_folder
+    from transformers_neuronx_amd.kernels.hip import HipOps
+    if dtype.endswith("library"):
+        dtype = "bfloat16"
+        monkeypatch.setattr(HipOps, "library_rows", 2)
+        monkeypatch.setattr(HipOps, "small_matrix", 0)
     folder, cfg, weights = (tiny_folders if dtype == "float32" else tiny_folders_bf16)["B"]
     requests = _requests(cfg, [60, 3, 90], seed=17)
     expected = _expected(weights, cfg, requests)

@@ -408,7 +408,8 @@ def test_fused_projection_writes_what_the_two_kernels_write(dtype, heads, kv, hs
     torch.testing.assert_close(q.float(), q_r.float(), **tol)
 
 
-@pytest.mark.parametrize("m,n,k", [(256, 96, 320), (300, 1000, 48), (513, 136, 1024)])
+@pytest.mark.parametrize("m,n,k", [(256, 96, 320), (300, 1000, 48), (513, 136, 1024), (17, 4096, 512), (64, 136, 2048),
+                                   (2048, 512, 1024)])
 def test_library_product_and_own_product_agree(m, n, k):
     """From `library_rows` rows on the plain product goes to the vendor library and our epilogue kernel
     follows; below it, and always when told so, our own tiled kernel does all of it."""
@@ -429,6 +430,14 @@ def test_library_product_and_own_product_agree(m, n, k):
     # the head's float32 output never goes through a bfloat16 product
     torch.testing.assert_close(lib.linear(x, w, None, out_f32=True), ref.linear(x, w, None, out_f32=True),
                                rtol=1e-3, atol=1e-3)
+    # nor does the sum with the residual: the library adds bias and residual to its float32 sums itself; with
+    # that switched off the product comes back in bfloat16 and our kernel makes the sum
+    exact = x.float() @ w.float().t() + res
+    torch.testing.assert_close(lib.linear(x, w, None, residual=res, out_f32=True), exact, rtol=1e-3, atol=1e-3)
+    torch.testing.assert_close(lib.linear(x, w, bias, residual=res, out_f32=True), exact + bias, rtol=1e-3, atol=1e-3)
+    rounded = HipOps(torch.bfloat16, DEV)
+    rounded.library_sum = False
+    torch.testing.assert_close(rounded.linear(x, w, bias, residual=res, out_f32=True), exact + bias, rtol=2e-2, atol=2e-2)
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 64, 128), (8, 4096, 512), (16, 320, 256), (13, 48, 1024), (64, 128, 384),

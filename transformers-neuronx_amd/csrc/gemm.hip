@@ -519,3 +519,158 @@ extern "C" int tnx_gemm_bf16_qkv(const void* x, const void* w, const void* w_til
   return gemm_bf16_dispatch(x, w, w_tiles, bias, nullptr, nullptr, TNX_BF16, TNX_ACT_NONE, M, N, K, force_tiled, &sc,
                             stream);
 }
+
+// ------------------------------------------------------------------ the vendor library, with a float32 sum
+//
+// out = x w^T + bias + residual with bfloat16 operands and everything after the product in float32: hipBLASLt
+// adds the bias in its epilogue and the residual as its C matrix, and writes float32, so the product is never
+// rounded to bfloat16 and no kernel of ours has to follow it. The library is the one the process has loaded
+// already (torch brings it); its entry points are looked up at run time, so nothing here is linked against it.
+// Returns 2 where that is not to be had (no library, no algorithm that fits the workspace): the caller then
+// takes the product from the library through torch and the sum from `tnx_epilogue`.
+#if __has_include(<hipblaslt/hipblaslt.h>)
+#include <dlfcn.h>
+#include <hipblaslt/hipblaslt.h>
+
+#include <map>
+#include <mutex>
+#include <tuple>
+
+namespace {
+struct LibraryApi {
+  decltype(&hipblasLtCreate) create = nullptr;
+  decltype(&hipblasLtMatmulDescCreate) desc_create = nullptr;
+  decltype(&hipblasLtMatmulDescSetAttribute) desc_set = nullptr;
+  decltype(&hipblasLtMatrixLayoutCreate) layout_create = nullptr;
+  decltype(&hipblasLtMatmulPreferenceCreate) pref_create = nullptr;
+  decltype(&hipblasLtMatmulPreferenceSetAttribute) pref_set = nullptr;
+  decltype(&hipblasLtMatmulPreferenceDestroy) pref_destroy = nullptr;
+  decltype(&hipblasLtMatmulAlgoGetHeuristic) heuristic = nullptr;
+  decltype(&hipblasLtMatmul) matmul = nullptr;
+  int state = 0;                  // 0 not tried, 1 ready, -1 not to be had
+};
+struct LibraryPlan {
+  hipblasLtMatmulDesc_t desc = nullptr;
+  hipblasLtMatrixLayout_t w = nullptr, x = nullptr, c = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+  size_t workspace = 0;
+  bool usable = false;
+};
+constexpr int MAX_DEVICES = 64;
+LibraryApi library_api;
+hipblasLtHandle_t library_handles[MAX_DEVICES] = {};
+std::map<std::tuple<int, int, int, int, int>, LibraryPlan> library_plans;     // device, M, N, K, what is added
+std::mutex library_mutex;
+
+bool library_ready() {
+  if (library_api.state != 0) return library_api.state > 0;
+  library_api.state = -1;
+  void* lib = dlopen("libhipblaslt.so.1", RTLD_NOW | RTLD_NOLOAD);      // the copy that is loaded, if one is
+  if (!lib) lib = dlopen("libhipblaslt.so.1", RTLD_NOW);
+  if (!lib) lib = dlopen("libhipblaslt.so", RTLD_NOW);
+  if (!lib) return false;
+#define TNX_LIBRARY_SYMBOL(field, name)                          \
+  library_api.field = (decltype(library_api.field))dlsym(lib, name); \
+  if (!library_api.field) return false;
+  TNX_LIBRARY_SYMBOL(create, "hipblasLtCreate")
+  TNX_LIBRARY_SYMBOL(desc_create, "hipblasLtMatmulDescCreate")
+  TNX_LIBRARY_SYMBOL(desc_set, "hipblasLtMatmulDescSetAttribute")
+  TNX_LIBRARY_SYMBOL(layout_create, "hipblasLtMatrixLayoutCreate")
+  TNX_LIBRARY_SYMBOL(pref_create, "hipblasLtMatmulPreferenceCreate")
+  TNX_LIBRARY_SYMBOL(pref_set, "hipblasLtMatmulPreferenceSetAttribute")
+  TNX_LIBRARY_SYMBOL(pref_destroy, "hipblasLtMatmulPreferenceDestroy")
+  TNX_LIBRARY_SYMBOL(heuristic, "hipblasLtMatmulAlgoGetHeuristic")
+  TNX_LIBRARY_SYMBOL(matmul, "hipblasLtMatmul")
+#undef TNX_LIBRARY_SYMBOL
+  library_api.state = 1;
+  return true;
+}
+
+// The plan of one product: descriptors and the first algorithm of the library's own ranking whose workspace
+// fits what the caller brings. Row-major out[M][N] = x[M][K] w[N][K]^T is, in the library's column-major
+// terms, D[N x M] = op_T(w as K x N) x (x as K x M).
+LibraryPlan make_plan(hipblasLtHandle_t handle, int M, int N, int K, bool with_bias, size_t workspace_bytes) {
+  LibraryPlan p;
+  const LibraryApi& a = library_api;
+  if (a.desc_create(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return p;
+  const hipblasOperation_t trans = HIPBLAS_OP_T, plain = HIPBLAS_OP_N;
+  bool ok = a.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &trans, sizeof(trans)) == HIPBLAS_STATUS_SUCCESS &&
+            a.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &plain, sizeof(plain)) == HIPBLAS_STATUS_SUCCESS;
+  if (with_bias) {
+    const hipblasLtEpilogue_t epilogue = HIPBLASLT_EPILOGUE_BIAS;
+    const hipDataType bias_type = HIP_R_32F;
+    ok = ok && a.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue)) == HIPBLAS_STATUS_SUCCESS &&
+         a.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type)) == HIPBLAS_STATUS_SUCCESS;
+  }
+  ok = ok && a.layout_create(&p.w, HIP_R_16BF, K, N, K) == HIPBLAS_STATUS_SUCCESS &&
+       a.layout_create(&p.x, HIP_R_16BF, K, M, K) == HIPBLAS_STATUS_SUCCESS &&
+       a.layout_create(&p.c, HIP_R_32F, N, M, N) == HIPBLAS_STATUS_SUCCESS;
+  if (!ok) return p;
+  hipblasLtMatmulPreference_t pref = nullptr;
+  if (a.pref_create(&pref) != HIPBLAS_STATUS_SUCCESS) return p;
+  constexpr int WANTED = 4;
+  hipblasLtMatmulHeuristicResult_t found[WANTED];
+  int count = 0;
+  if (a.pref_set(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &workspace_bytes, sizeof(workspace_bytes)) ==
+          HIPBLAS_STATUS_SUCCESS &&
+      a.heuristic(handle, p.desc, p.w, p.x, p.c, p.c, pref, WANTED, found, &count) == HIPBLAS_STATUS_SUCCESS) {
+    for (int i = 0; i < count && i < WANTED; ++i) {
+      // an algorithm is taken only with all the workspace it asks for
+      if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= workspace_bytes) {
+        p.algo = found[i].algo;
+        p.workspace = found[i].workspaceSize;
+        p.usable = true;
+        break;
+      }
+    }
+  }
+  a.pref_destroy(pref);
+  return p;
+}
+}  // namespace
+
+extern "C" int tnx_gemm_sum_library(const void* x, const void* w, const float* bias, const float* residual, float* out,
+                                    int M, int N, int K, void* workspace, size_t workspace_bytes,
+                                    hipStream_t stream) {
+  TNX_REQUIRE(M > 0 && N > 0 && K > 0 && N % 8 == 0 && K % 8 == 0, "gemm_sum_library: bad sizes M=%d N=%d K=%d", M, N, K);
+  TNX_REQUIRE(((uintptr_t)x | (uintptr_t)w | (uintptr_t)out | (uintptr_t)residual | (uintptr_t)bias |
+               (uintptr_t)workspace) % 16 == 0,
+              "gemm_sum_library: operands must be 16-byte aligned");
+  TNX_REQUIRE(out != residual, "gemm_sum_library: the sum is not made in place");
+  std::lock_guard<std::mutex> lock(library_mutex);
+  if (!library_ready()) return 2;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= MAX_DEVICES) return 2;
+  if (!library_handles[device] && library_api.create(&library_handles[device]) != HIPBLAS_STATUS_SUCCESS) {
+    library_handles[device] = nullptr;
+    return 2;
+  }
+  const auto key = std::make_tuple(device, M, N, K, (bias ? 1 : 0) | (residual ? 2 : 0));
+  auto it = library_plans.find(key);
+  if (it == library_plans.end())
+    it = library_plans.emplace(key, make_plan(library_handles[device], M, N, K, bias != nullptr, workspace_bytes)).first;
+  const LibraryPlan& p = it->second;
+  if (!p.usable || p.workspace > workspace_bytes) return 2;
+  if (bias) {
+    const void* bias_ptr = bias;
+    if (library_api.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias_ptr, sizeof(bias_ptr)) !=
+        HIPBLAS_STATUS_SUCCESS)
+      return 2;
+  }
+  const float one = 1.f, zero = 0.f;
+  const hipblasStatus_t st =
+      library_api.matmul(library_handles[device], p.desc, &one, w, p.w, x, p.x, residual ? &one : &zero,
+                         residual ? (const void*)residual : (const void*)out, p.c, out, p.c, &p.algo, workspace,
+                         workspace_bytes, stream);
+  if (st != HIPBLAS_STATUS_SUCCESS) {
+    tnx_set_error("gemm_sum_library: the library refused the product (status %d) for M=%d N=%d K=%d", (int)st, M, N, K);
+    return 1;
+  }
+  return 0;
+}
+#else
+extern "C" int tnx_gemm_sum_library(const void*, const void*, const float*, const float*, float*, int, int, int, void*,
+                                    size_t, hipStream_t) {
+  return 2;
+}
+#endif

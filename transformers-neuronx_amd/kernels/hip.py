@@ -39,6 +39,8 @@ _SIGNATURES = {
         "tnx_gemm_bf16_qkv": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
                               _c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int,
                               _c_int, _c_void_p],
+        "tnx_gemm_sum_library": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+                                 _c_void_p, ctypes.c_size_t, _c_void_p],
     },
     "attention": {
         "tnx_qkv_write": [_c_void_p, _c_int, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
@@ -319,6 +321,17 @@ class HipOps:
             # (and applies ReLU) before it rounds; with a residual, bias and sum are ours, in float32. The
             # float32 head keeps our kernel: its output is not rounded to bfloat16 on the way.
             xa = self.cast(x, torch.bfloat16)
+            if residual is not None and out_f32 and act in (None, "none") and self.library_sum:
+                # the library itself adds bias and residual to its float32 sums: nothing is rounded on the way
+                out = torch.empty(m, n, dtype=torch.float32, device=x.device)
+                space = self._library_workspace(x.device)
+                rc = library("gemm").tnx_gemm_sum_library(_ptr(xa), _ptr(w), _ptr(bias), _ptr(residual), _ptr(out), m, n,
+                                                          k, _ptr(space), space.numel(), _stream())
+                if rc == 0:
+                    return out
+                if rc != 2:
+                    raise RuntimeError(f"tnx_gemm_sum_library: {library('gemm').tnx_last_error().decode()}")
+                # 2: not to be had here; the product through torch and the sum by our kernel, below
             if bias is not None and residual is None and not out_f32:
                 b16 = self._bias_bf16(bias)
                 if act == "relu":
@@ -342,6 +355,18 @@ class HipOps:
             self._call("gemm", "tnx_gemm_bf16", _ptr(xa), _ptr(w), _ptr(tiles), _ptr(bias), _ptr(residual),
                        _ptr(out), _code(out_dtype), _ACT[act], m, n, k, int(force_tiled), _stream())
         return out
+
+    library_sum = True      # out = x w^T + bias + residual in one call of the vendor library, where it is to be had
+    _workspaces: Dict[str, torch.Tensor] = {}
+
+    @classmethod
+    def _library_workspace(cls, device) -> torch.Tensor:
+        """Memory the library's algorithms may ask for (those that split the inner dimension over blocks keep
+        partial sums there), one block per device, made at the first product and kept."""
+        key = str(device)
+        if key not in cls._workspaces:
+            cls._workspaces[key] = torch.empty(32 << 20, dtype=torch.uint8, device=device)
+        return cls._workspaces[key]
 
     # From this many rows on, plain bfloat16 products go to the vendor library (0: never). Up to 16 rows our
     # own kernel streams the weight as fast as the library does and fuses what follows the product.
