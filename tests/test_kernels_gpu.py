@@ -436,7 +436,7 @@ def test_library_product_and_own_product_agree(m, n, k):
     torch.testing.assert_close(lib.linear(x, w, None, residual=res, out_f32=True), exact, rtol=1e-3, atol=1e-3)
     torch.testing.assert_close(lib.linear(x, w, bias, residual=res, out_f32=True), exact + bias, rtol=1e-3, atol=1e-3)
     rounded = HipOps(torch.bfloat16, DEV)
-    rounded.library_sum = False
+    rounded.library_direct = False
     torch.testing.assert_close(rounded.linear(x, w, bias, residual=res, out_f32=True), exact + bias, rtol=2e-2, atol=2e-2)
 
 

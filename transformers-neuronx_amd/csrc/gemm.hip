@@ -520,14 +520,22 @@ extern "C" int tnx_gemm_bf16_qkv(const void* x, const void* w, const void* w_til
                             stream);
 }
 
-// ------------------------------------------------------------------ the vendor library, with a float32 sum
+// ------------------------------------------------------------------------------------- the vendor library
 //
-// out = x w^T + bias + residual with bfloat16 operands and everything after the product in float32: hipBLASLt
-// adds the bias in its epilogue and the residual as its C matrix, and writes float32, so the product is never
-// rounded to bfloat16 and no kernel of ours has to follow it. The library is the one the process has loaded
-// already (torch brings it); its entry points are looked up at run time, so nothing here is linked against it.
-// Returns 2 where that is not to be had (no library, no algorithm that fits the workspace): the caller then
-// takes the product from the library through torch and the sum from `tnx_epilogue`.
+// out = act(x w^T + bias) + residual for many rows, as one call of hipBLASLt: bfloat16 operands, float32 sums,
+// the bias (float32) and ReLU in the library's epilogue, and either a bfloat16 result or, for a product that
+// ends in the residual sum, the float32 residual as the library's C matrix and a float32 result, so that such
+// a product is never rounded to bfloat16 and no kernel of ours has to follow it. The library is the one the
+// process has loaded already (torch brings it); its entry points are looked up at run time, so nothing here
+// is linked against it.
+// The library ranks its algorithms for a product by a model of its own. Up to TUNED_ROWS rows (decode batches,
+// short portions of prompts) that ranking is often far off (128 x 4,096 over 16,384: first choice 116 us,
+// sixth 68 us), so there the first six are timed once, on the operands of the first call, with the caches
+// flushed before each run as a step finds them, and the quickest is kept. An algorithm is run only with all
+// the workspace it asks for.
+// Returns 0 when done, 1 on an error, 2 where this is not to be had (no library, an activation it has not,
+// no algorithm that fits) and the caller goes another way, 3 when the algorithms are to be timed first and no
+// memory to flush the caches with came along: the caller calls again with some.
 #if __has_include(<hipblaslt/hipblaslt.h>)
 #include <dlfcn.h>
 #include <hipblaslt/hipblaslt.h>
@@ -556,10 +564,18 @@ struct LibraryPlan {
   size_t workspace = 0;
   bool usable = false;
 };
-constexpr int MAX_DEVICES = 64;
+struct LibraryCall {              // the operands of one product, as the library takes them
+  const void *x, *w, *c;
+  void* out;
+  float beta;
+  void* workspace;
+  size_t workspace_bytes;
+  hipStream_t stream;
+};
+constexpr int MAX_DEVICES = 64, CANDIDATES = 6, TUNED_ROWS = 256;
 LibraryApi library_api;
 hipblasLtHandle_t library_handles[MAX_DEVICES] = {};
-std::map<std::tuple<int, int, int, int, int>, LibraryPlan> library_plans;     // device, M, N, K, what is added
+std::map<std::tuple<int, int, int, int, int>, LibraryPlan> library_plans;     // device, M, N, K, what follows
 std::mutex library_mutex;
 
 bool library_ready() {
@@ -569,7 +585,7 @@ bool library_ready() {
   if (!lib) lib = dlopen("libhipblaslt.so.1", RTLD_NOW);
   if (!lib) lib = dlopen("libhipblaslt.so", RTLD_NOW);
   if (!lib) return false;
-#define TNX_LIBRARY_SYMBOL(field, name)                          \
+#define TNX_LIBRARY_SYMBOL(field, name)                              \
   library_api.field = (decltype(library_api.field))dlsym(lib, name); \
   if (!library_api.field) return false;
   TNX_LIBRARY_SYMBOL(create, "hipblasLtCreate")
@@ -586,57 +602,116 @@ bool library_ready() {
   return true;
 }
 
-// The plan of one product: descriptors and the first algorithm of the library's own ranking whose workspace
-// fits what the caller brings. Row-major out[M][N] = x[M][K] w[N][K]^T is, in the library's column-major
-// terms, D[N x M] = op_T(w as K x N) x (x as K x M).
-LibraryPlan make_plan(hipblasLtHandle_t handle, int M, int N, int K, bool with_bias, size_t workspace_bytes) {
+hipblasStatus_t library_run(hipblasLtHandle_t handle, const LibraryPlan& p, const hipblasLtMatmulAlgo_t& algo,
+                            const LibraryCall& call) {
+  const float one = 1.f;
+  return library_api.matmul(handle, p.desc, &one, call.w, p.w, call.x, p.x, &call.beta, call.c, p.c, call.out, p.c,
+                            &algo, call.workspace, call.workspace_bytes, call.stream);
+}
+
+// Reads `bytes` of memory and keeps nothing: what the caches held before is pushed out by clean lines, as
+// after the attention of a step, which has read the keys and values of every request.
+__global__ void __launch_bounds__(256) library_flush_kernel(const float4* __restrict__ p, size_t n, float* sink) {
+  float a = 0.f;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+    const float4 v = p[i];
+    a += v.x + v.y + v.z + v.w;
+  }
+  if (a == 12345.678f) *sink = a;      // never true for memory that holds no such sum; keeps the loads alive
+}
+
+// Time in ms of one run of an algorithm with cold caches, or a negative number if it cannot be run.
+float library_time(hipblasLtHandle_t handle, const LibraryPlan& p, const hipblasLtMatmulAlgo_t& algo,
+                   const LibraryCall& call, void* flush, size_t flush_bytes, hipEvent_t begin, hipEvent_t end) {
+  for (int warm = 0; warm < 2; ++warm)
+    if (library_run(handle, p, algo, call) != HIPBLAS_STATUS_SUCCESS) return -1.f;
+  float total = 0.f;
+  for (int run = 0; run < 3; ++run) {
+    library_flush_kernel<<<2048, 256, 0, call.stream>>>((const float4*)flush, flush_bytes / 16, (float*)flush);
+    if (hipGetLastError() != hipSuccess || hipEventRecord(begin, call.stream) != hipSuccess) return -1.f;
+    if (library_run(handle, p, algo, call) != HIPBLAS_STATUS_SUCCESS) return -1.f;
+    float ms = 0.f;
+    if (hipEventRecord(end, call.stream) != hipSuccess || hipEventSynchronize(end) != hipSuccess ||
+        hipEventElapsedTime(&ms, begin, end) != hipSuccess)
+      return -1.f;
+    total += ms;
+  }
+  return total;
+}
+
+// The plan of one product: descriptors and an algorithm. Row-major out[M][N] = x[M][K] w[N][K]^T is, in the
+// library's column-major terms, D[N x M] = op_T(w as K x N) (x as K x M).
+LibraryPlan make_plan(hipblasLtHandle_t handle, int M, int N, int K, const float* bias, bool relu, bool out_f32,
+                      const LibraryCall& call, void* flush, size_t flush_bytes) {
   LibraryPlan p;
   const LibraryApi& a = library_api;
   if (a.desc_create(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return p;
   const hipblasOperation_t trans = HIPBLAS_OP_T, plain = HIPBLAS_OP_N;
   bool ok = a.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &trans, sizeof(trans)) == HIPBLAS_STATUS_SUCCESS &&
             a.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &plain, sizeof(plain)) == HIPBLAS_STATUS_SUCCESS;
-  if (with_bias) {
-    const hipblasLtEpilogue_t epilogue = HIPBLASLT_EPILOGUE_BIAS;
-    const hipDataType bias_type = HIP_R_32F;
-    ok = ok && a.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue)) == HIPBLAS_STATUS_SUCCESS &&
-         a.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type)) == HIPBLAS_STATUS_SUCCESS;
+  if (bias || relu) {
+    const hipblasLtEpilogue_t epilogue =
+        bias ? (relu ? HIPBLASLT_EPILOGUE_RELU_BIAS : HIPBLASLT_EPILOGUE_BIAS) : HIPBLASLT_EPILOGUE_RELU;
+    ok = ok && a.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue)) == HIPBLAS_STATUS_SUCCESS;
   }
+  if (bias) {
+    const hipDataType bias_type = HIP_R_32F;
+    const void* bias_ptr = bias;
+    ok = ok && a.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type)) == HIPBLAS_STATUS_SUCCESS &&
+         a.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias_ptr, sizeof(bias_ptr)) == HIPBLAS_STATUS_SUCCESS;
+  }
+  const hipDataType out_type = out_f32 ? HIP_R_32F : HIP_R_16BF;
   ok = ok && a.layout_create(&p.w, HIP_R_16BF, K, N, K) == HIPBLAS_STATUS_SUCCESS &&
        a.layout_create(&p.x, HIP_R_16BF, K, M, K) == HIPBLAS_STATUS_SUCCESS &&
-       a.layout_create(&p.c, HIP_R_32F, N, M, N) == HIPBLAS_STATUS_SUCCESS;
+       a.layout_create(&p.c, out_type, N, M, N) == HIPBLAS_STATUS_SUCCESS;
   if (!ok) return p;
   hipblasLtMatmulPreference_t pref = nullptr;
   if (a.pref_create(&pref) != HIPBLAS_STATUS_SUCCESS) return p;
-  constexpr int WANTED = 4;
-  hipblasLtMatmulHeuristicResult_t found[WANTED];
+  hipblasLtMatmulHeuristicResult_t found[CANDIDATES];
   int count = 0;
-  if (a.pref_set(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &workspace_bytes, sizeof(workspace_bytes)) ==
-          HIPBLAS_STATUS_SUCCESS &&
-      a.heuristic(handle, p.desc, p.w, p.x, p.c, p.c, pref, WANTED, found, &count) == HIPBLAS_STATUS_SUCCESS) {
-    for (int i = 0; i < count && i < WANTED; ++i) {
-      // an algorithm is taken only with all the workspace it asks for
-      if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= workspace_bytes) {
-        p.algo = found[i].algo;
-        p.workspace = found[i].workspaceSize;
-        p.usable = true;
-        break;
+  const size_t room = call.workspace_bytes;
+  if (a.pref_set(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &room, sizeof(room)) != HIPBLAS_STATUS_SUCCESS ||
+      a.heuristic(handle, p.desc, p.w, p.x, p.c, p.c, pref, CANDIDATES, found, &count) != HIPBLAS_STATUS_SUCCESS)
+    count = 0;
+  a.pref_destroy(pref);
+  int fits[CANDIDATES], n_fit = 0;
+  for (int i = 0; i < count && i < CANDIDATES; ++i)
+    if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= room) fits[n_fit++] = i;
+  if (n_fit == 0) return p;
+  int pick = fits[0];
+  if (flush && n_fit > 1) {
+    hipEvent_t begin = nullptr, end = nullptr;
+    if (hipEventCreate(&begin) == hipSuccess && hipEventCreate(&end) == hipSuccess) {
+      float best = -1.f;
+      for (int j = 0; j < n_fit; ++j) {
+        const float t = library_time(handle, p, found[fits[j]].algo, call, flush, flush_bytes, begin, end);
+        if (t >= 0.f && (best < 0.f || t < best)) {
+          best = t;
+          pick = fits[j];
+        }
       }
     }
+    if (begin) hipEventDestroy(begin);
+    if (end) hipEventDestroy(end);
   }
-  a.pref_destroy(pref);
+  p.algo = found[pick].algo;
+  p.workspace = found[pick].workspaceSize;
+  p.usable = true;
   return p;
 }
 }  // namespace
 
-extern "C" int tnx_gemm_sum_library(const void* x, const void* w, const float* bias, const float* residual, float* out,
-                                    int M, int N, int K, void* workspace, size_t workspace_bytes,
-                                    hipStream_t stream) {
-  TNX_REQUIRE(M > 0 && N > 0 && K > 0 && N % 8 == 0 && K % 8 == 0, "gemm_sum_library: bad sizes M=%d N=%d K=%d", M, N, K);
+extern "C" int tnx_gemm_library(const void* x, const void* w, const float* bias, const float* residual, void* out,
+                                int out_dtype, int act, int M, int N, int K, void* workspace, size_t workspace_bytes,
+                                void* flush, size_t flush_bytes, int tune, hipStream_t stream) {
+  TNX_REQUIRE(M > 0 && N > 0 && K > 0 && N % 8 == 0 && K % 8 == 0, "gemm_library: bad sizes M=%d N=%d K=%d", M, N, K);
+  TNX_REQUIRE(out_dtype == TNX_F32 || out_dtype == TNX_BF16, "gemm_library: the result is float32 or bfloat16");
+  TNX_REQUIRE(residual == nullptr || out_dtype == TNX_F32, "gemm_library: a residual is added to a float32 result only");
   TNX_REQUIRE(((uintptr_t)x | (uintptr_t)w | (uintptr_t)out | (uintptr_t)residual | (uintptr_t)bias |
                (uintptr_t)workspace) % 16 == 0,
-              "gemm_sum_library: operands must be 16-byte aligned");
-  TNX_REQUIRE(out != residual, "gemm_sum_library: the sum is not made in place");
+              "gemm_library: operands must be 16-byte aligned");
+  TNX_REQUIRE(out != (const void*)residual, "gemm_library: the sum is not made in place");
+  if (act != TNX_ACT_NONE && act != TNX_ACT_RELU) return 2;
   std::lock_guard<std::mutex> lock(library_mutex);
   if (!library_ready()) return 2;
   int device = 0;
@@ -645,10 +720,22 @@ extern "C" int tnx_gemm_sum_library(const void* x, const void* w, const float* b
     library_handles[device] = nullptr;
     return 2;
   }
-  const auto key = std::make_tuple(device, M, N, K, (bias ? 1 : 0) | (residual ? 2 : 0));
+  const LibraryCall call = {x, w, residual ? (const void*)residual : (const void*)out, out, residual ? 1.f : 0.f,
+                            workspace, workspace_bytes, stream};
+  const int what = (bias ? 1 : 0) | (residual ? 2 : 0) | (out_dtype == TNX_F32 ? 4 : 0) | (act == TNX_ACT_RELU ? 8 : 0);
+  const auto key = std::make_tuple(device, M, N, K, what);
   auto it = library_plans.find(key);
-  if (it == library_plans.end())
-    it = library_plans.emplace(key, make_plan(library_handles[device], M, N, K, bias != nullptr, workspace_bytes)).first;
+  if (it == library_plans.end()) {
+    bool timed = tune && M <= TUNED_ROWS;
+    if (timed) {
+      // nothing is timed inside a recording: the first choice of the library's ranking stands in there
+      hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+      if (hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) timed = false;
+    }
+    if (timed && (flush == nullptr || flush_bytes == 0)) return 3;
+    it = library_plans.emplace(key, make_plan(library_handles[device], M, N, K, bias, act == TNX_ACT_RELU,
+                                              out_dtype == TNX_F32, call, timed ? flush : nullptr, flush_bytes)).first;
+  }
   const LibraryPlan& p = it->second;
   if (!p.usable || p.workspace > workspace_bytes) return 2;
   if (bias) {
@@ -657,20 +744,16 @@ extern "C" int tnx_gemm_sum_library(const void* x, const void* w, const float* b
         HIPBLAS_STATUS_SUCCESS)
       return 2;
   }
-  const float one = 1.f, zero = 0.f;
-  const hipblasStatus_t st =
-      library_api.matmul(library_handles[device], p.desc, &one, w, p.w, x, p.x, residual ? &one : &zero,
-                         residual ? (const void*)residual : (const void*)out, p.c, out, p.c, &p.algo, workspace,
-                         workspace_bytes, stream);
+  const hipblasStatus_t st = library_run(library_handles[device], p, p.algo, call);
   if (st != HIPBLAS_STATUS_SUCCESS) {
-    tnx_set_error("gemm_sum_library: the library refused the product (status %d) for M=%d N=%d K=%d", (int)st, M, N, K);
+    tnx_set_error("gemm_library: the library refused the product (status %d) for M=%d N=%d K=%d", (int)st, M, N, K);
     return 1;
   }
   return 0;
 }
 #else
-extern "C" int tnx_gemm_sum_library(const void*, const void*, const float*, const float*, float*, int, int, int, void*,
-                                    size_t, hipStream_t) {
+extern "C" int tnx_gemm_library(const void*, const void*, const float*, const float*, void*, int, int, int, int, int,
+                                void*, size_t, void*, size_t, int, hipStream_t) {
   return 2;
 }
 #endif

@@ -39,8 +39,8 @@ _SIGNATURES = {
         "tnx_gemm_bf16_qkv": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
                               _c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int,
                               _c_int, _c_void_p],
-        "tnx_gemm_sum_library": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
-                                 _c_void_p, ctypes.c_size_t, _c_void_p],
+        "tnx_gemm_library": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
+                             _c_int, _c_void_p, ctypes.c_size_t, _c_void_p, ctypes.c_size_t, _c_int, _c_void_p],
     },
     "attention": {
         "tnx_qkv_write": [_c_void_p, _c_int, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
@@ -316,22 +316,16 @@ class HipOps:
             _want(residual, "residual", torch.float32, (m, n))
         out_dtype = torch.float32 if out_f32 else self.dtype
         if (self._library_product(m, n, k, w, force_tiled) and (residual is not None or not out_f32)):
-            # Many rows: the plain product goes to the vendor library (hipBLASLt through torch), and one
-            # kernel of ours does what follows it. Where the result stays bfloat16 the library adds the bias
-            # (and applies ReLU) before it rounds; with a residual, bias and sum are ours, in float32. The
-            # float32 head keeps our kernel: its output is not rounded to bfloat16 on the way.
+            # Many rows: the product goes to the vendor library (hipBLASLt), with what follows it where the
+            # library can do that itself: bias and ReLU before it rounds a bfloat16 result, or bias and the
+            # residual added to its float32 sums for a float32 result. The float32 head keeps our kernel.
             xa = self.cast(x, torch.bfloat16)
-            if residual is not None and out_f32 and act in (None, "none") and self.library_sum:
-                # the library itself adds bias and residual to its float32 sums: nothing is rounded on the way
-                out = torch.empty(m, n, dtype=torch.float32, device=x.device)
-                space = self._library_workspace(x.device)
-                rc = library("gemm").tnx_gemm_sum_library(_ptr(xa), _ptr(w), _ptr(bias), _ptr(residual), _ptr(out), m, n,
-                                                          k, _ptr(space), space.numel(), _stream())
-                if rc == 0:
+            if self.library_direct and act in (None, "none", "relu") and (residual is None or out_f32):
+                out = torch.empty(m, n, dtype=out_dtype, device=x.device)
+                if self._library_call(xa, w, bias, residual, out, act, m, n, k):
                     return out
-                if rc != 2:
-                    raise RuntimeError(f"tnx_gemm_sum_library: {library('gemm').tnx_last_error().decode()}")
-                # 2: not to be had here; the product through torch and the sum by our kernel, below
+            # Not to be had that way (another activation, no library to be found, no algorithm that fits):
+            # the product through torch, and one kernel of ours for what follows it.
             if bias is not None and residual is None and not out_f32:
                 b16 = self._bias_bf16(bias)
                 if act == "relu":
@@ -356,8 +350,31 @@ class HipOps:
                        _ptr(out), _code(out_dtype), _ACT[act], m, n, k, int(force_tiled), _stream())
         return out
 
-    library_sum = True      # out = x w^T + bias + residual in one call of the vendor library, where it is to be had
+    library_direct = True   # many-rows products as calls of the vendor library itself, with what follows them
+    library_tune = True     # and its algorithms timed once for products of few rows
     _workspaces: Dict[str, torch.Tensor] = {}
+
+    def _library_call(self, xa, w, bias, residual, out, act, m, n, k) -> bool:
+        """`out = act(xa w^T + bias) + residual` by the vendor library; False where that is not to be had."""
+        lib = library("gemm")
+        space = self._library_workspace(xa.device)
+
+        def call(flush, tune):
+            return lib.tnx_gemm_library(_ptr(xa), _ptr(w), _ptr(bias), _ptr(residual), _ptr(out), _code(out.dtype),
+                                        _ACT[act], m, n, k, _ptr(space), space.numel(), _ptr(flush),
+                                        flush.numel() if flush is not None else 0, int(tune), _stream())
+        rc = call(None, self.library_tune)
+        if rc == 3:
+            # the algorithms for this size are timed now, once: with memory to push the operands out of the
+            # caches, as large as the last-level cache; without it, if the device has no room, nothing is timed
+            try:
+                flush = torch.empty(256 << 20, dtype=torch.uint8, device=xa.device)
+            except torch.OutOfMemoryError:
+                flush = None
+            rc = call(flush, flush is not None)
+        if rc == 1:
+            raise RuntimeError(f"tnx_gemm_library: {lib.tnx_last_error().decode()}")
+        return rc == 0
 
     @classmethod
     def _library_workspace(cls, device) -> torch.Tensor:
