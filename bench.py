@@ -65,7 +65,7 @@ def main():
     ap.add_argument("--mix", action="store_true",
                     help="instead: 64 requests with prompts of 16 to 1,024 tokens and 256 new tokens each, all "
                          "queued at once (BASELINE.json's continuous-batching workload); prints its own line")
-    ap.add_argument("--big-batch", type=int, default=64, help="the larger batch of `points` (66b: 32 fits)")
+    ap.add_argument("--big-batch", type=int, default=64, help="the larger batch of `points` (cut to what fits the device at the full context)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -84,7 +84,24 @@ def main():
         raw["num_hidden_layers"] = args.layers
     cfg = OPTConfig.from_dict(raw)
     dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
-    max_batch = args.batch if args.no_points else max(args.batch, args.big_batch)
+    item = 2 if dtype == torch.bfloat16 else 4
+    kv_bytes_per_token = 2 * cfg.num_hidden_layers * cfg.hidden_size * item
+    # the larger batch of `points` is cut to what the device holds beside the weights at the full context
+    weights = item * (cfg.num_hidden_layers * (4 * cfg.hidden_size ** 2 + 2 * cfg.hidden_size * cfg.ffn_dim)
+                      + (cfg.vocab_size + cfg.max_position_embeddings) * cfg.hidden_size)
+    # (the random weights are drawn apart and fused afterwards: a quarter of them is held twice meanwhile, and
+    # what that leaves free again is in pieces too small for the cache's blocks)
+    room = int(0.95 * torch.cuda.mem_get_info()[1]) - int(1.27 * weights) - (4 << 30)
+    fits = max(1, room // (kv_bytes_per_token * CONTEXT))
+    if args.big_batch > fits and not (args.no_points or args.prefill_only):
+        print(f"[bench] {args.big_batch} requests of {CONTEXT} tokens do not fit beside {weights / 1e9:.0f} GB of "
+              f"weights; the larger batch is {fits}", file=sys.stderr, flush=True)
+        args.big_batch = fits
+    if args.batch > fits:
+        print(f"bench.py: {args.batch} requests of {CONTEXT} tokens do not fit beside {weights / 1e9:.0f} GB of weights "
+              f"on this device ({fits} do)")
+        return 2
+    max_batch = args.batch if args.no_points or args.prefill_only else max(args.batch, args.big_batch)
     ecfg = EngineConfig(dtype=dtype, page_size=64, max_tokens=max_batch * CONTEXT, max_num_seqs=max_batch,
                         max_num_batched_tokens=max(2048, PREFILL_TOKENS), max_model_len=CONTEXT,
                         prompts_first=True)
@@ -94,8 +111,6 @@ def main():
     print(f"[bench] model ready in {time.time() - t0:.1f} s "
           f"({runner.model.weight_bytes / 1e9:.2f} GB of weights)", file=sys.stderr, flush=True)
     engine = LLMEngine(runner, ecfg)
-    item = 2 if dtype == torch.bfloat16 else 4
-    kv_bytes_per_token = 2 * cfg.num_hidden_layers * cfg.hidden_size * item
     gen = torch.Generator().manual_seed(1)
 
     def decode(batch, steps, warmup):

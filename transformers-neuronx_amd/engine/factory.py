@@ -64,6 +64,10 @@ def build_runner(model_config, source, cfg: EngineConfig) -> ModelRunner:
     if hasattr(ops, "decode_copies"):
         ops.decode_copies = _room_for_weight_copies(cfg, model, bytes_per_page, device)
     model.load(source, ops, cfg.dtype, device)
+    if hasattr(source, "release"):
+        source.release()        # before the cache is sized and made: what the source held is free again,
+        if device.type == "cuda":  # and goes back to the device, so that the cache's large blocks find room
+            torch.cuda.empty_cache()
     num_pages = size_page_pool(cfg, bytes_per_page, device)
     cache = CacheManager(needs, cfg.page_size, num_pages, cfg.max_num_seqs, cfg.dtype, device)
     return ModelRunner(model, cache, ops, use_graphs=cfg.use_graphs)

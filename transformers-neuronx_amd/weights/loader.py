@@ -109,6 +109,10 @@ class TensorDict:
     def tensor(self, name):
         return self._t[name]
 
+    def release(self):
+        """The model is loaded: tensors it made its own forms of (the fused QKV matrix) are not held any longer."""
+        self._t.clear()
+
 
 def _base_model_name(name: str) -> Optional[str]:
     return name[len("model."):] if name.startswith("model.") else None
