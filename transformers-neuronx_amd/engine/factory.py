@@ -86,5 +86,5 @@ def runner_from_random(model_config, seed: int, cfg: EngineConfig) -> ModelRunne
     spec = arch.build_spec(model_config)
     decls = DecoderModel(spec).param_decls()
     storage = torch.float32 if cfg.dtype == torch.float32 else torch.bfloat16
-    tensors = random_tensors(decls, spec.init_std, seed, storage, device)
-    return build_runner(model_config, TensorDict(tensors), cfg)
+    source = TensorDict(random_tensors(decls, spec.init_std, seed, storage, device))
+    return build_runner(model_config, source, cfg)       # the source alone holds the tensors, and lets go of them

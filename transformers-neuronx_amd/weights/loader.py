@@ -92,7 +92,7 @@ class TensorDict:
     """The same interface over tensors held in memory (random weights without a folder)."""
 
     def __init__(self, tensors: Dict[str, torch.Tensor]):
-        self._t = tensors
+        self._t = dict(tensors)         # a map of its own: `release` empties this one, not the caller's
 
     def names(self):
         return list(self._t)
