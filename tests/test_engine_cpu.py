@@ -152,6 +152,46 @@ def test_running_ahead_changes_nothing_but_the_call_that_reports(tiny_folders, n
         assert outs == want and reasons == ["eos" if i == 3 else "length" for i in range(6)] and n > 0
 
 
+@pytest.mark.parametrize("run_ahead", [False, True])
+def test_prompts_first_ends_when_pages_run_out(tiny_folders, run_ahead):
+    """With `prompts_first` decoding requests wait for prompts, but a prompt that was put back for want of
+    pages can only go on when the decoding requests have gone on and ended: they must not wait for it. The
+    same holds when more requests wait than there are slots. The tokens are those of the other order."""
+    folder, cfg, weights = tiny_folders["A"]
+    prompts = list(_requests(cfg["vocab_size"], [30, 30, 30, 30, 30], 6).values())
+    sp = SamplingParams(max_new_tokens=40, do_sample=False, ignore_eos=True)
+
+    def generate(prompts_first, max_tokens, max_num_seqs=8):
+        cfg_ = EngineConfig(dtype="float32", kernels="reference", device="cpu", page_size=16, max_tokens=max_tokens,
+                            max_num_seqs=max_num_seqs, prompts_first=prompts_first, run_ahead=run_ahead)
+        runner = runner_from_folder(folder, cfg_)
+        engine = LLMEngine(runner, cfg_)
+        ids = [engine.add_request(p, sp) for p in prompts]
+        for _ in range(2000):
+            if not engine.has_work:
+                break
+            engine.step()
+        assert not engine.has_work, "the engine makes no progress"
+        runner.cache.check()
+        return [engine.requests[i].output for i in ids], engine.scheduler.num_preemptions
+
+    want, _ = generate(False, 512)
+    tight, n = generate(True, 128)               # 8 pages of 16 for 5 x 69 tokens
+    assert n > 0 and tight == want
+    few_slots, _ = generate(True, 512, max_num_seqs=2)
+    assert few_slots == want
+
+
+def test_a_step_that_plans_nothing_while_work_waits_raises(tiny_folders):
+    folder, cfg, _ = tiny_folders["A"]
+    runner, ecfg = _runner(folder, 128)
+    engine = LLMEngine(runner, ecfg)
+    engine.add_request([5, 6, 7], SamplingParams(max_new_tokens=4))
+    engine.scheduler.schedule = lambda: []          # a scheduler that has work and plans none of it
+    with pytest.raises(RuntimeError, match="no progress"):
+        engine.run()
+
+
 def test_sampled_tokens_follow_the_plain_sampler(tiny_folders):
     folder, cfg, weights = tiny_folders["A"]
     prompt = _requests(cfg["vocab_size"], [13], 4)["r0"]

@@ -56,6 +56,7 @@ class LLMEngine:
         self.logits_hook: Optional[Callable] = None
         self.run_ahead = bool(getattr(config, "run_ahead", True))
         self._started: Optional[_StartedStep] = None
+        self._planned = False                  # the last call of `step()` found something to run
 
     # ---------------------------------------------------------------- requests
 
@@ -82,6 +83,7 @@ class LLMEngine:
     def _start(self) -> Optional[_StartedStep]:
         """Plan a step, run it, choose its tokens on the device and record it with the tokens pending."""
         runs = self.scheduler.schedule()
+        self._planned = bool(runs)
         if not runs:
             return None
         t0 = time.perf_counter()
@@ -111,6 +113,7 @@ class LLMEngine:
             it = iter(self.runner.ops.receive_tokens(step.sent))
             tokens = [next(it) if r.samples else None for r in step.runs]
         kept = self.scheduler.resolve(step.runs, tokens)
+        self.scheduler.finished.clear()        # the engine reports ends through `StepOutput`; nothing piles up
         if self.record_timings:
             self.runner.ops.synchronize()
             self.timings.append({"seconds": time.perf_counter() - step.started,
@@ -142,7 +145,11 @@ class LLMEngine:
     def run(self, on_token: Optional[Callable[[StepOutput], None]] = None) -> None:
         """Step until every request has ended."""
         while self.has_work:
-            for out in self.step():
+            idle = self._started is None
+            outs = self.step()
+            if idle and not self._planned and self.scheduler.has_work:
+                raise RuntimeError("no progress: requests wait, the scheduler plans no step and none is under way")
+            for out in outs:
                 if on_token:
                     on_token(out)
 
@@ -152,13 +159,21 @@ class LLMEngine:
         plist = params if isinstance(params, (list, tuple)) else [params] * len(prompts)
         ids = [self.add_request(p, sp) for p, sp in zip(prompts, plist)]
         self.run()
-        return [list(self.requests[i].output) for i in ids]
+        return [list(self.pop_request(i).output) for i in ids]
+
+    def pop_request(self, req_id: Hashable) -> Request:
+        """Hand over a request that has ended and forget it. A request stays in `requests`, with its prompt
+        and output, until this is called (or `reset`): a caller that drives `step()` itself calls it when it
+        has seen the request's last token."""
+        req = self.requests[req_id]
+        if not req.finished:
+            raise ValueError(f"request {req_id!r} has not ended")
+        return self.requests.pop(req_id)
 
     def reset(self) -> None:
         """Forget every request and give back all pages (reference: `reset()` zero-fills
         the caches, decoder.py:1957-1969; here nothing needs clearing)."""
         self._started = None
-        self.scheduler.waiting.clear()
-        self.scheduler.running.clear()
+        self.scheduler.reset()
         self.runner.cache.reset()
         self.requests.clear()

@@ -38,10 +38,10 @@ class _Staging:
         n = flat.size
         self.turn ^= 1
         i = self.turn
+        if self.done[i] is not None:
+            self.done[i].synchronize()         # also before a buffer is replaced: its copy may still read it
         if self.buffers[i] is None or self.buffers[i][0].numel() < n:
             self.buffers[i] = self.ops.pinned_ints(max(2 * n, 1024))
-        elif self.done[i] is not None:
-            self.done[i].synchronize()
         self.buffers[i][0].numpy()[:n] = flat
         if dst is None:
             dst = torch.empty(n, dtype=torch.int32, device=device)

@@ -102,6 +102,7 @@ class Scheduler:
         self.finished: List[Request] = []
         self._arrivals = 0
         self.num_preemptions = 0
+        self._short = False      # pages have run out and no request has ended since
 
     # ---------------------------------------------------------------- arrivals
 
@@ -123,6 +124,14 @@ class Scheduler:
     @property
     def has_work(self) -> bool:
         return bool(self.waiting or self.running)
+
+    def reset(self) -> None:
+        """Forget every request and every count (the pages are the cache manager's to give back)."""
+        self.waiting.clear()
+        self.running.clear()
+        self.finished.clear()
+        self.num_preemptions = 0
+        self._short = False
 
     # ---------------------------------------------------------------- one step's plan
 
@@ -164,22 +173,33 @@ class Scheduler:
                 self._preempt_last(req)
                 planned[:] = [p for p in planned if p.request is not victim]
 
-    def schedule(self) -> List[ScheduledRun]:
-        budget = self.max_num_batched_tokens
-        before_all = self.num_preemptions     # a request can have left `running` only if something was put back
-        planned: List[ScheduledRun] = []
-        blocked = False                       # pages ran out: admit nothing new this step
-        # 1. one token for every decoding request, oldest first
-        hold = self.prompts_first and (bool(self.waiting) or any(not r.decoding for r in self.running))
+    def _plan_decoding(self, planned: List[ScheduledRun], budget: int, before_all: int) -> tuple:
+        """One token for every decoding request, oldest first. Returns (budget left, pages ran out)."""
+        blocked = False
         for req in list(self.running):
-            if hold or (self.num_preemptions != before_all and req not in self.running) or not req.decoding \
-                    or budget <= 0:
+            if (self.num_preemptions != before_all and req not in self.running) or not req.decoding or budget <= 0:
                 continue
             before = self.num_preemptions
             if self._reserve(req, req.num_computed + 1, planned):
                 planned.append(ScheduledRun(req, req.num_computed, 1))
                 budget -= 1
             blocked |= self.num_preemptions != before
+        return budget, blocked
+
+    def schedule(self) -> List[ScheduledRun]:
+        budget = self.max_num_batched_tokens
+        before_all = self.num_preemptions     # a request can have left `running` only if something was put back
+        planned: List[ScheduledRun] = []
+        blocked = False                       # pages ran out: admit nothing new this step
+        # With `prompts_first` decoding requests wait while a prompt is waiting or under way, but only as
+        # long as prompts can get on: once pages have run out (`_short`, until a request ends and frees
+        # some) the decoding requests go first again, since only they can end and free pages; and a step
+        # in which no prompt could be planned (no slot, no page) is given to them too.
+        hold = (self.prompts_first and not self._short
+                and (bool(self.waiting) or any(not r.decoding for r in self.running)))
+        # 1. one token for every decoding request, oldest first
+        if not hold:
+            budget, blocked = self._plan_decoding(planned, budget, before_all)
         # 2. the next portion of every prompt under way
         planned_ids = {id(p.request) for p in planned}
         for req in list(self.running):
@@ -205,12 +225,17 @@ class Scheduler:
                 if not self.running:
                     raise OutOfPages(f"request {req.req_id!r} alone does not fit the page pool "
                                      f"({req.num_computed + count} tokens wanted)")
+                self._short = True
                 break
             self.cache.grow(req.req_id, req.num_computed + count)
             self.waiting.popleft()
             self.running.append(req)
             planned.append(ScheduledRun(req, req.num_computed, count))
             budget -= count
+        if self.num_preemptions != before_all:
+            self._short = True
+        if hold and not planned:
+            budget, blocked = self._plan_decoding(planned, budget, before_all)
         # a request put back after it was planned is no longer in `running`
         live = {id(r) for r in self.running}
         return [p for p in planned if id(p.request) in live]
@@ -228,6 +253,7 @@ class Scheduler:
             self.waiting.remove(req)
         if self.cache.has(req.req_id):
             self.cache.free_request(req.req_id)
+        self._short = False
         self.finished.append(req)
         ended.append(req)
 

@@ -201,10 +201,10 @@ class HipOps:
         n = flat.size
         self._ints_turn ^= 1
         i = self._ints_turn
+        if self._ints_done[i] is not None:
+            self._ints_done[i].synchronize()   # also before a buffer is replaced: its copy may still read it
         if self._ints[i] is None or self._ints[i][0].numel() < n:
             self._ints[i] = self.pinned_ints(max(2 * n, 1024))
-        elif self._ints_done[i] is not None:
-            self._ints_done[i].synchronize()
         self._ints[i][0].numpy()[:n] = flat
         dst = torch.empty(n, dtype=torch.int32, device=self.device)
         self.copy_ints(dst, self._ints[i], n)
