@@ -144,6 +144,8 @@ class EngineConfig:
     max_tokens       the most tokens live requests hold at a time
     max_num_seqs     the most live requests (slots of per-request state)
     max_num_batched_tokens   token budget of one step
+    chunk_size       the most tokens of one prompt that one step takes (its portion); None: what is left
+                     of the step's token budget
     max_model_len    longest request (prompt + generated); capped by the model
     kernels          "hip" (the product path) or "reference" (the plain torch
                      rendition of every kernel, for debugging on any device;
@@ -157,6 +159,8 @@ class EngineConfig:
                      what fits beside the cache
     run_ahead        a step is started before the host has read the tokens of the step before it (they
                      stay on the device for it); generation is the same, tokens are reported one call later
+    seed             the random stream of a request whose `SamplingParams.seed` is None is keyed by this
+                     plus the number of requests the engine took before it
     """
     dtype: torch.dtype = torch.bfloat16
     page_size: int = 64
@@ -164,6 +168,7 @@ class EngineConfig:
     max_tokens: Optional[int] = None
     max_num_seqs: int = 64
     max_num_batched_tokens: int = 2048
+    chunk_size: Optional[int] = None
     max_model_len: Optional[int] = None
     kernels: str = "hip"
     device: str = "cuda:0"
@@ -182,3 +187,5 @@ class EngineConfig:
             raise ValueError(f"kernels must be 'hip' or 'reference', got {self.kernels!r}")
         if self.max_num_seqs <= 0 or self.max_num_batched_tokens <= 0:
             raise ValueError("max_num_seqs and max_num_batched_tokens must be positive")
+        if self.chunk_size is not None and self.chunk_size <= 0:
+            raise ValueError(f"chunk_size must be positive, got {self.chunk_size}")

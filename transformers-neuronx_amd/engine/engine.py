@@ -2,6 +2,7 @@
 function and the sampler; everything between a request's tokens and its next
 token passes through `step()`.
 """
+import dataclasses
 import itertools
 import time
 from dataclasses import dataclass
@@ -46,10 +47,11 @@ class LLMEngine:
         self.runner, self.config = runner, config
         max_len = min(config.max_model_len or runner.max_positions, runner.max_positions)
         self.scheduler = Scheduler(runner.cache, config.max_num_seqs, config.max_num_batched_tokens, max_len,
-                                   prompts_first=config.prompts_first)
+                                   max_portion=config.chunk_size, prompts_first=config.prompts_first)
         self.sampler = Sampler(runner.ops, runner.model.device)
         self.requests: Dict[Hashable, Request] = {}
         self._ids = itertools.count()
+        self._taken = 0                        # requests taken since the start or the last reset
         self.timings: List[dict] = []          # one record per step when `record_timings`
         self.record_timings = False
         # called with (requests that sample in this step, their logits [n, vocab] float32) before the draw
@@ -69,6 +71,10 @@ class LLMEngine:
         prompt = [int(t) for t in prompt]
         if prompt and not 0 <= min(prompt) <= max(prompt) < self.runner.vocab:
             raise ValueError(f"request {rid!r}: a token id of the prompt is outside the vocabulary of {self.runner.vocab}")
+        if params.seed is None:
+            # a stream of the request's own, the same whatever else runs beside it
+            params = dataclasses.replace(params, seed=int(self.config.seed) + self._taken)
+        self._taken += 1
         req = Request(rid, prompt, params)
         self.scheduler.add(req)
         self.requests[rid] = req
@@ -176,4 +182,5 @@ class LLMEngine:
         self._started = None
         self.scheduler.reset()
         self.runner.cache.reset()
+        self._taken = 0
         self.requests.clear()

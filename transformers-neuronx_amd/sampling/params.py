@@ -17,7 +17,8 @@ class SamplingParams:
     min_tokens_to_keep  neither filter leaves fewer tokens than this (:204-205, :232;
                  `top_p_min_tokens` of the `GenerationConfig`)
     seed         the request's own random stream: draw number n of the request uses the
-                 counter n, whatever else is in the batch
+                 counter n, whatever else is in the batch; None lets the engine give one
+                 (its own seed plus the request's number of arrival)
     deterministic  every draw uses 0.5 in place of a random number (hlo.py:2455-2456)
     ban_eos      the end-of-sequence token is never chosen (`scores[:, eos] = -inf`,
                  sampling.py:143-144, the OPT loop's behaviour)
@@ -29,7 +30,7 @@ class SamplingParams:
     temperature: float = 1.0
     top_k: int = 0
     top_p: float = 1.0
-    seed: int = 0
+    seed: Optional[int] = 0
     min_tokens_to_keep: int = 1
     deterministic: bool = False
     eos_token_id: Optional[int] = None

@@ -35,7 +35,7 @@ class Sampler:
         temp = np.array([0.0 if p.greedy else p.temperature for p in params], dtype=np.float32)
         top_k = np.array([p.top_k for p in params], dtype=np.int32)
         top_p = np.array([p.top_p for p in params], dtype=np.float32)
-        seeds = np.array([p.seed for p in params], dtype=np.int64)
+        seeds = np.array([p.seed or 0 for p in params], dtype=np.int64)
         counters = np.array([-1 if p.deterministic else n for p, n in zip(params, draws)], dtype=np.int64)
         least = np.array([p.min_tokens_to_keep for p in params], dtype=np.int32)
         if hasattr(self.ops, "send_ints"):
