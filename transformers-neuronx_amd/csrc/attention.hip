@@ -6,6 +6,8 @@
 // A token at position p of run r lies in page table[r][p / page_size] at place p % page_size.
 // Reads are bounded by the reader's own position, so what an earlier holder left in a page is never seen.
 #include "common.h"
+#include "tnx_attention.h"
+#include <mutex>
 
 TNX_DEFINE_ERROR_API
 
@@ -1074,11 +1076,11 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, 
   }
 }
 
-extern "C" int tnx_attention_decode(const void* q, const void* k_pages, const void* v_pages, const int* run_start,
-                                    const int* cached_lens, const int* table, int table_width, int page_size,
-                                    int num_pages, const int* decode_runs, int num_decode, void* out, float* part_o,
-                                    float* part_ml, int num_heads, int num_kv, int head_size, int window,
-                                    int num_splits, int waves, const int* longest, hipStream_t stream) {
+static int attention_decode_run(const void* q, const void* k_pages, const void* v_pages, const int* run_start,
+                                const int* cached_lens, const int* table, int table_width, int page_size,
+                                int num_pages, const int* decode_runs, int num_decode, void* out, float* part_o,
+                                float* part_ml, int num_heads, int num_kv, int head_size, int window,
+                                int num_splits, int waves, const int* longest, hipStream_t stream) {
   TNX_REQUIRE(num_heads > 0 && num_kv > 0 && num_heads % num_kv == 0, "attention_decode: bad head counts");
   TNX_REQUIRE(head_size % 16 == 0 && head_size >= 16 && head_size <= 256,
               "attention_decode: head size %d is not a multiple of 16 in [16, 256]", head_size);
@@ -1123,4 +1125,64 @@ extern "C" int tnx_attention_decode(const void* q, const void* k_pages, const vo
     TNX_CHECK_LAUNCH("attention_decode_merge");
   }
   return 0;
+}
+
+extern "C" int tnx_attention_decode(const void* q, const void* k_pages, const void* v_pages, const int* run_start,
+                                    const int* cached_lens, const int* table, int table_width, int page_size,
+                                    int num_pages, const int* decode_runs, int num_decode, void* out, float* part_o,
+                                    float* part_ml, int num_heads, int num_kv, int head_size, int window,
+                                    int num_splits, int waves, const int* longest, hipStream_t stream) {
+  return attention_decode_run(q, k_pages, v_pages, run_start, cached_lens, table, table_width, page_size, num_pages,
+                              decode_runs, num_decode, out, part_o, part_ml, num_heads, num_kv, head_size, window,
+                              num_splits, waves, longest, stream);
+}
+
+// The partial results of split keys for callers that cannot allocate: one array per GPU, held until the
+// process ends. In host code this name is a stand-in, not a device address: the address on the current
+// device comes from hipGetSymbolAddress, once per device, and only that address is handed to kernels.
+static __device__ __align__(256) float tnx_decode_scratch[TNX_DECODE_SCRATCH_FLOATS];
+
+#define TNX_MAX_DEVICES 64
+static float* decode_scratch_of_device[TNX_MAX_DEVICES];
+static std::mutex decode_scratch_lock;
+
+extern "C" int tnx_attention_decode_static(const void* q, const void* k_pages, const void* v_pages,
+                                           const int* run_start, const int* cached_lens, const int* table,
+                                           int table_width, int page_size, int num_pages, const int* decode_runs,
+                                           int num_decode, void* out, int num_heads, int num_kv, int head_size,
+                                           int window, int num_splits, int waves, const int* longest,
+                                           hipStream_t stream) {
+  TNX_REQUIRE(num_decode >= 0 && num_heads > 0 && head_size > 0 && num_splits >= 1,
+              "attention_decode_static: bad sizes");
+  const long long partials = (long long)num_decode * num_heads * num_splits;
+  const long long floats = num_splits > 1 ? partials * (head_size + 2) : 0;
+  TNX_REQUIRE(floats <= TNX_DECODE_SCRATCH_FLOATS,
+              "attention_decode_static: %d requests x %d heads x %d splits at head size %d need %lld floats of "
+              "partial results; the static array holds %d. Use fewer splits, or tnx_attention_decode with a "
+              "workspace of the caller's",
+              num_decode, num_heads, num_splits, head_size, floats, (int)TNX_DECODE_SCRATCH_FLOATS);
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  TNX_REQUIRE(e == hipSuccess && device >= 0 && device < TNX_MAX_DEVICES,
+              "attention_decode_static: no current device (%s)", hipGetErrorString(e));
+  float* scratch;
+  {
+    std::lock_guard<std::mutex> hold(decode_scratch_lock);
+    if (decode_scratch_of_device[device] == nullptr) {
+      float* address = nullptr;
+      e = hipGetSymbolAddress((void**)&address, HIP_SYMBOL(tnx_decode_scratch));
+      TNX_REQUIRE(e == hipSuccess && address != nullptr,
+                  "attention_decode_static: the static array has no address on device %d (%s)", device,
+                  hipGetErrorString(e));
+      decode_scratch_of_device[device] = address;
+    }
+    scratch = decode_scratch_of_device[device];
+  }
+  // weighted values first, then (maximum, sum) pairs; every partial that the merge reads is written by this
+  // call's first kernel, so nothing of an earlier call's contents has to be cleared
+  float* part_o = scratch;
+  float* part_ml = scratch + partials * head_size;
+  return attention_decode_run(q, k_pages, v_pages, run_start, cached_lens, table, table_width, page_size, num_pages,
+                              decode_runs, num_decode, out, part_o, part_ml, num_heads, num_kv, head_size, window,
+                              num_splits, waves, longest, stream);
 }

@@ -44,7 +44,9 @@ def find_hipcc() -> Optional[str]:
 
 def source_hash(module: str) -> str:
     h = hashlib.sha256()
-    for name in (f"{module}.hip", "common.h"):
+    for name in (f"{module}.hip", "common.h", f"tnx_{module}.h"):
+        if name.startswith("tnx_") and not os.path.exists(os.path.join(CSRC, name)):
+            continue                       # a header of its own entry points: not every module has one
         with open(os.path.join(CSRC, name), "rb") as fp:
             h.update(fp.read())
     h.update(" ".join(FLAGS).encode())
