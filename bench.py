@@ -72,7 +72,8 @@ def main():
         return 2
 
     import torch
-    from transformers_neuronx_amd.config import EngineConfig, OPTConfig
+    from transformers_neuronx_amd.config import EngineConfig
+    from transformers_neuronx_amd.opt.config import OPTConfig
     from transformers_neuronx_amd.engine.engine import LLMEngine
     from transformers_neuronx_amd.engine.factory import runner_from_random
     from transformers_neuronx_amd.sampling import SamplingParams

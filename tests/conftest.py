@@ -52,7 +52,7 @@ TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
 def tiny_folders(tmp_path_factory):
     """{name: (folder, raw config, float32 tensors by name)} of the two tiny models, float32 on disk."""
     from safetensors.torch import load_file
-    from transformers_neuronx_amd.config import OPTConfig
+    from transformers_neuronx_amd.opt.config import OPTConfig
     from transformers_neuronx_amd.weights import write_random_model
     out = {}
     for name, (raw, seed) in TINY.items():
@@ -68,7 +68,7 @@ def tiny_folders(tmp_path_factory):
 def tiny_folders_bf16(tmp_path_factory):
     """The same models with matrices stored in bfloat16 (norm parameters and biases in float32)."""
     from safetensors.torch import load_file
-    from transformers_neuronx_amd.config import OPTConfig
+    from transformers_neuronx_amd.opt.config import OPTConfig
     from transformers_neuronx_amd.weights import write_random_model
     out = {}
     for name, (raw, seed) in TINY.items():

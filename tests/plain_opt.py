@@ -1,7 +1,7 @@
 """A plain, slow OPT: whole sequences, no cache, no batching, one function per part.
 
 It is written from the formulas in the reference (paths below are relative to
-`/root/reference/src/transformers_neuronx/`) and shares no code with the
+the reference's package folder `src/transformers_neuronx/`) and shares no code with the
 package under test. It takes the model as a dict of config.json keys and a dict
 of tensors by checkpoint name, and works in any floating dtype (float32 by
 default; float64 to tell which of two float32 results is the more exact).
@@ -158,9 +158,11 @@ def embed(tokens, w, cfg):
 def head(x, w, cfg):
     """layers/transformer.py:196-208: final LayerNorm, then logits with the
     `[vocab, width]` head weight, which is the token table when absent
-    (opt/model.py:204-205). The final norm exists in pre-norm order only;
-    `project_out` (no bias) comes before the head when the widths differ."""
-    if cfg.get("do_layer_norm_before", True):
+    (opt/model.py:204-205). The final norm exists in pre-norm order only, and not
+    when the configuration's `_remove_final_layer_norm` (a key the reference lists,
+    opt/gen_random_pretrained.py:114, and never reads) is true: parity unpinned for
+    that key; `project_out` (no bias) comes before the head when the widths differ."""
+    if cfg.get("do_layer_norm_before", True) and not cfg.get("_remove_final_layer_norm", False):
         g, b = _norm_params(w, "model.decoder.final_layer_norm", cfg.get("layer_norm_elementwise_affine", True))
         x = layer_norm(x, g, b, cfg.get("layer_norm_eps", 1e-5))
     if cfg.get("word_embed_proj_dim", cfg["hidden_size"]) != cfg["hidden_size"]:

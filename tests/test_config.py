@@ -5,7 +5,8 @@ import pytest
 
 from conftest import TINY_A, TINY_B
 from transformers_neuronx_amd.config import (ConfigError, EngineConfig, NeuronConfig, ContinuousBatchingConfig,
-                                             OPTConfig, known_architectures, parse_dtype, read_config, resolve)
+                                             known_architectures, parse_dtype, read_config, resolve)
+from transformers_neuronx_amd.opt.config import OPTConfig
 
 
 def test_reads_every_key():
@@ -64,7 +65,7 @@ def test_registry():
     with pytest.raises(ConfigError, match="known architectures"):
         resolve({"architectures": ["LlamaForCausalLM"], "model_type": "llama"})
     from transformers_neuronx_amd.opt.model import OPTForSampling
-    assert resolve({"model_type": "opt"}).model_class is OPTForSampling
+    assert resolve({"model_type": "opt"}).user_class() is OPTForSampling
 
 
 def test_engine_config():

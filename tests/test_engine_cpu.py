@@ -10,7 +10,8 @@ import torch
 import plain_opt
 import schedules
 from conftest import TINY
-from transformers_neuronx_amd.config import EngineConfig, OPTConfig
+from transformers_neuronx_amd.config import EngineConfig
+from transformers_neuronx_amd.opt.config import OPTConfig
 from transformers_neuronx_amd.engine import StepEntry
 from transformers_neuronx_amd.engine.engine import LLMEngine
 from transformers_neuronx_amd.engine.factory import runner_from_folder
@@ -399,3 +400,78 @@ def run_toy_routed_model(ops_kind, dtype, device, tol):
 
 def test_toy_routed_parts_on_the_host():
     run_toy_routed_model("reference", torch.float32, "cpu", 2e-5)
+
+
+def run_toy_rotating_model(ops_kind, dtype, device, tol):
+    """Attention whose queries and keys are turned by an encoding defined in the tests, a norm that brings a
+    kernel of its own, tensor names of its own: built from the registries and stepped under every way of
+    cutting, without a change to the framework."""
+    import toy_parts
+    from transformers_neuronx_amd.cache import CacheManager
+    from transformers_neuronx_amd.engine import DecoderModel, ModelRunner
+    from transformers_neuronx_amd.kernels import make_ops
+    from transformers_neuronx_amd.weights import TensorDict, random_tensors
+    spec = toy_parts.toy_spec_rotating()
+    model = DecoderModel(spec)
+    tensors = random_tensors(model.param_decls(), spec.init_std, 6, torch.float32)
+    assert "blocks.1.attn.wk.weight" in tensors and tensors["blocks.0.attn.wk.weight"].shape == (32, 96)
+    ops = make_ops(ops_kind, dtype, device)
+    model.load(TensorDict(tensors), ops, dtype, device)
+    runner = ModelRunner(model, CacheManager(model.cache_needs(), 16, 12, 4, dtype, device), ops, use_graphs=True)
+    requests = _requests(157, [70, 33, 100], 10)
+    expected = {rid: toy_parts.toy_rotating_plain_logits(tensors, toks) for rid, toks in requests.items()}
+    for steps, place in (schedules.whole(requests), schedules.portions(requests),
+                         schedules.mixed(requests, max_tokens=192, page=16, seed=2, tail=8, max_live=3)):
+        for rec in steps:
+            logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in rec["entries"]])
+            for row in range(logits.shape[0]):
+                rid, pos = place[(rec["step"], row)]
+                want = expected[rid][pos]
+                err = float((logits[row].cpu() - want).abs().max() / want.abs().max())
+                assert err < tol, (rec["step"], rid, pos, err)
+            for rid in rec["end"]:
+                runner.finish(rid)
+            runner.cache.check()
+        assert not runner.cache.requests
+
+
+def test_toy_rotating_parts_on_the_host():
+    run_toy_rotating_model("reference", torch.float32, "cpu", 2e-5)
+
+
+def test_toy_rotation_counts_distances_only():
+    """What pins the toy's plain form: with every position shifted by the same amount the logits stay; with
+    the keys turned the other way (a wrong sign) they would not."""
+    import toy_parts
+    from transformers_neuronx_amd.engine import DecoderModel
+    from transformers_neuronx_amd.weights import random_tensors
+    spec = toy_parts.toy_spec_rotating()
+    tensors = random_tensors(DecoderModel(spec).param_decls(), spec.init_std, 6, torch.float32)
+    toks = _requests(157, [40], 3)["r0"]
+    a = toy_parts.toy_rotating_plain_logits(tensors, toks)
+    b = toy_parts.toy_rotating_plain_logits(tensors, toks, first_position=37)
+    assert float((a - b).abs().max() / a.abs().max()) < 1e-4
+    c = toy_parts.toy_rotating_plain_logits(tensors, toks[::-1])
+    assert float((a - c).abs().max() / a.abs().max()) > 1e-2       # and positions do matter
+
+
+def test_model_without_the_norm_before_the_head(tmp_path):
+    """`_remove_final_layer_norm` of an OPT config.json: the engine and the plain implementation both leave
+    the norm out, and a model that keeps it answers differently."""
+    from safetensors.torch import load_file
+    from transformers_neuronx_amd.weights import write_random_model
+    from conftest import TINY_A
+    raw = dict(TINY_A, _remove_final_layer_norm=True)
+    folder = write_random_model(OPTConfig.from_dict(raw), str(tmp_path / "m"), 3, dtype="float32")
+    weights = load_file(folder + "/model.safetensors")
+    toks = _requests(512, [23], 1)["r0"]
+    runner, _ = _runner(folder, 64)
+    got = runner.step([StepEntry("a", toks, list(range(len(toks))))])
+    want = plain_opt.forward_logits(weights, raw, toks)
+    assert float((got - want).abs().max()) < 1e-5
+    g = torch.Generator().manual_seed(0)
+    with_norm = dict(weights)
+    with_norm["model.decoder.final_layer_norm.weight"] = 1 + 0.5 * torch.randn(64, generator=g)
+    with_norm["model.decoder.final_layer_norm.bias"] = torch.randn(64, generator=g)
+    other = plain_opt.forward_logits(with_norm, TINY_A, toks)
+    assert float((other - want).abs().max()) > 1e-2

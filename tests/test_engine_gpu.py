@@ -63,7 +63,7 @@ CASES = [("A", [5, 17, 31, 100, 128]), ("B", [1, 9, 40, 77, 120, 256]), ("C", [3
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name,lengths", CASES)
-@pytest.mark.parametrize("page_size", [16, 64])
+@pytest.mark.parametrize("page_size", [16, 64, 48])     # 48: no power of two, the general kernels take it
 def test_schedules_agree_with_plain(tiny_folders, tiny_folders_bf16, tmp_path, dtype, name, lengths, page_size):
     folder, cfg, weights = (tiny_folders if dtype == "float32" else tiny_folders_bf16)[name]
     requests = _requests(cfg, lengths, seed=len(lengths))
@@ -127,7 +127,7 @@ def test_pages_are_used_again_without_leaking(tiny_folders, tmp_path):
 def test_greedy_generation_through_the_entry_point(tiny_folders, amp, tmp_path):
     from safetensors.torch import load_file
     from transformers_neuronx_amd import OPTForSampling
-    from transformers_neuronx_amd.config import OPTConfig
+    from transformers_neuronx_amd.opt.config import OPTConfig
     from transformers_neuronx_amd.kernels import hip
     from transformers_neuronx_amd.weights import write_random_model
     # with weights as narrow as A's the greedy path repeats one token; a third model has A's sizes and
@@ -183,6 +183,16 @@ def test_toy_routed_parts_on_the_gpu(dtype):
     """A routed feed-forward and another position encoding, defined in the tests, on the HIP backend."""
     from test_engine_cpu import run_toy_routed_model
     run_toy_routed_model("hip", dtype, DEV, 2e-5 if dtype == torch.float32 else 3e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_toy_rotating_parts_on_the_gpu(dtype):
+    """Queries and keys turned by an encoding of the tests, and a norm whose HIP kernel lives under tests/
+    and is registered, compiled and called without a change to the package."""
+    from test_engine_cpu import run_toy_rotating_model
+    from transformers_neuronx_amd.kernels import hip
+    run_toy_rotating_model("hip", dtype, DEV, 2e-5 if dtype == torch.float32 else 3e-2)
+    assert "toy_norm" in hip.loaded_libraries()
 
 
 def test_trace_run_as_a_program(tiny_folders, tmp_path):
@@ -283,51 +293,61 @@ FULL_SIZES = {
 
 
 @pytest.mark.parametrize("size", list(FULL_SIZES))
-def test_bfloat16_against_float32_at_full_layer_sizes(size):
+def test_full_layer_sizes_against_plain(size):
     """A few layers of the sizes of OPT-6.7B (width 4096, 32 heads of 128, inner width 16384, vocabulary
-    50272), OPT-2.7B and OPT-350m: the bfloat16 engine against the float32 engine on the same (bfloat16-stored) random weights,
-    under a schedule that takes a long prompt in portions, decodes beside another prompt, and ends with
-    recorded decode steps. The reference's own yardstick for such a pair is `allclose(atol=1.0,
-    rtol=1e-3)` with equal argmax (generation_demo.py:437-443); here the bound is the bfloat16 one of the
-    other tests."""
-    from transformers_neuronx_amd.config import EngineConfig, OPTConfig
+    50272), OPT-2.7B and OPT-350m on bfloat16-stored random weights: the float32 engine and the bfloat16
+    engine against the plain implementation, under a schedule that takes a long prompt in portions, decodes
+    beside another prompt, and ends with recorded decode steps. The reference's own yardstick for a
+    low-precision run against a float32 one is `allclose(atol=1.0, rtol=1e-3)` with equal argmax
+    (generation_demo.py:437-443); here the bounds are those of the other tests."""
+    from transformers_neuronx_amd.config import EngineConfig
+    from transformers_neuronx_amd.opt.config import OPTConfig
     from transformers_neuronx_amd.engine import DecoderModel, StepEntry
     from transformers_neuronx_amd.engine.factory import build_runner
     from transformers_neuronx_amd.opt.spec import opt_spec
     from transformers_neuronx_amd.weights import TensorDict, random_tensors
     cfg = OPTConfig.from_dict(FULL_SIZES[size])
+    raw = cfg.to_dict()
     spec = opt_spec(cfg)
     tensors = random_tensors(DecoderModel(spec).param_decls(), spec.init_std, 3, torch.bfloat16, DEV)
     g = torch.Generator().manual_seed(0)
-    long = torch.randint(3, cfg.vocab_size, (700,), generator=g).tolist()
+    long = torch.randint(3, cfg.vocab_size, (420,), generator=g).tolist()
     short = torch.randint(3, cfg.vocab_size, (40,), generator=g).tolist()
+    # (request, first token, count, wanted places) step by step
+    plan = [[("a", 0, 300, [299])], [("a", 300, 110, [0, 109])], [("a", 410, 1, [0]), ("b", 0, 30, [29])]]
+    plan += [[("a", 411 + i, 1, [0]), ("b", 30 + i, 1, [0])] for i in range(9)]
+    toks = {"a": long, "b": short}
+    # the plain implementation: each request whole, then the head on the wanted positions only
+    weights = {k: v.float().cpu() for k, v in tensors.items()}
+    hidden = {}
+    for rid, t in toks.items():
+        x = plain_opt.embed(torch.tensor(t), weights, raw)
+        for i in range(cfg.num_hidden_layers):
+            x = plain_opt.block(x, weights, raw, i)
+        hidden[rid] = x
+    places = [(rid, first + w) for step in plan for rid, first, n, want in step for w in want]
+    want = torch.cat([plain_opt.head(hidden[rid][pos:pos + 1], weights, raw) for rid, pos in places])
+    scale = float(want.abs().max())
+    top2 = want.topk(2, dim=-1).values
 
     def run(dtype):
         ecfg = EngineConfig(dtype=dtype, page_size=64, max_tokens=1024, max_num_seqs=4)
         runner = build_runner(cfg, TensorDict(tensors), ecfg)
         rows = []
-
-        def step(parts):
-            entries, n = [], 0
-            for rid, toks, want in parts:
-                entries.append(StepEntry(rid, toks, want))
-                n += len(want)
-            rows.append(runner.step(entries).float().cpu())
-        step([("a", long[:300], [299])])
-        step([("a", long[300:650], [0, 349])])
-        step([("a", long[650:651], [0]), ("b", short[:30], [29])])        # one token beside a portion
-        for i in range(651, 660):
-            step([("a", long[i:i + 1], [0]), ("b", short[i - 621:i - 620], [0])])   # recorded decode steps
+        for step in plan:
+            rows.append(runner.step([StepEntry(rid, toks[rid][first:first + n], w) for rid, first, n, w in step])
+                        .float().cpu())
+        assert runner.graph_replays == 9
         return torch.cat(rows)
 
-    low, high = run("bfloat16"), run("float32")
-    scale = float(high.abs().max())
-    err = float((low - high).abs().max()) / scale
-    assert err <= TOL["bfloat16"], err
-    # where float32 has a clear winner bfloat16 names the same token
-    top2 = high.topk(2, dim=-1).values
-    clear = (top2[:, 0] - top2[:, 1]) > 4 * TOL["bfloat16"] * scale
-    assert bool((low.argmax(-1) == high.argmax(-1))[clear].all())
+    for dtype in ("float32", "bfloat16"):
+        got = run(dtype)
+        err = float((got - want).abs().max()) / scale
+        assert err <= TOL[dtype], (dtype, err)
+        # where the plain implementation has a clear winner the engine names the same token
+        clear = (top2[:, 0] - top2[:, 1]) > 4 * TOL[dtype] * scale
+        assert bool(clear.any()), "no row has a clear winner: the comparison of choices would be empty"
+        assert bool((got.argmax(-1) == want.argmax(-1))[clear].all())
 
 
 def _odd(v, heads, hs, layers, ffn, proj, pre, act, bias, affine, eps):
@@ -358,7 +378,7 @@ ODD = [
 @pytest.mark.parametrize("index", range(len(ODD)))
 def test_odd_sizes(tmp_path, dtype, index):
     from safetensors.torch import load_file
-    from transformers_neuronx_amd.config import OPTConfig
+    from transformers_neuronx_amd.opt.config import OPTConfig
     from transformers_neuronx_amd.weights import write_random_model
     raw = ODD[index]
     folder = str(tmp_path / "model")
@@ -377,7 +397,7 @@ def test_odd_sizes(tmp_path, dtype, index):
 def test_command_line_dump_and_analyze(tiny_folders, tmp_path, capsys):
     """`opt_demo run --dump_logits` writes the logits each token was chosen from; `analyze` compares two
     runs by the reference's yardstick (generation_demo.py:404-443) and fails when they differ."""
-    from transformers_neuronx_amd.config import OPTConfig
+    from transformers_neuronx_amd.opt.config import OPTConfig
     from transformers_neuronx_amd.opt import demo
     folder, cfg, weights = tiny_folders["A"]
     prompt = [5, 17, 3, 200, 9]

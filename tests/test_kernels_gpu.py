@@ -153,6 +153,11 @@ ATTN_CASES = [
     (3, 3, 80, 64, [1, 1], [700, 1300]),
     (2, 2, 112, 16, [1, 5], [900, 40]),
     (2, 1, 96, 32, [1, 1, 1], [300, 5, 64]),
+    # pages whose size is no power of two: prompts alone (the prompt kernel without LDS staging) and
+    # prompts beside decoded tokens (the general kernel)
+    (4, 2, 64, 48, [100, 7], [30, 200]),
+    (3, 3, 128, 80, [1, 50, 1], [170, 95, 3]),
+    (2, 2, 32, 48, [1, 1], [500, 47]),
 ]
 
 
@@ -258,6 +263,45 @@ def test_attention_finds_a_far_key():
                                torch.full_like(out_in, 5.0).float(), rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("mode", ["staged", "direct", "plain"])
+def test_windowed_attention_over_pages_given_back(mode):
+    """A windowed group gives back the pages its queries have passed: their table entries are -1, and the
+    first tile of keys a prompt kernel computes can hold such entries beside live pages. What lies in the
+    page such an entry is clamped to (here NaN) must not reach the result."""
+    dtype = torch.bfloat16
+    hip, ref = _ops(dtype)
+    if mode == "direct":
+        hip.prefill_direct = True
+    elif mode == "plain":
+        hip.force_plain_attention = True
+    heads, kv, hs, ps, window = 2, 1, 64, 16, 40
+    runs, cached = [70, 1, 20], [100, 130, 64]
+    num_pages = 40
+    ctx = _make_step(runs, cached, ps, num_pages - 1, seed=4)
+    view = ctx.groups["full"]
+    tab = view.block_table.cpu().numpy().copy()
+    tab[tab >= 0] += 1                                             # page 0 of the pool is no one's
+    for i, c in enumerate(cached):
+        gone = max(0, c - window + 1) // ps                        # pages wholly below the first query's window
+        tab[i, :gone] = -1
+    assert (tab[0, :3] == -1).all() and tab[0, 3] >= 0             # keys 0..47 gone, 48..63 live: one tile
+    view.block_table.copy_(torch.from_numpy(tab).to(DEV))
+    g = torch.Generator(device=DEV).manual_seed(12)
+    kp = torch.randn(num_pages, kv, ps, hs, device=DEV, generator=g).to(dtype)
+    vp = torch.randn(num_pages, kv, hs, ps, device=DEV, generator=g).to(dtype)
+    q = (torch.randn(ctx.num_tokens, heads * hs, device=DEV, generator=g) / 8).to(dtype)
+    want = ref.attention(q, heads, kv, hs, ctx, view, kp, vp, window)
+    # every page that no table names holds NaN now, page 0 (where -1 is clamped to) among them
+    live = set(tab[tab >= 0].tolist())
+    for page in range(num_pages):
+        if page not in live:
+            kp[page] = float("nan")
+            vp[page] = float("nan")
+    got = hip.attention(q, heads, kv, hs, ctx, view, kp, vp, window)
+    assert not torch.isnan(got.float()).any()
+    torch.testing.assert_close(got.float(), want.float(), rtol=2e-2, atol=2e-2)
+
+
 def test_attention_refuses_bad_head_size():
     hip, _ = _ops(torch.float32)
     ctx = _make_step([1], [0], 16, 2, seed=1)
@@ -281,27 +325,42 @@ def test_argmax_and_sampling(vocab):
     top_k = torch.tensor([0, 50, 1, 5, 0, vocab + 5] * 4, device=DEV, dtype=torch.int32)
     top_p = torch.tensor([1.0, 1.0, 0.9, 0.5, 0.3, 0.99, 1.0, 0.05] * 3, device=DEV)
     seeds = torch.arange(rows, device=DEV, dtype=torch.int64) * 7919 + 1
+
+    def same_or_on_a_boundary(t_h, t_r, top_p, counters, least=None):
+        """Every row is one of 24 different combinations of options, so every row must agree; a draw may
+        fall to the neighbouring token only where the random number lies on the boundary between the two
+        (within the rounding of the float32 sums), which the plain sampler's own sums show."""
+        import plain_opt
+        for i in torch.nonzero(t_h != t_r).flatten().tolist():
+            assert float(temp[i]) > 0 and int(top_k[i]) != 1, f"row {i} is greedy and differs"
+            n = int(counters[i])
+            u = 0.5 if n < 0 else plain_opt.philox_uniform(int(seeds[i]), n)
+            k = int(top_k[i]) or None
+            values, indices = plain_opt.filter_top_k_top_p(logits[i].cpu() / float(temp[i]), k, float(top_p[i]),
+                                                           int(least[i]) if least is not None else 1)
+            order = torch.argsort(indices)
+            cum = torch.cumsum(torch.softmax(values[order].double(), -1), -1)
+            kept = set(indices.tolist())
+            assert int(t_h[i]) in kept, f"row {i}: token {int(t_h[i])} is outside what the filters keep"
+            assert float((cum - u).abs().min()) < 1e-5, (i, int(t_h[i]), int(t_r[i]), u)
+
     for step in range(6):
         counters = torch.full((rows,), step, device=DEV, dtype=torch.int64)
         t_h = hip.sample(logits, temp, top_k, top_p, seeds, counters)
         t_r = ref.sample(logits, temp, top_k, top_p, seeds, counters)
-        assert (t_h == t_r).float().mean() >= 0.95, (t_h, t_r)    # a draw on a boundary may round either way
+        same_or_on_a_boundary(t_h, t_r, top_p, counters)
     # never fewer than `min_keep` tokens, and the constant 0.5 in place of a random number (counter < 0)
     least = torch.tensor([1, 3, 40, 7] * 6, device=DEV, dtype=torch.int32)
     tight_p = torch.full((rows,), 0.01, device=DEV)             # top-p alone would keep one token
     fixed = torch.full((rows,), -1, device=DEV, dtype=torch.int64)
     t_h = hip.sample(logits, temp, top_k, tight_p, seeds, fixed, least)
     t_r = ref.sample(logits, temp, top_k, tight_p, seeds, fixed, least)
-    assert (t_h == t_r).float().mean() >= 0.95, (t_h, t_r)
+    same_or_on_a_boundary(t_h, t_r, tight_p, fixed, least)
     for step in range(4):
         counters = torch.full((rows,), step, device=DEV, dtype=torch.int64)
         t_h = hip.sample(logits, temp, top_k, tight_p, seeds, counters, least)
         t_r = ref.sample(logits, temp, top_k, tight_p, seeds, counters, least)
-        assert (t_h == t_r).float().mean() >= 0.95, (t_h, t_r)
-        # a row that keeps 40 tokens does draw others than the best one
-    picks = torch.stack([hip.sample(logits, temp, top_k, tight_p, seeds,
-                                    torch.full((rows,), s, device=DEV, dtype=torch.int64), least) for s in range(12)])
-    assert len(set(picks[:, 2].tolist())) > 1 and len(set(picks[:, 4].tolist())) == 1
+        same_or_on_a_boundary(t_h, t_r, tight_p, counters, least)
 
 
 def test_sampling_distribution():

@@ -8,6 +8,7 @@ import torch
 import plain_opt
 
 pytestmark = pytest.mark.gpu
+QKVO = ("q_proj", "k_proj", "v_proj", "out_proj")     # the names the tests' tensors carry
 DEV = "cuda:0"
 
 
@@ -46,7 +47,7 @@ def test_norm_part(dtype, affine, eps):
 @pytest.mark.parametrize("act,bias", [("relu", True), ("gelu", False), ("gelu_new", True)])
 def test_feed_forward_part(dtype, act, bias):
     from transformers_neuronx_amd.parts import FEED_FORWARDS, PartSpec
-    ffn = FEED_FORWARDS.build(PartSpec("dense", dict(width=48, inner=136, activation=act, bias=bias)))
+    ffn = FEED_FORWARDS.build(PartSpec("dense", dict(up_name="fc1", down_name="fc2", width=48, inner=136, activation=act, bias=bias)))
     g = torch.Generator(device=DEV).manual_seed(1)
     t = {"p.fc1.weight": (torch.randn(136, 48, device=DEV, generator=g) / 7).to(dtype),
          "p.fc2.weight": (torch.randn(48, 136, device=DEV, generator=g) / 11).to(dtype),
@@ -95,7 +96,7 @@ def test_attention_part_in_two_steps(dtype, heads, kv, hs, bias, window):
     from transformers_neuronx_amd.engine.batch import StepEntry, build_context
     from transformers_neuronx_amd.parts import MIXERS, PartSpec
     width = heads * hs
-    mixer = MIXERS.build(PartSpec("attention", dict(width=width, num_heads=heads, head_size=hs, num_kv_heads=kv,
+    mixer = MIXERS.build(PartSpec("attention", dict(names=QKVO, width=width, num_heads=heads, head_size=hs, num_kv_heads=kv,
                                                     bias=bias, window=window)))
     g = torch.Generator(device=DEV).manual_seed(heads)
     t = {}
@@ -170,8 +171,8 @@ def test_block_arrangements(dtype, order):
     from transformers_neuronx_amd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, PartSpec, Stream)
     width, heads, hs, inner, n, ps = 64, 2, 32, 160, 23, 16
     norm = PartSpec("layer_norm", dict(width=width, eps=2e-5, affine=True))
-    mixer = MIXERS.build(PartSpec("attention", dict(width=width, num_heads=heads, head_size=hs)))
-    ffn = FEED_FORWARDS.build(PartSpec("dense", dict(width=width, inner=inner, activation="relu")))
+    mixer = MIXERS.build(PartSpec("attention", dict(names=QKVO, width=width, num_heads=heads, head_size=hs)))
+    ffn = FEED_FORWARDS.build(PartSpec("dense", dict(up_name="fc1", down_name="fc2", width=width, inner=inner, activation="relu")))
     n1, n2 = NORMS.build(norm), NORMS.build(norm)
     block = BLOCKS.build(PartSpec(order), mixer, ffn, n1, n2)
     named = [(mixer, "model.decoder.layers.0.self_attn."), (ffn, "model.decoder.layers.0."),

@@ -7,7 +7,7 @@ import torch
 from safetensors.torch import load_file, save_file
 
 from conftest import TINY_A, TINY_B
-from transformers_neuronx_amd.config import OPTConfig
+from transformers_neuronx_amd.opt.config import OPTConfig
 from transformers_neuronx_amd.engine.model import DecoderModel, model_param_decls
 from transformers_neuronx_amd.opt.spec import opt_spec
 from transformers_neuronx_amd.weights import (Checkpoint, TensorDict, WeightsError, check, load_tensors,
@@ -63,6 +63,8 @@ def test_dtype_rule():
     bf, f32, f16 = torch.bfloat16, torch.float32, torch.float16
     assert target_dtype("matrix", f16, bf) == bf and target_dtype("matrix", bf, bf) == bf
     assert target_dtype("matrix", f32, bf) == f32            # a tensor stored in 32-bit stays so
+    assert target_dtype("matrix", f32, bf, cast_float32=True) == bf      # unless its rounding is asked for
+    assert target_dtype("vector", f32, bf, cast_float32=True) == f32
     assert target_dtype("vector", bf, bf) == f32 and target_dtype("table", f16, bf) == bf
     assert target_dtype("matrix", bf, f32) == f32 and target_dtype("index", torch.int64, bf) == torch.int32
 
@@ -94,12 +96,21 @@ def test_base_model_names_and_untied_head(tmp_path):
     folder = write_random_model(cfg, str(tmp_path / "m"), seed=0, dtype="float32")
     t = load_file(folder + "/model.safetensors")
     stripped = {k[len("model."):] if k.startswith("model.") else k: v for k, v in t.items()}
-    got = load_tensors(_decls(TINY_A), TensorDict(stripped), torch.float32, "cpu")
+    got = load_tensors(_decls(TINY_A), TensorDict(stripped), torch.float32, "cpu", base_prefix="model.")
     assert torch.equal(got["model.decoder.layers.0.fc1.weight"], t["model.decoder.layers.0.fc1.weight"])
-    # a copy of the tied head in the file is accepted and not read
-    with_head = dict(t, **{"lm_head.weight": torch.zeros(512, 64)})
+    # the prefix a base model's checkpoint lacks is the architecture's to name, not the loader's
+    assert opt_spec(cfg).base_model_prefix == "model."
+    with pytest.raises(WeightsError, match="missing"):
+        load_tensors(_decls(TINY_A), TensorDict(stripped), torch.float32, "cpu")
+    # a copy of the tied head in the file is accepted when it says what the table says, and not read
+    with_head = dict(t, **{"lm_head.weight": t["model.decoder.embed_tokens.weight"].clone()})
     got = load_tensors(_decls(TINY_A), TensorDict(with_head), torch.float32, "cpu")
-    assert torch.equal(got["lm_head.weight"], t["model.decoder.embed_tokens.weight"])
+    assert got["lm_head.weight"] is got["model.decoder.embed_tokens.weight"]
+    # a head that differs from the table it is tied to belongs to another model: refused
+    with pytest.raises(WeightsError, match="tied tensors differ: lm_head.weight") as err:
+        load_tensors(_decls(TINY_A), TensorDict(dict(t, **{"lm_head.weight": torch.zeros(512, 64)})),
+                     torch.float32, "cpu")
+    assert err.value.tied_differ == [("lm_head.weight", "model.decoder.embed_tokens.weight")]
     # untied: the head is its own tensor and must be there
     untied = _decls(dict(TINY_A, tie_word_embeddings=False))
     with pytest.raises(WeightsError, match="lm_head.weight"):
@@ -128,3 +139,27 @@ def test_sharded_checkpoint(tmp_path):
     json.dump({"weight_map": weight_map}, open(os.path.join(folder, "model.safetensors.index.json"), "w"))
     got = load_tensors(_decls(TINY_A), Checkpoint(folder), torch.float32, "cpu")
     assert all(torch.equal(got[k], t[k]) for k in t)
+
+
+def test_what_is_said_about_dtypes_at_load(tmp_path, capsys):
+    """A bfloat16 engine says so when it keeps 32-bit matrices as they are (their products then run on the
+    float32 kernel), rounds them when asked to, and says when float16 storage loses bits."""
+    cfg = OPTConfig.from_dict(TINY_A)
+    folder = write_random_model(cfg, str(tmp_path / "m"), seed=0, dtype="float32")
+    kept = load_tensors(_decls(TINY_A), Checkpoint(folder), torch.bfloat16, "cpu")
+    assert kept["model.decoder.layers.0.fc1.weight"].dtype == torch.float32
+    assert "stored in 32-bit and stay so" in capsys.readouterr().err
+    cast = load_tensors(_decls(TINY_A), Checkpoint(folder), torch.bfloat16, "cpu", cast_float32=True)
+    assert cast["model.decoder.layers.0.fc1.weight"].dtype == torch.bfloat16
+    assert cast["model.decoder.layers.0.fc1.bias"].dtype == torch.float32
+    assert capsys.readouterr().err == ""
+    t = {k: (v.half() if v.dim() == 2 else v) for k, v in load_file(folder + "/model.safetensors").items()}
+    load_tensors(_decls(TINY_A), TensorDict(t), torch.bfloat16, "cpu")
+    assert "stored in float16 and are rounded to bfloat16" in capsys.readouterr().err
+
+
+def test_final_norm_can_be_left_out():
+    decls = {d.name for d in _decls(dict(TINY_A, _remove_final_layer_norm=True))}
+    assert "model.decoder.final_layer_norm.weight" not in decls
+    assert "model.decoder.layers.1.final_layer_norm.weight" in decls
+    assert "model.decoder.final_layer_norm.weight" in {d.name for d in _decls(TINY_A)}

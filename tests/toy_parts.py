@@ -10,6 +10,9 @@ from transformers_neuronx_amd.parts import (CacheNeed, LayerCall, LayerSpec, Mix
                                             register_mixer)
 
 
+QKVO = ("q_proj", "k_proj", "v_proj", "out_proj")     # the names the toy models give their attention tensors
+
+
 @register_mixer("toy_ema")
 class ToyEmaMixer(Mixer):
     """y_t = s_t, s_t = decay * s_{t-1} + (1 - decay) * (h_t W^T), s_{-1} = 0: a running average kept in a
@@ -47,15 +50,15 @@ class ToyEmaMixer(Mixer):
 def toy_spec(width=64, heads=4, inner=96, vocab=300, positions=160, window=24, eps=1e-5):
     hs = width // heads
     norm = PartSpec("layer_norm", dict(width=width, eps=eps, affine=True))
-    ffn = PartSpec("dense", dict(width=width, inner=inner, activation="gelu_new", bias=True))
+    ffn = PartSpec("dense", dict(up_name="fc1", down_name="fc2", width=width, inner=inner, activation="gelu_new", bias=True))
 
     def layer(i, mixer, block="pre_norm"):
         return LayerSpec(prefix=f"layers.{i}.", block=block, mixer=mixer, feed_forward=ffn, mixer_norm=norm,
                          feed_forward_norm=norm, mixer_name="mix.", feed_forward_name="ffn.",
                          mixer_norm_name="norm1", feed_forward_norm_name="norm2")
-    full = PartSpec("attention", dict(width=width, num_heads=heads, head_size=hs, num_kv_heads=heads // 2))
-    windowed = PartSpec("attention", dict(width=width, num_heads=heads, head_size=hs, window=window))
-    reader = PartSpec("attention", dict(width=width, num_heads=heads, head_size=hs, num_kv_heads=heads // 2,
+    full = PartSpec("attention", dict(names=QKVO, width=width, num_heads=heads, head_size=hs, num_kv_heads=heads // 2))
+    windowed = PartSpec("attention", dict(names=QKVO, width=width, num_heads=heads, head_size=hs, window=window))
+    reader = PartSpec("attention", dict(names=QKVO, width=width, num_heads=heads, head_size=hs, num_kv_heads=heads // 2,
                                         own_kv=False))
     ema = PartSpec("toy_ema", dict(width=width, decay=0.75))
     layers = (layer(0, full), layer(1, ema), layer(2, windowed), layer(3, reader))
@@ -182,9 +185,9 @@ def toy_spec_routed(width=48, heads=3, inner=40, experts=3, vocab=211, positions
     one (norms before); sinusoid positions; no norm before the head."""
     hs = width // heads
     norm = PartSpec("layer_norm", dict(width=width, eps=eps, affine=True))
-    attention = PartSpec("attention", dict(width=width, num_heads=heads, head_size=hs))
+    attention = PartSpec("attention", dict(names=QKVO, width=width, num_heads=heads, head_size=hs))
     routed = PartSpec("toy_routed", dict(width=width, inner=inner, experts=experts))
-    dense = PartSpec("dense", dict(width=width, inner=2 * inner, activation="relu", bias=False))
+    dense = PartSpec("dense", dict(up_name="fc1", down_name="fc2", width=width, inner=2 * inner, activation="relu", bias=False))
 
     def layer(i, ffn, block):
         return LayerSpec(prefix=f"layers.{i}.", block=block, mixer=attention, feed_forward=ffn, mixer_norm=norm,
@@ -232,3 +235,126 @@ def toy_routed_plain_logits(w, tokens, width=48, heads=3, experts=3, eps=1e-4, b
     h = torch.relu(plain_opt.linear(ln(x, p + "norm2"), w[p + "ffn.fc1.weight"]))
     x = x + plain_opt.linear(h, w[p + "ffn.fc2.weight"])
     return plain_opt.linear(x, w["embed.weight"])
+
+
+# ---------------------------------------------------------------- an encoding that turns queries and keys, a norm with a kernel of its own
+
+import ctypes  # noqa: E402
+import os  # noqa: E402
+
+from transformers_neuronx_amd.parts import Norm, register_norm  # noqa: E402
+
+TOY_KERNEL_SOURCE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "toy_kernels", "toy_norm.hip")
+
+
+def register_toy_kernels():
+    """The toy norm's kernel module: its source and its C signature, registered from outside the package."""
+    from transformers_neuronx_amd.kernels import build, hip
+    build.register_module("toy_norm", TOY_KERNEL_SOURCE)
+    vp, ci, cf = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+    hip.register_signatures("toy_norm", {"tnx_toy_scale_norm": [vp, vp, cf, vp, vp, ci, ci, ci, vp]})
+
+
+@register_position("toy_rotation")
+class ToyRotation(PositionEncoding):
+    """Turns every pair (x[2i], x[2i+1]) of each query and key head by the angle position * base^(-2i/head_size),
+    so that a score depends on the distance of query and key only. Torch operations on the device: a toy."""
+
+    def __init__(self, base: float):
+        self.base = base
+
+    def on_query_key(self, qkv, ctx, num_heads, num_kv_heads, head_size):
+        t = qkv.shape[0]
+        turned = (num_heads + num_kv_heads) * head_size            # queries and keys; values stay
+        x = qkv[:, :turned].float().reshape(t, -1, head_size // 2, 2)
+        freq = self.base ** (-torch.arange(head_size // 2, device=qkv.device, dtype=torch.float32) * 2 / head_size)
+        angle = ctx.positions.float()[:, None, None] * freq[None, None, :]
+        cos, sin = torch.cos(angle), torch.sin(angle)
+        out = torch.stack([x[..., 0] * cos - x[..., 1] * sin, x[..., 0] * sin + x[..., 1] * cos], dim=-1)
+        return torch.cat([out.reshape(t, turned).to(qkv.dtype), qkv[:, turned:]], dim=1).contiguous()
+
+
+@register_norm("toy_scale_norm")
+class ToyScaleNorm(Norm):
+    """y = x * w / sqrt(mean(x^2) + eps). On the HIP backend it runs a kernel of its own, compiled from a
+    source under tests/ and reached through `ops.call`; elsewhere torch."""
+
+    recordable = True
+
+    def __init__(self, width: int, eps: float):
+        self.width, self.eps = width, eps
+
+    def param_decls(self, prefix):
+        return [ParamDecl(prefix + ".weight", (self.width,), "vector", "around_one")]
+
+    def load(self, tensors, prefix, ops, dtype):
+        super().load(tensors, prefix, ops, dtype)
+        self.weight = tensors[prefix + ".weight"]
+        if getattr(ops, "name", "") == "hip":
+            register_toy_kernels()
+
+    def forward(self, x, want_f32, want_compute):
+        if getattr(self.ops, "name", "") != "hip":
+            y = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + self.eps) * self.weight
+            return (y if want_f32 else None), (y.to(self.dtype) if want_compute else None)
+        same = self.dtype == torch.float32
+        out_f32 = torch.empty_like(x) if (want_f32 or (want_compute and same)) else None
+        out_cd = torch.empty_like(x, dtype=self.dtype) if (want_compute and not same) else None
+        ops = self.ops
+        ops.call("toy_norm", "tnx_toy_scale_norm", ops.pointer(x), ops.pointer(self.weight), float(self.eps),
+                 ops.pointer(out_f32), ops.pointer(out_cd), 1, x.shape[0], x.shape[1], ops.stream())
+        return (out_f32 if want_f32 else None), ((out_f32 if same else out_cd) if want_compute else None)
+
+
+def toy_spec_rotating(width=96, heads=3, kv_heads=1, inner=72, vocab=157, positions=150, eps=1e-3, base=100.0):
+    """Two layers of attention whose queries and keys are turned by their positions (no encoding at the
+    input), grouped heads, a scale-only norm with its own kernel, names of its own for every tensor."""
+    hs = width // heads
+    norm = PartSpec("toy_scale_norm", dict(width=width, eps=eps))
+    mixer = PartSpec("attention", dict(width=width, num_heads=heads, head_size=hs, num_kv_heads=kv_heads, bias=False,
+                                       names=("wq", "wk", "wv", "wo"), rotation=PartSpec("toy_rotation", dict(base=base))))
+    ffn = PartSpec("dense", dict(width=width, inner=inner, activation="gelu", bias=False, up_name="up", down_name="down"))
+    layers = tuple(LayerSpec(prefix=f"blocks.{i}.", block="pre_norm", mixer=mixer, feed_forward=ffn, mixer_norm=norm,
+                             feed_forward_norm=norm, mixer_name="attn.", feed_forward_name="mlp.",
+                             mixer_norm_name="attn_norm", feed_forward_norm_name="mlp_norm") for i in range(2))
+    embedding = PartSpec("token_table", dict(vocab=vocab, embed_width=width, width=width, position=PartSpec("none", {}),
+                                             table_name="tokens.weight", projection_name=None, position_name=None))
+    head = PartSpec("vocab_projection", dict(vocab=vocab, embed_width=width, width=width, norm=norm,
+                                             weight_name="out.weight", tied_to=None, projection_name=None,
+                                             norm_name="out_norm"))
+    return ModelSpec(hidden_size=width, vocab_size=vocab, max_positions=positions, embedding=embedding, layers=layers,
+                     schedule=ModelSpec.sequential(2), head=head, init_std=0.1)
+
+
+def toy_rotating_plain_logits(w, tokens, width=96, heads=3, kv_heads=1, eps=1e-3, base=100.0, first_position=0):
+    """The rotating toy model on one whole sequence; `first_position` shifts every position (the logits must
+    not change: only distances count)."""
+    w = {k: v.float() for k, v in w.items()}
+    n, hs = len(tokens), width // heads
+    x = w["tokens.weight"][torch.tensor(tokens)]
+    pos = torch.arange(first_position, first_position + n, dtype=torch.float32)
+    freq = base ** (-torch.arange(hs // 2, dtype=torch.float32) * 2 / hs)
+    angle = pos[:, None] * freq[None, :]
+    cos, sin = torch.cos(angle)[:, None, :], torch.sin(angle)[:, None, :]
+
+    def norm(t, name):
+        return t * torch.rsqrt((t * t).mean(-1, keepdim=True) + eps) * w[name + ".weight"]
+
+    def turn(t, nh):
+        t = t.reshape(n, nh, hs // 2, 2)
+        return torch.stack([t[..., 0] * cos - t[..., 1] * sin, t[..., 0] * sin + t[..., 1] * cos], -1).reshape(n, nh * hs)
+
+    for i in range(2):
+        p = f"blocks.{i}."
+        h = norm(x, p + "attn_norm")
+        q = turn(plain_opt.linear(h, w[p + "attn.wq.weight"]), heads)
+        k = turn(plain_opt.linear(h, w[p + "attn.wk.weight"]), kv_heads)
+        v = plain_opt.linear(h, w[p + "attn.wv.weight"])
+        group = heads // kv_heads
+        k = k.reshape(n, kv_heads, hs).repeat_interleave(group, dim=1).reshape(n, width)
+        v = v.reshape(n, kv_heads, hs).repeat_interleave(group, dim=1).reshape(n, width)
+        x = x + plain_opt.linear(plain_opt.causal_attention(q, k, v, heads), w[p + "attn.wo.weight"])
+        h = norm(x, p + "mlp_norm")
+        x = x + plain_opt.linear(plain_opt.activation(plain_opt.linear(h, w[p + "mlp.up.weight"]), "gelu"),
+                                 w[p + "mlp.down.weight"])
+    return plain_opt.linear(norm(x, "out_norm"), w["out.weight"])

@@ -1,7 +1,7 @@
 """An inference engine for OPT-family decoders on one AMD MI355X."""
 __version__ = "0.1.0"
 
-from .config import (ContinuousBatchingConfig, EngineConfig, GenerationConfig, NeuronConfig, OPTConfig)  # noqa: F401
+from .config import ContinuousBatchingConfig, EngineConfig, GenerationConfig, NeuronConfig  # noqa: F401
 from .sampling import SamplingParams  # noqa: F401
 
 

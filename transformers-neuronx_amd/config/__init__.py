@@ -1,4 +1,5 @@
-from .model_config import ConfigError, ModelConfig, OPTConfig
+from .model_config import REQUIRED, ConfigError, ModelConfig
 from .engine_config import (ContinuousBatchingConfig, EngineConfig, GenerationConfig,
                             NeuronConfig, parse_dtype)
-from .registry import Architecture, known_architectures, read_config, register_architecture, resolve
+from .registry import (Architecture, add_architecture_package, known_architectures, read_config,
+                       register_architecture, resolve)

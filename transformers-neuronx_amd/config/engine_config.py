@@ -159,6 +159,9 @@ class EngineConfig:
                      what fits beside the cache
     run_ahead        a step is started before the host has read the tokens of the step before it (they
                      stay on the device for it); generation is the same, tokens are reported one call later
+    cast_float32_weights   bfloat16 engine: matrices stored in 32-bit are rounded to bfloat16 at load, as the
+                     reference's amp='bf16' does; left False such a matrix stays in 32-bit and its product
+                     runs on the float32 kernel (a line on stderr says so)
     seed             the random stream of a request whose `SamplingParams.seed` is None is keyed by this
                      plus the number of requests the engine took before it
     """
@@ -177,6 +180,7 @@ class EngineConfig:
     prompts_first: bool = False
     run_ahead: bool = True
     weight_copies: Optional[bool] = None
+    cast_float32_weights: bool = False
     seed: int = 0
 
     def __post_init__(self):

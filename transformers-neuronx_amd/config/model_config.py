@@ -2,20 +2,21 @@
 
 A configuration class lists the keys of its architecture's config.json, their
 types and defaults; `from_dict` checks them and names the key at fault. Nothing
-else in the package holds a model size.
+else in the package holds a model size. This module holds the base class only:
+an architecture's configuration lives in the architecture's own package.
 """
 import dataclasses
 import json
 import os
 from dataclasses import dataclass
-from typing import Any, ClassVar, Dict, Optional, Tuple
+from typing import Any, ClassVar, Dict
 
 
 class ConfigError(ValueError):
     """A config.json key is missing, of the wrong type, or out of range."""
 
 
-_REQUIRED = dataclasses.MISSING
+REQUIRED = dataclasses.MISSING      # the default of a key that config.json must give
 
 
 @dataclass(frozen=True)
@@ -30,7 +31,7 @@ class ModelConfig:
         for f in dataclasses.fields(cls):
             if f.name in raw and raw[f.name] is not None:
                 values[f.name] = cls._coerce(f, raw[f.name])
-            elif f.default is _REQUIRED and f.default_factory is _REQUIRED:
+            elif f.default is REQUIRED and f.default_factory is REQUIRED:
                 raise ConfigError(f"config.json of {cls.architecture}: required key '{f.name}' is missing")
         cfg = cls(**values)
         cfg.validate()
@@ -76,82 +77,3 @@ class ModelConfig:
         os.makedirs(folder, exist_ok=True)
         with open(os.path.join(folder, "config.json"), "w") as fp:
             json.dump(self.to_dict(), fp, indent=2)
-
-
-ACTIVATIONS: Tuple[str, ...] = ("relu", "gelu", "gelu_new")
-
-
-@dataclass(frozen=True)
-class OPTConfig(ModelConfig):
-    """The keys of an OPT config.json.
-
-    The reference copies ten of them (opt/config.py:22-40: activation_function,
-    eos/pad_token_id, ffn_dim, hidden_size, max_position_embeddings,
-    num_attention_heads, num_hidden_layers, vocab_size, word_embed_proj_dim) and
-    refuses `do_layer_norm_before=false` (:23-24); the full key set is that of
-    opt/gen_random_pretrained.py:105-140. Here every option of the family is
-    honoured: post-norm order, embedding width different from the hidden width,
-    no biases, norms without affine parameters.
-    `layer_norm_eps` is not a key of published OPT checkpoints; it defaults to the
-    value the reference fixes in code (hlo.py:51, 1e-5).
-    """
-
-    architecture: ClassVar[str] = "OPTForCausalLM"
-    model_type: ClassVar[str] = "opt"
-
-    vocab_size: int = _REQUIRED
-    hidden_size: int = _REQUIRED
-    num_hidden_layers: int = _REQUIRED
-    num_attention_heads: int = _REQUIRED
-    ffn_dim: int = _REQUIRED
-    max_position_embeddings: int = _REQUIRED
-    word_embed_proj_dim: Optional[int] = None
-    do_layer_norm_before: bool = True
-    activation_function: str = "relu"
-    enable_bias: bool = True
-    layer_norm_elementwise_affine: bool = True
-    layer_norm_eps: float = 1e-5
-    tie_word_embeddings: bool = True
-    bos_token_id: int = 2
-    eos_token_id: int = 2
-    pad_token_id: int = 1
-    init_std: float = 0.02
-    torch_dtype: str = "float16"
-
-    def __post_init__(self):
-        if self.word_embed_proj_dim is None:
-            object.__setattr__(self, "word_embed_proj_dim", self.hidden_size)
-
-    @staticmethod
-    def _coerce(f, value):
-        if f.name == "word_embed_proj_dim":
-            if isinstance(value, bool) or not isinstance(value, int):
-                raise ConfigError(f"key 'word_embed_proj_dim' must be an integer, got {value!r}")
-            return value
-        return ModelConfig._coerce(f, value)
-
-    @property
-    def head_size(self) -> int:
-        return self.hidden_size // self.num_attention_heads
-
-    def validate(self) -> None:
-        for key in ("vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads",
-                    "ffn_dim", "max_position_embeddings", "word_embed_proj_dim"):
-            if getattr(self, key) <= 0:
-                raise ConfigError(f"key '{key}' must be positive, got {getattr(self, key)}")
-        if self.hidden_size % self.num_attention_heads:
-            raise ConfigError(
-                f"key 'hidden_size' ({self.hidden_size}) must be a multiple of "
-                f"'num_attention_heads' ({self.num_attention_heads})")
-        if self.activation_function not in ACTIVATIONS:
-            raise ConfigError(
-                f"key 'activation_function' must be one of {ACTIVATIONS}, got {self.activation_function!r}")
-        if self.layer_norm_eps <= 0:
-            raise ConfigError(f"key 'layer_norm_eps' must be positive, got {self.layer_norm_eps}")
-        if self.torch_dtype not in ("float32", "float16", "bfloat16"):
-            raise ConfigError(f"key 'torch_dtype' must be float32, float16 or bfloat16, got {self.torch_dtype!r}")
-
-    def to_dict(self) -> Dict[str, Any]:
-        d = super().to_dict()
-        d["model_type"] = self.model_type
-        return d

@@ -4,10 +4,11 @@ The name is `config.json["architectures"][0]`; `model_type` is the fallback key,
 as in the reference's `modeling_auto.py:5-47`, which keys on `model_type` and
 asserts on an unknown one.
 """
+import importlib
 import json
 import os
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, Optional, Type
+from typing import Any, Callable, Dict, List, Type, Union
 
 from .model_config import ConfigError, ModelConfig
 
@@ -18,10 +19,31 @@ class Architecture:
     model_type: str                # e.g. "opt"
     config_class: Type[ModelConfig]
     build_spec: Callable           # config -> parts.spec.ModelSpec
-    model_class: Optional[type] = None   # user-facing class (set when its module is imported)
+    # the user-facing class, or where it is found ("package.module:Class", imported when first asked for);
+    # None: the architecture-free class serves
+    model_class: Union[type, str, None] = None
+
+    def user_class(self) -> type:
+        if isinstance(self.model_class, str):
+            module, _, name = self.model_class.partition(":")
+            self.model_class = getattr(importlib.import_module(module), name)
+        if self.model_class is None:
+            from ..causal_lm import CausalLMForSampling
+            return CausalLMForSampling
+        return self.model_class
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
+
+# Packages that register an architecture when they are imported. Another architecture is another package
+# that calls `register_architecture`, and its name here (or a call of `add_architecture_package`, or just
+# its import before a model folder is read).
+ARCHITECTURE_PACKAGES: List[str] = ["transformers_neuronx_amd.opt"]
+
+
+def add_architecture_package(module: str) -> None:
+    if module not in ARCHITECTURE_PACKAGES:
+        ARCHITECTURE_PACKAGES.append(module)
 
 
 def register_architecture(name: str, model_type: str, config_class, build_spec, model_class=None) -> Architecture:
@@ -36,8 +58,8 @@ def known_architectures():
 
 
 def _load_builtin():
-    # The built-in architectures register themselves on import.
-    from .. import opt  # noqa: F401
+    for module in ARCHITECTURE_PACKAGES:
+        importlib.import_module(module)
 
 
 def resolve(raw: Dict[str, Any]) -> Architecture:

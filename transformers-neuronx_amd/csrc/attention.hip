@@ -612,10 +612,13 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
       if (tid + 256 * j < v_chunks) {
         bf16x8 v = vreg[j];
         const int k0 = tile0 + 8 * vc_kc[j];
-        if (k0 + 8 > total) {                 // keys beyond the request: their values must not be NaN
+        // Keys beyond the request, and keys that no query of the block sees any more (their pages may have
+        // been given back: the lookup then leads to some other page): their probabilities are zero, and
+        // their values must not be NaN.
+        if (k0 + 8 > total || k0 < blk_lo) {
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if (k0 + e >= total) v[e] = 0;
+            if (k0 + e >= total || k0 + e < blk_lo) v[e] = 0;
         }
         *(bf16x8*)(vd + vc_d[j] * VSTR + vc_kc[j] * 8) = v;
       }
@@ -840,7 +843,10 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
                                      const int* cached_lens, const int* table, int table_width, int page_size,
                                      int num_pages, const int* tile_run, const int* tile_q0, int num_tiles, void* out,
                                      int num_heads, int num_kv, int head_size, int window, int direct,
-                                     hipStream_t stream) {
+                                     int query_tile, hipStream_t stream) {
+  TNX_REQUIRE(query_tile == PREFILL_Q_TILE,
+              "attention_prefill: the tiles hold %d queries each, the kernels take %d: a tile's later queries would "
+              "be skipped", query_tile, PREFILL_Q_TILE);
   TNX_REQUIRE(num_heads > 0 && num_kv > 0 && num_heads % num_kv == 0, "attention_prefill: bad head counts");
   TNX_REQUIRE(head_size % 16 == 0 && head_size >= 16 && head_size <= 256,
               "attention_prefill: head size %d is not a multiple of 16 in [16, 256]", head_size);

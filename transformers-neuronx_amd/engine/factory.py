@@ -63,7 +63,7 @@ def build_runner(model_config, source, cfg: EngineConfig) -> ModelRunner:
     bytes_per_page = CacheManager.bytes_per_page(needs, cfg.page_size, cfg.dtype)
     if hasattr(ops, "decode_copies"):
         ops.decode_copies = _room_for_weight_copies(cfg, model, bytes_per_page, device)
-    model.load(source, ops, cfg.dtype, device)
+    model.load(source, ops, cfg.dtype, device, cast_float32=cfg.cast_float32_weights)
     if hasattr(source, "release"):
         source.release()        # before the cache is sized and made: what the source held is free again,
         if device.type == "cuda":  # and goes back to the device, so that the cache's large blocks find room

@@ -79,8 +79,8 @@ class DecoderModel:
 
     # ---------------------------------------------------------------- weights
 
-    def load(self, source, ops, dtype: torch.dtype, device) -> "DecoderModel":
-        tensors = load_tensors(self.param_decls(), source, dtype, device)
+    def load(self, source, ops, dtype: torch.dtype, device, cast_float32: bool = False) -> "DecoderModel":
+        tensors = load_tensors(self.param_decls(), source, dtype, device, self.spec.base_model_prefix, cast_float32)
         self.embedding.load(tensors, "", ops, dtype)
         for layer in self.layers:
             layer.load(tensors, ops, dtype)

@@ -25,6 +25,21 @@ FLAGS = ["-O3", f"--offload-arch={ARCH}", "-shared", "-fPIC", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 _locks = {m: threading.Lock() for m in MODULES}
+_SOURCES: Dict[str, str] = {m: os.path.join(CSRC, f"{m}.hip") for m in MODULES}
+
+
+def register_module(name: str, source: str) -> None:
+    """A kernel module from outside the package: a part that needs a kernel of its own names its source
+    here (and its C signatures with `hip.register_signatures`), and reaches it through `HipOps.call`. The
+    library is built like the others, beside its source (folder `lib/`), and `common.h` is on its include path."""
+    if name in _SOURCES and os.path.abspath(_SOURCES[name]) != os.path.abspath(source):
+        raise BuildError(f"a kernel module named {name!r} is registered already, from {_SOURCES[name]}")
+    _SOURCES[name] = source
+    _locks.setdefault(name, threading.Lock())
+
+
+def modules() -> List[str]:
+    return list(_SOURCES)
 
 
 class BuildError(RuntimeError):
@@ -44,17 +59,20 @@ def find_hipcc() -> Optional[str]:
 
 def source_hash(module: str) -> str:
     h = hashlib.sha256()
-    for name in (f"{module}.hip", "common.h", f"tnx_{module}.h"):
-        if name.startswith("tnx_") and not os.path.exists(os.path.join(CSRC, name)):
-            continue                       # a header of its own entry points: not every module has one
-        with open(os.path.join(CSRC, name), "rb") as fp:
+    src = _SOURCES[module]
+    own_header = os.path.join(os.path.dirname(src), f"tnx_{module}.h")   # its entry points: not every module has one
+    for path in (src, os.path.join(CSRC, "common.h"), own_header):
+        if path == own_header and not os.path.exists(path):
+            continue
+        with open(path, "rb") as fp:
             h.update(fp.read())
     h.update(" ".join(FLAGS).encode())
     return h.hexdigest()[:16]
 
 
-def _lib_dirs() -> List[str]:
-    dirs = [os.path.join(CSRC, "lib")]
+def _lib_dirs(module: Optional[str] = None) -> List[str]:
+    src_dir = os.path.dirname(_SOURCES[module]) if module in _SOURCES else CSRC
+    dirs = [os.path.join(src_dir, "lib")]
     home = os.environ.get("XDG_CACHE_HOME") or (os.path.join(os.environ["HOME"], ".cache")
                                                 if os.environ.get("HOME") else None)
     if home:
@@ -69,15 +87,15 @@ def lib_name(module: str) -> str:
 
 def find_library(module: str) -> Optional[str]:
     name = lib_name(module)
-    for d in _lib_dirs():
+    for d in _lib_dirs(module):
         path = os.path.join(d, name)
         if os.path.exists(path):
             return path
     return None
 
 
-def _writable_dir() -> str:
-    for d in _lib_dirs():
+def _writable_dir(module: Optional[str] = None) -> str:
+    for d in _lib_dirs(module):
         try:
             os.makedirs(d, exist_ok=True)
             probe = os.path.join(d, f".probe-{os.getpid()}-{threading.get_ident()}")
@@ -87,12 +105,12 @@ def _writable_dir() -> str:
             return d
         except OSError:
             continue
-    raise BuildError("no folder to keep compiled kernels in: tried " + ", ".join(_lib_dirs()))
+    raise BuildError("no folder to keep compiled kernels in: tried " + ", ".join(_lib_dirs(module)))
 
 
 def compile_module(module: str, force: bool = False) -> str:
     """Compile `csrc/<module>.hip` for gfx950; returns the library's path."""
-    if module not in MODULES:
+    if module not in _SOURCES:
         raise BuildError(f"unknown kernel module {module!r}")
     with _locks[module]:
         if not force:
@@ -103,10 +121,10 @@ def compile_module(module: str, force: bool = False) -> str:
         if hipcc is None:
             raise BuildError(f"the HIP kernels of '{module}' are not built and hipcc was not found "
                              "(looked at $HIPCC, PATH and /opt/rocm/bin)")
-        out_dir = _writable_dir()
+        out_dir = _writable_dir(module)
         out = os.path.join(out_dir, lib_name(module))
         tmp = f"{out}.{os.getpid()}.tmp"
-        cmd = [hipcc] + FLAGS + [os.path.join(CSRC, f"{module}.hip"), "-o", tmp]
+        cmd = [hipcc] + FLAGS + ["-I", CSRC, _SOURCES[module], "-o", tmp]
         _log(f"compiling {module}.hip for {ARCH} ...")
         start = time.time()
         proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, cwd=out_dir)
@@ -147,7 +165,7 @@ def build_all(force: bool = True) -> Dict[str, str]:
         except BuildError as e:   # collected and raised together
             errors.append(str(e))
 
-    threads = [threading.Thread(target=work, args=(m,)) for m in MODULES]
+    threads = [threading.Thread(target=work, args=(m,)) for m in modules()]
     for t in threads:
         t.start()
     for t in threads:

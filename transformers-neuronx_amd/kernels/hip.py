@@ -50,7 +50,7 @@ _SIGNATURES = {
                               _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_attention_prefill": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                   _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
-                                  _c_int, _c_void_p],
+                                  _c_int, _c_int, _c_void_p],
         "tnx_attention_decode": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                  _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
                                  _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
@@ -67,6 +67,12 @@ _SIGNATURES = {
                        _c_int, _c_void_p],
     },
 }
+
+
+def register_signatures(module: str, signatures: Dict[str, list]) -> None:
+    """The C entry points (name -> ctypes argument types, all returning int) of a kernel module registered
+    with `build.register_module`."""
+    _SIGNATURES.setdefault(module, {}).update(signatures)
 
 
 class PreparedWeight:
@@ -161,6 +167,14 @@ class HipOps:
         rc = getattr(lib, fn)(*args)
         if rc != 0:
             raise RuntimeError(f"{fn}: {lib.tnx_last_error().decode()}")
+
+    def call(self, module: str, fn: str, *args) -> None:
+        """An entry point of any registered kernel module (also one a part brought itself); `stream()` and
+        `pointer()` give what such entry points take."""
+        self._call(module, fn, *args)
+
+    stream = staticmethod(_stream)
+    pointer = staticmethod(_ptr)
 
     # ---------------------------------------------------------------- input end
 
@@ -432,8 +446,14 @@ class HipOps:
         tiles = None
         if isinstance(w, PreparedWeight):
             w, tiles = w.tensor, w.tiles
-        if (self.dtype != torch.bfloat16 or w.dtype != torch.bfloat16
-                or self._library_product(ctx.num_tokens, w.shape[0], w.shape[1], w, force_tiled)):
+        if self.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and self._library_product(
+                ctx.num_tokens, w.shape[0], w.shape[1], w, force_tiled):
+            # many rows: the bias joins the library's float32 sums before they are rounded, once, as in the
+            # fused kernel below, so that keys and values are cached with the same rounding whichever path
+            # a token took; the queries are scaled after that
+            return self.qkv_write(self.linear(h, w, bias), None, num_heads, num_kv_write, head_size, scale, ctx,
+                                  view, k_pages, v_pages)
+        if self.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
             return self.qkv_write(self.linear(h, w, None), bias, num_heads, num_kv_write, head_size, scale, ctx,
                                   view, k_pages, v_pages)
         t = ctx.num_tokens
@@ -498,7 +518,8 @@ class HipOps:
                        _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(view.block_table), view.width,
                        view.page_size, num_pages, _ptr(ctx.tile_run), _ptr(ctx.tile_start), ctx.tile_run.numel(),
                        _ptr(out), num_heads, num_kv_heads, head_size, window,
-                       int(self.prefill_direct) or self._prefill_sets(ctx, num_heads, window), _stream())
+                       int(self.prefill_direct) or self._prefill_sets(ctx, num_heads, window), ctx.query_tile,
+                       _stream())
         n_dec = ctx.decode_runs.numel()
         if n_dec:
             splits, waves = self._decode_splits(ctx, n_dec * num_heads, window, head_size <= 128)

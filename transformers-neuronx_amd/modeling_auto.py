@@ -12,8 +12,4 @@ class NeuronAutoModelForCausalLM:
             arch, _ = read_config(pretrained_model_name_or_path)
         except ConfigError as e:
             raise AssertionError(f"{e} (not supported by this engine)") from None
-        from . import opt  # noqa: F401   importing an architecture's package sets its model class
-        from .opt import model  # noqa: F401
-        if arch.model_class is None:
-            raise AssertionError(f"the architecture {arch.name!r} has no model class")
-        return arch.model_class.from_pretrained(pretrained_model_name_or_path, *model_args, **kwargs)
+        return arch.user_class().from_pretrained(pretrained_model_name_or_path, *model_args, **kwargs)

@@ -11,7 +11,7 @@ import argparse
 import json
 import os
 
-from ..config.model_config import OPTConfig
+from .config import OPTConfig
 from ..weights.random_init import write_random_model
 
 

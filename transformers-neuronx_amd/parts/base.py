@@ -85,15 +85,18 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    """Where positions enter. `at_input(x, positions)` adds to the embedded
-    tokens (learned or fixed tables); `on_query_key` is the hook of encodings
-    that turn queries and keys inside a mixer. A part leaves the hook it does
-    not use as it is."""
+    """Where positions enter. `at_input(x, positions, want_compute)` adds to the embedded tokens (learned or
+    fixed tables) and returns `(float32, compute dtype or None)`. `on_query_key(qkv, ctx, num_heads,
+    num_kv_heads, head_size)` is the hook of encodings that turn queries and keys inside a mixer: the
+    attention mixer calls it, when its spec names such an encoding as `rotation`, with the step's
+    `[T, (num_heads + 2 num_kv_heads) * head_size]` projections (bias added, query not yet scaled) and
+    `ctx.positions`, and stores what it returns. A part leaves the hook it does not use as it is."""
 
     def at_input(self, x, positions, want_compute: bool):
         return None
 
-    rotates_query_key = False
+    def on_query_key(self, qkv, ctx, num_heads: int, num_kv_heads: int, head_size: int):
+        return qkv
 
 
 class Block(Part):

@@ -12,8 +12,8 @@ class DenseFeedForward(FeedForward):
 
     recordable = True
 
-    def __init__(self, width: int, inner: int, activation: str, bias: bool = True,
-                 up_name: str = "fc1", down_name: str = "fc2"):
+    def __init__(self, width: int, inner: int, activation: str, up_name: str, down_name: str, bias: bool = True):
+        """`up_name`, `down_name`: the checkpoint's names of the two matrices, relative to the part's prefix."""
         self.width, self.inner, self.activation, self.has_bias = width, inner, activation, bias
         self.up_name, self.down_name = up_name, down_name
 

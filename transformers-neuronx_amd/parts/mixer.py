@@ -4,7 +4,7 @@ from typing import Dict, List, Optional
 
 import torch
 
-from .base import CacheNeed, Mixer, register_mixer
+from .base import POSITIONS, CacheNeed, Mixer, register_mixer
 from .spec import ParamDecl
 
 
@@ -22,14 +22,18 @@ class Attention(Mixer):
 
     `num_kv_heads < num_heads` groups query heads over shared key/value heads.
     `own_kv=False` builds a mixer without key/value projections that reads the
-    cache another call of the run order writes.
+    cache another call of the run order writes. `rotation` names a position
+    encoding (a `PartSpec` of the position registry) whose `on_query_key` turns
+    the queries and keys before they are scaled and stored; OPT has none.
     """
 
     recordable = True
 
-    def __init__(self, width: int, num_heads: int, head_size: int, num_kv_heads: Optional[int] = None,
+    def __init__(self, width: int, num_heads: int, head_size: int, names, num_kv_heads: Optional[int] = None,
                  bias: bool = True, window: Optional[int] = None, scale: Optional[float] = None,
-                 own_kv: bool = True, names=("q_proj", "k_proj", "v_proj", "out_proj")):
+                 own_kv: bool = True, rotation=None):
+        """`names`: the checkpoint's names of the query, key, value and output projections, relative to
+        the mixer's prefix (the architecture's spec gives them)."""
         self.width, self.num_heads, self.head_size = width, num_heads, head_size
         self.num_kv_heads = num_kv_heads if num_kv_heads is not None else num_heads
         if self.num_heads % self.num_kv_heads:
@@ -39,6 +43,11 @@ class Attention(Mixer):
         self.has_bias, self.window, self.own_kv = bias, window, own_kv
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_size)
         self.names = tuple(names)
+        self.rotation = POSITIONS.build(rotation) if rotation is not None else None
+        if self.rotation is not None and not getattr(self.rotation, "recordable", False):
+            self.recordable = False
+        if len(self.names) != 4:
+            raise ValueError("names: the query, key, value and output projections, four names")
 
     def cache_need(self) -> Optional[CacheNeed]:
         return CacheNeed("paged", kv_heads=self.num_kv_heads, head_size=self.head_size, window=self.window)
@@ -56,6 +65,8 @@ class Attention(Mixer):
         d.append(ParamDecl(f"{prefix}{on}.weight", (self.width, q_out)))
         if self.has_bias:
             d.append(ParamDecl(f"{prefix}{on}.bias", (self.width,), "vector"))
+        if self.rotation is not None:
+            d += self.rotation.param_decls(prefix + "rotation")
         return d
 
     def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
@@ -69,11 +80,23 @@ class Attention(Mixer):
                       if self.has_bias else None)
         self.w_out = ops.prepare_weight(tensors[f"{prefix}{on}.weight"])
         self.b_out = tensors[f"{prefix}{on}.bias"] if self.has_bias else None
+        if self.rotation is not None:
+            self.rotation.load(tensors, prefix + "rotation", ops, dtype)
 
     def forward(self, h, ctx, cache, residual):
         if cache.writes != self.own_kv:
             raise ValueError("an attention mixer with own_kv writes its cache; one without reads another's")
         view = ctx.groups[cache.group]
+        kv_write = self.num_kv_heads if self.own_kv else 0
+        if self.rotation is not None:
+            # the projections with their bias, turned by the encoding, then scaled and stored
+            qkv = self.ops.linear(h, self.w_qkv, self.b_qkv)
+            qkv = self.rotation.on_query_key(qkv, ctx, self.num_heads, kv_write, self.head_size)
+            q = self.ops.qkv_write(qkv, None, self.num_heads, kv_write, self.head_size, self.scale, ctx, view,
+                                   cache.k_pages, cache.v_pages)
+            c = self.ops.attention(q, self.num_heads, self.num_kv_heads, self.head_size, ctx, view,
+                                   cache.k_pages, cache.v_pages, self.window)
+            return self.ops.linear(c, self.w_out, self.b_out, residual=residual, out_f32=True)
         q = self.ops.qkv_project(h, self.w_qkv, self.b_qkv, self.num_heads,
                                  self.num_kv_heads if self.own_kv else 0, self.head_size, self.scale, ctx, view,
                                  cache.k_pages, cache.v_pages)

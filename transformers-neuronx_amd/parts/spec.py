@@ -82,6 +82,9 @@ class ModelSpec:
     schedule: Tuple[LayerCall, ...]
     head: PartSpec                  # final norm, optional projection, vocabulary projection
     init_std: float = 0.02
+    # A checkpoint of the base model alone names its tensors without this leading piece; the loader
+    # tries a declared name without it when the name itself is absent ("" : no such form).
+    base_model_prefix: str = ""
 
     @staticmethod
     def sequential(n_layers: int) -> Tuple[LayerCall, ...]:

@@ -30,9 +30,10 @@ _ST_DTYPES = {
 class WeightsError(ValueError):
     """The checkpoint does not hold what the model declares."""
 
-    def __init__(self, missing, unexpected, wrong_shape, wrong_dtype=()):
+    def __init__(self, missing, unexpected, wrong_shape, wrong_dtype=(), tied_differ=()):
         self.missing, self.unexpected = list(missing), list(unexpected)
         self.wrong_shape, self.wrong_dtype = list(wrong_shape), list(wrong_dtype)
+        self.tied_differ = list(tied_differ)
         lines = ["checkpoint does not match the model:"]
         if self.missing:
             lines.append(f"  missing tensors ({len(self.missing)}): " + ", ".join(self.missing))
@@ -42,6 +43,9 @@ class WeightsError(ValueError):
             lines.append(f"  wrong shape: {name} is {list(got)}, expected {list(want)}")
         for name, got in self.wrong_dtype:
             lines.append(f"  wrong dtype: {name} is {got}, expected a floating type")
+        for name, other in self.tied_differ:
+            lines.append(f"  tied tensors differ: {name} is in the checkpoint and is not equal to {other}, "
+                         f"which the configuration ties it to")
         super().__init__("\n".join(lines))
 
 
@@ -114,36 +118,38 @@ class TensorDict:
         self._t.clear()
 
 
-def _base_model_name(name: str) -> Optional[str]:
-    return name[len("model."):] if name.startswith("model.") else None
+def _base_model_name(name: str, base_prefix: str) -> Optional[str]:
+    """A checkpoint of the base model alone (without the head's wrapper) names its tensors without the
+    wrapper's prefix; the architecture's spec says what that prefix is."""
+    return name[len(base_prefix):] if base_prefix and name.startswith(base_prefix) else None
 
 
-def resolve_names(decls: Iterable[ParamDecl], source) -> Dict[str, Optional[str]]:
+def _find(name: str, source, base_prefix: str) -> Optional[str]:
+    for cand in (name, _base_model_name(name, base_prefix)):
+        if cand is not None and cand in source:
+            return cand
+    return None
+
+
+def resolve_names(decls: Iterable[ParamDecl], source, base_prefix: str = "") -> Dict[str, Optional[str]]:
     """Declared name -> name in the source (itself, its base-model form, or the
     tensor it is tied to); None when absent."""
     out = {}
     for d in decls:
-        found = None
-        for cand in (d.name, _base_model_name(d.name)):
-            if cand is not None and cand in source:
-                found = cand
-                break
+        found = _find(d.name, source, base_prefix)
         if d.tied_to is not None:
-            # A tied tensor is the tensor it is tied to; a copy in the file is not read.
-            for cand in (d.tied_to, _base_model_name(d.tied_to)):
-                if cand is not None and cand in source:
-                    found = cand
-                    break
+            # A tied tensor is the tensor it is tied to; a copy in the file is compared with it, not used.
+            found = _find(d.tied_to, source, base_prefix) or found
         out[d.name] = found
     return out
 
 
-def check(decls: List[ParamDecl], source) -> Dict[str, Optional[str]]:
+def check(decls: List[ParamDecl], source, base_prefix: str = "") -> Dict[str, Optional[str]]:
     """Raise one `WeightsError` for everything that is wrong; return the name map."""
-    names = resolve_names(decls, source)
+    names = resolve_names(decls, source, base_prefix)
     missing = [n for n, src in names.items() if src is None]
     used = {src for src in names.values() if src is not None}
-    declared = {d.name for d in decls} | {b for d in decls if (b := _base_model_name(d.name))}
+    declared = {d.name for d in decls} | {b for d in decls if (b := _base_model_name(d.name, base_prefix))}
     unexpected = [n for n in source.names() if n not in used and n not in declared]
     wrong_shape, wrong_dtype = [], []
     for d in decls:
@@ -164,34 +170,64 @@ def check(decls: List[ParamDecl], source) -> Dict[str, Optional[str]]:
     return names
 
 
-def target_dtype(role: str, stored: torch.dtype, compute: torch.dtype) -> torch.dtype:
+def target_dtype(role: str, stored: torch.dtype, compute: torch.dtype, cast_float32: bool = False) -> torch.dtype:
     """The dtype a tensor is kept in on the device.
 
     float32 engine: every floating tensor in float32. bfloat16 engine: 16-bit
-    tensors in bfloat16, a tensor stored in 32-bit stays in 32-bit; biases and
-    norm parameters are widened to float32 (value-preserving), which is what the
-    kernels read; integer tables in int32."""
+    tensors in bfloat16, a tensor stored in 32-bit stays in 32-bit unless
+    `cast_float32` asks for its rounding (the reference's `amp='bf16'` rounds
+    every weight, module.py:395-432); biases and norm parameters are widened to
+    float32 (value-preserving), which is what the kernels read; integer tables in
+    int32."""
     if role == "index":
         return torch.int32
     if compute == torch.float32 or role == "vector":
         return torch.float32
-    if stored in (torch.float32, torch.float64):
+    if stored in (torch.float32, torch.float64) and not cast_float32:
         return torch.float32
     return torch.bfloat16
 
 
-def load_tensors(decls: List[ParamDecl], source, compute: torch.dtype, device) -> Dict[str, torch.Tensor]:
+def load_tensors(decls: List[ParamDecl], source, compute: torch.dtype, device, base_prefix: str = "",
+                 cast_float32: bool = False) -> Dict[str, torch.Tensor]:
     """Check, then read every declared tensor to `device` in its target dtype.
     Tensors that resolve to the same source tensor share one device buffer."""
-    names = check(decls, source)
+    names = check(decls, source, base_prefix)
     by_source: Dict[tuple, torch.Tensor] = {}
     out = {}
+    kept_wide, halves = [], []
+    tied_differ = []
     for d in decls:
         src = names[d.name]
-        dt = target_dtype(d.role, source.dtype(src), compute)
+        stored = source.dtype(src)
+        dt = target_dtype(d.role, stored, compute, cast_float32)
+        if dt == torch.float32 and compute != torch.float32 and d.role in ("matrix", "table"):
+            kept_wide.append(d.name)
+        if stored == torch.float16 and dt == torch.bfloat16:
+            halves.append(d.name)
         key = (src, dt)
         if key not in by_source:
             t = source.tensor(src)
             by_source[key] = t.to(device=device, dtype=dt).contiguous()
         out[d.name] = by_source[key]
+        if d.tied_to is not None:
+            own = _find(d.name, source, base_prefix)
+            if own is not None and own != src:
+                # the checkpoint holds a copy of its own of the tied tensor (the reference takes the
+                # tie for granted, module.py:142-159): it must say the same, or the file is another model's
+                a, b = source.tensor(own), source.tensor(src)
+                if a.shape != b.shape or not torch.equal(a, b.to(a.dtype)):
+                    tied_differ.append((own, src))
+    if tied_differ:
+        raise WeightsError([], [], [], [], tied_differ)
+    import sys
+    if halves:
+        print(f"[transformers_neuronx_amd] {len(halves)} tensors are stored in float16 and are rounded to bfloat16, "
+              f"the one 16-bit format of the kernels (3 bits of the fraction are lost; first: {halves[0]}); "
+              f"dtype float32 keeps every bit", file=sys.stderr, flush=True)
+    if kept_wide:
+        print(f"[transformers_neuronx_amd] {len(kept_wide)} matrices are stored in 32-bit and stay so in this "
+              f"{str(compute).replace('torch.', '')} engine (first: {kept_wide[0]}): their products run on the "
+              f"float32 kernel, slower and at twice the memory; cast_float32_weights=True rounds them at load",
+              file=sys.stderr, flush=True)
     return out
