@@ -7,7 +7,9 @@ One JSON line: `value` is decoded tokens per second at batch 8 and a 2,048-token
 (a "step" is one decode step of the whole engine: schedule, model, sampling);
 `prefill` is one 2,048-token prompt in one step; `roofline` sets the bytes a decode step has
 to read (every weight once, and the cache of the live requests) against its time; `points`
-holds decoding at batch 1 and 64. The measuring follows the reference's own benchmark
+holds decoding at batch 1 and 64 (tokens a second, milliseconds a step, share of the memory roofline) and the
+whole way of batch 8 from 512-token prompts to the 2,048-token context (mean tokens a second, its share of the
+roofline at the mean context, and the percentiles of the time between two steps). The measuring follows the reference's own benchmark
 (generation_demo.py:107-187: warm-up runs, then timed ones; random token ids as prompts,
 :492-494). Weights and prompts are synthetic and seeded; there are no published numbers of
 the reference to compare with, so `vs_baseline` is null.
@@ -21,12 +23,12 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-# OPT-6.7B: the sizes of BASELINE.json's configs[2]
+# OPT-6.7B: the measurement of record
 MODEL = dict(architectures=["OPTForCausalLM"], model_type="opt", vocab_size=50272, hidden_size=4096,
              num_hidden_layers=32, num_attention_heads=32, ffn_dim=16384, max_position_embeddings=2048,
              word_embed_proj_dim=4096, do_layer_norm_before=True, activation_function="relu", enable_bias=True,
              layer_norm_elementwise_affine=True, init_std=0.02, torch_dtype="bfloat16")
-# The other sizes BASELINE.json names, for `--model` (the default run and its JSON line stay OPT-6.7B)
+# Two more members of the family, for `--model` (the default run and its JSON line stay OPT-6.7B)
 OTHER_MODELS = {
     "350m": dict(hidden_size=1024, num_hidden_layers=24, num_attention_heads=16, ffn_dim=4096, word_embed_proj_dim=512,
                  do_layer_norm_before=False),
@@ -59,12 +61,12 @@ def main():
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--prefill-only", action="store_true", help="measure the prompt step alone (for profiles)")
     ap.add_argument("--model", default="6.7b", choices=["6.7b"] + sorted(OTHER_MODELS),
-                    help="layer sizes: OPT-6.7B (the measurement of record) or another size BASELINE.json names")
+                    help="layer sizes: OPT-6.7B (the measurement of record), OPT-350m or OPT-66B")
     ap.add_argument("--do-sample", action="store_true",
                     help="decode with temperature 0.8, top-k 50 and top-p 0.95 instead of greedily")
     ap.add_argument("--mix", action="store_true",
                     help="instead: 64 requests with prompts of 16 to 1,024 tokens and 256 new tokens each, all "
-                         "queued at once (BASELINE.json's continuous-batching workload); prints its own line")
+                         "queued at once (a continuous-batching workload); prints its own line")
     ap.add_argument("--big-batch", type=int, default=64, help="the larger batch of `points` (cut to what fits the device at the full context)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -114,11 +116,12 @@ def main():
     engine = LLMEngine(runner, ecfg)
     gen = torch.Generator().manual_seed(1)
 
-    def decode(batch, steps, warmup):
+    def decode(batch, steps, warmup, prompt_len=None, latencies=None):
         """Tokens per second, seconds per step and bytes per step of `steps` decode steps that end at
-        the full context."""
+        the full context (or begin after prompts of `prompt_len` tokens)."""
         engine.reset()
-        prompt_len = CONTEXT - (steps + warmup) - 1
+        if prompt_len is None:
+            prompt_len = CONTEXT - (steps + warmup) - 1
         for i in range(batch):
             params = SamplingParams(max_new_tokens=steps + warmup + 1, do_sample=args.do_sample, temperature=0.8,
                                     top_k=50, top_p=0.95, seed=i, ignore_eos=True)
@@ -131,9 +134,14 @@ def main():
         torch.cuda.synchronize()
         start = time.perf_counter()
         lens = made = 0
+        last = start
         for _ in range(steps):
             lens += sum(r.num_computed for r in engine.requests.values())
             made += len(engine.step())
+            if latencies is not None:        # host time between two steps: the device sets the pace
+                now = time.perf_counter()
+                latencies.append(now - last)
+                last = now
         torch.cuda.synchronize()
         sec = (time.perf_counter() - start) / steps
         assert made == batch * steps, f"{made} tokens in {steps} steps of batch {batch}"
@@ -210,9 +218,25 @@ def main():
         points = {}
         for b, k, w in ((1, min(args.steps, 64), args.warmup),
                         (args.big_batch, min(args.steps, 32), min(args.warmup, 4))):
-            v, s, _ = decode(b, k, w)
+            v, s, rd = decode(b, k, w)
             points[f"decode_b{b}"] = round(v, 2)
+            points[f"decode_b{b}_ms"] = round(s * 1e3, 4)
+            points[f"decode_b{b}_hbm_frac"] = round(rd / s / 1e9 / PEAK_HBM_GBS, 4)
             print(f"[bench] decode batch {b}: {v:.1f} tok/s, {s * 1e3:.2f} ms/step", file=sys.stderr, flush=True)
+        # the whole way from 512-token prompts to the full context, as the reference's benchmark generates whole
+        # sequences (generation_demo.py:159-187) and reports the percentiles of their latency
+        lat = []
+        first = 512
+        k = CONTEXT - first - 1 - 4
+        v, s, rd = decode(args.batch, k, 4, prompt_len=first, latencies=lat)
+        lat.sort()
+        points["decode_512_to_2048"] = round(v, 2)
+        points["decode_512_to_2048_ms"] = round(s * 1e3, 4)
+        points["decode_512_to_2048_hbm_frac"] = round(rd / s / 1e9 / PEAK_HBM_GBS, 4)
+        for q in (0, 50, 90, 95, 99, 100):
+            points[f"step_latency_p{q}_ms"] = round(lat[min(len(lat) - 1, int(len(lat) * q / 100))] * 1e3, 4)
+        print(f"[bench] decode batch {args.batch}, 512 -> 2,048: {v:.1f} tok/s, {s * 1e3:.2f} ms/step",
+              file=sys.stderr, flush=True)
         out["points"] = points
     print(json.dumps(out))
     return 0

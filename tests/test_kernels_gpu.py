@@ -421,11 +421,12 @@ def test_bfloat16_attention_kernels_agree(case, window):
         forced.prefill_direct = sets
         o_forced = forced.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)
         torch.testing.assert_close(o_forced.float(), o_plain.float(), rtol=2e-2, atol=2e-2)
-    narrow = HipOps(torch.bfloat16, DEV)
-    narrow.decode_wide_blocks = 0                 # blocks of four waves only, twice the splits
-    narrow.decode_blocks_wanted = 1 << 20
-    o_narrow = narrow.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)
-    torch.testing.assert_close(o_narrow.float(), o_plain.float(), rtol=2e-2, atol=2e-2)
+    wide = HipOps(torch.bfloat16, DEV)
+    wide.decode_waves = 8                         # blocks of eight waves
+    for wanted in (1 << 20, 1):
+        wide.decode_blocks_wanted = wanted
+        o_wide = wide.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)
+        torch.testing.assert_close(o_wide.float(), o_plain.float(), rtol=2e-2, atol=2e-2)
     one = HipOps(torch.bfloat16, DEV)
     one.decode_blocks_wanted = 1                  # no split at all
     o_one = one.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)

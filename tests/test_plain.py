@@ -190,3 +190,92 @@ def test_greedy_is_argmax_of_the_last_position():
     assert out[:3] == [5, 9, 11] and len(out) == 7
     assert out[3] == int(plain_opt.forward_logits(w, TINY_A, [5, 9, 11])[-1].argmax())
     assert out[4] == int(plain_opt.forward_logits(w, TINY_A, out[:4])[-1].argmax())
+
+
+def _constant_norm(w, name, width, value):
+    """A norm whose output is the same vector for every token: weight 0, bias `value`."""
+    w[name + ".weight"] = torch.zeros(width)
+    w[name + ".bias"] = value.clone()
+
+
+def test_which_norm_feeds_which_half():
+    """Pins the composition of a block from outside its own text. A norm with weight 0 and bias c hands the
+    same vector c to whatever it feeds. Pre-norm: with `self_attn_layer_norm` made so, every token's query,
+    key and value are those of c, attention averages equal values, and the first half adds one and the same
+    vector out_proj(v_proj(c)) to every token, which library routines give; with `final_layer_norm` made so
+    the second half adds fc2(act(fc1(c))). If the norms were exchanged, or a half read the stream instead of
+    its norm, neither would hold."""
+    cfg = dict(TINY_A)
+    p = "model.decoder.layers.0."
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(9, 64, generator=g)
+    c = torch.randn(64, generator=g)
+    lin = torch.nn.functional.linear
+    # the first half
+    w = plain_opt.random_weights(cfg, 3)
+    _constant_norm(w, p + "self_attn_layer_norm", 64, c)
+    for k in ("fc1.weight", "fc2.weight", "fc1.bias", "fc2.bias"):
+        w[p + k] = torch.zeros_like(w[p + k])                     # the second half adds nothing
+    added = lin(lin(c, w[p + "self_attn.v_proj.weight"], w[p + "self_attn.v_proj.bias"]),
+                w[p + "self_attn.out_proj.weight"], w[p + "self_attn.out_proj.bias"])
+    torch.testing.assert_close(plain_opt.block(x, w, cfg, 0), x + added, rtol=1e-5, atol=1e-5)
+    # the second half
+    w = plain_opt.random_weights(cfg, 3)
+    _constant_norm(w, p + "final_layer_norm", 64, c)
+    for k in ("q_proj", "k_proj", "v_proj", "out_proj"):
+        w[p + f"self_attn.{k}.weight"] = torch.zeros_like(w[p + f"self_attn.{k}.weight"])
+        w[p + f"self_attn.{k}.bias"] = torch.zeros_like(w[p + f"self_attn.{k}.bias"])
+    added = lin(torch.relu(lin(c, w[p + "fc1.weight"], w[p + "fc1.bias"])), w[p + "fc2.weight"], w[p + "fc2.bias"])
+    torch.testing.assert_close(plain_opt.block(x, w, cfg, 0), x + added, rtol=1e-5, atol=1e-5)
+
+
+def test_post_norm_order_and_no_norm_before_the_head():
+    """Post-norm: the stream after the first half is that half's norm, so with that norm constant the second
+    half sees c alone and the block's output is norm2(c + ffn(c)) for every token; and with the last block's
+    second norm constant the logits are the head of c, nothing in between (no further norm: a post-norm
+    model has none before its head)."""
+    cfg = dict(TINY_B)
+    width = cfg["hidden_size"]
+    affine = dict(cfg, layer_norm_elementwise_affine=True)        # so that the norms have parameters to set
+    w = plain_opt.random_weights(affine, 4)
+    p = "model.decoder.layers.0."
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(7, width, generator=g)
+    c = torch.randn(width, generator=g)
+    lin = torch.nn.functional.linear
+    _constant_norm(w, p + "self_attn_layer_norm", width, c)
+    inner = torch.nn.functional.gelu(lin(c, w[p + "fc1.weight"]))
+    want = torch.nn.functional.layer_norm(c + lin(inner, w[p + "fc2.weight"]), (width,),
+                                          w[p + "final_layer_norm.weight"], w[p + "final_layer_norm.bias"],
+                                          cfg["layer_norm_eps"])
+    got = plain_opt.block(x, w, affine, 0)
+    torch.testing.assert_close(got, want.expand_as(got), rtol=1e-5, atol=1e-5)
+    # the head
+    last = f"model.decoder.layers.{cfg['num_hidden_layers'] - 1}."
+    w = plain_opt.random_weights(affine, 4)
+    _constant_norm(w, last + "final_layer_norm", width, c)
+    logits = plain_opt.forward_logits(w, affine, [5, 9, 300, 4])
+    want = lin(lin(c, w["model.decoder.project_out.weight"]), w["model.decoder.embed_tokens.weight"])
+    torch.testing.assert_close(logits, want.expand_as(logits), rtol=1e-5, atol=1e-5)
+
+
+def test_pre_norm_head_norms_the_stream_once():
+    """Pre-norm: the logits are head(final_layer_norm(stream)); with that norm constant they are the head of
+    c, and with all blocks adding nothing and the norm real they are the head of the normed embedding."""
+    cfg = dict(TINY_A)
+    w = plain_opt.random_weights(cfg, 5)
+    g = torch.Generator().manual_seed(9)
+    c = torch.randn(64, generator=g)
+    lin = torch.nn.functional.linear
+    w1 = dict(w)
+    _constant_norm(w1, "model.decoder.final_layer_norm", 64, c)
+    logits = plain_opt.forward_logits(w1, cfg, [5, 9, 300])
+    torch.testing.assert_close(logits, lin(c, w["model.decoder.embed_tokens.weight"]).expand_as(logits),
+                               rtol=1e-5, atol=1e-5)
+    wz = {k: (torch.zeros_like(v) if (".layers." in k and ("proj" in k or "fc" in k)) else v) for k, v in w.items()}
+    toks = torch.tensor([5, 9, 300])
+    x = w["model.decoder.embed_tokens.weight"][toks] + w["model.decoder.embed_positions.weight"][2:5]
+    want = lin(torch.nn.functional.layer_norm(x, (64,), w["model.decoder.final_layer_norm.weight"],
+                                              w["model.decoder.final_layer_norm.bias"], 1e-5),
+               w["model.decoder.embed_tokens.weight"])
+    torch.testing.assert_close(plain_opt.forward_logits(wz, cfg, toks.tolist()), want, rtol=1e-5, atol=1e-5)

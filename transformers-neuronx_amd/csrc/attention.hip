@@ -904,132 +904,209 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
 
 // ------------------------------------------------------------------------------------------ bfloat16, decoding
 
-// One query per request over its pages. The keys of a request are split over `num_splits` blocks; a block's
-// NW waves (four or eight) take 64-key tiles in turn. A tile of keys of one head is read as it lies in memory, 16 bytes
-// a lane: lane l holds chunk l % CPR (8 head-size elements) of key l / CPR of each group of 64 / CPR keys.
-// The partial dot products are summed over the CPR lanes of a key by a butterfly that halves what each lane
-// keeps at every step, so that in the end every lane holds the score of one key of the tile. Values lie
-// transposed ([head_size][page_size]), so lane l holds 8 keys (l % 8) of head-size element l / 8 of each
-// group of 8 elements, and the output is a sum over 8 neighbouring lanes, taken once at the end.
-// No load depends on a branch: keys beyond the request read a valid place and get weight zero.
-// Partial results (maximum, sum, weighted values, all float32) of waves meet in LDS and those of splits in
-// a workspace that a second kernel merges. The page size is a power of two here.
-template <int CPR, int NW>
-__global__ void __launch_bounds__(64 * NW, (CPR <= 8 ? 16 / NW : (CPR == 16 ? 8 / NW : 1)))
-attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
-                        const bf16_t* __restrict__ v_pages, const int* __restrict__ run_start,
-                        const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
-                        int page_shift, int num_pages, const int* __restrict__ decode_runs, bf16_t* __restrict__ out,
-                        float* __restrict__ part_o, float* __restrict__ part_ml, int num_heads, int num_kv,
-                        int window, int num_splits, const int* __restrict__ longest_ptr, int head_size) {
-  constexpr int KPI = 64 / CPR;       // keys per load instruction of a wave
-  constexpr int DH = CPR * 8;         // the lanes' layout is made for this head size; `head_size` <= DH
-  const int cpr = head_size / 8;      // chunks a key really has: lanes of higher chunks repeat the last one
-  __shared__ float sm_p[NW][64];
+// One query per request over its pages, on the matrix unit. The keys of a request are split over `num_splits`
+// blocks; a block's NW waves (four or eight) take 64-key tiles in turn. Partial results (maximum, sum, weighted
+// values, all float32) of waves meet in LDS and those of splits in a workspace that a second kernel merges. The
+// page size is a power of two here.
+// The one query of a (request, head) is the B operand of S^T = K q in all 16 of
+// its columns (the products cost nothing more, and with them the scores come out in the accumulator layout
+// that is at once the B operand of O^T += V^T P^T, as in the prompt kernel); row r of key block kb of a 64-key
+// tile is key 32 (kb / 2) + 8 (r / 4) + 4 (kb % 2) + r % 4, so that the probabilities a lane holds are those of
+// 8 consecutive keys and the values are read 16 bytes a lane as they lie. A tile costs 32 matrix
+// instructions and some 150 others, where dot products on the vector unit took a thousand: the step of a few
+// requests is the time its instructions take to arrive from memory, and the step of many requests was close
+// to the vector unit's limit (measured at head size 128, context 2,048: 18.1 -> 15.6 us for one request,
+// 52.4 -> 49.7 for 8, 381 -> 369 for 64).
+// The pages of a tile are looked up with scalar loads (a tile's keys lie in at most four pages, the same for
+// every lane), which do not queue behind the tile data; the next tile's keys are asked for as soon as this
+// tile's scores are made, its values as soon as this tile's are used (NDB <= 8; beyond that the registers
+// hold one of the two at a time).
+template <int NDB, int NW>
+__global__ void __launch_bounds__(64 * NW, (NDB <= 8 ? 8 / NW : 1))
+attention_decode_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
+                             const bf16_t* __restrict__ v_pages, const int* __restrict__ run_start,
+                             const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
+                             int page_shift, int num_pages, const int* __restrict__ decode_runs,
+                             bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
+                             int num_heads, int num_kv, int window, int num_splits,
+                             const int* __restrict__ longest_ptr, int head_size) {
+  constexpr int NKS = (NDB + 1) / 2;  // steps of 32 over the head size
+  constexpr int DH = 16 * NDB;        // the registers are laid out for this head size; `head_size` <= DH
+  constexpr bool PIPE = NDB <= 8;     // keys and values of different tiles are in registers together
   __shared__ float sm_o[NW][DH];
   __shared__ float sm_m[NW], sm_l[NW];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane & 15, g = lane >> 4;
   const int split = blockIdx.x, h = blockIdx.y, dz = blockIdx.z;
   const int kvh = h / (num_heads / num_kv);
   const int run = decode_runs[dz];
+  const int longest_given = longest_ptr[0];
   const int t = run_start[run];
   const int pos = cached_lens[run];   // the query's own position; its key is stored already
   const int* tab = table + (size_t)run * table_width;
   const int nq = num_heads * head_size;
   const int page_size = 1 << page_shift, pmask = page_size - 1;
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  // The longest range of keys any decoding request of the step reads is given in device memory, so that a
-  // recorded launch stays valid while the requests grow; every split takes an equal share of it, in 64s.
-  const int longest = window > 0 ? min(longest_ptr[0], window + 64) : longest_ptr[0];
+  const int last_key = table_width * page_size - 1;      // the last key the table has a place for
+  const int longest = window > 0 ? min(longest_given, window + 64) : longest_given;
   const int keys_per_split = (((longest + num_splits - 1) / num_splits) + 63) & ~63;
+  const size_t head_stride = (size_t)page_size * head_size;   // elements of one head of one page
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  // the pages of a tile's four blocks of 16 keys (a block of 16 lies in one page; pages of 64 keys and more
+  // hold a whole tile): the same for every lane
+  auto lookup = [&](int (&pg)[4], int tile0) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int key = __builtin_amdgcn_readfirstlane(min(tile0 + 16 * c, last_key));
+      pg[c] = min(max(tab[key >> page_shift], 0), num_pages - 1);
+    }
+  };
+  bf16x8 kf[4][NKS], vf[NDB][2];
+  // a lane's chunk of 8 elements at head-size offset 32 ks + 8 g; where the head ends inside a step the lanes
+  // beyond it read the last chunk again and drop it
+  const int dlast = head_size - 8;
+  auto load_keys = [&](const int (&pg)[4], int tile0) {
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      const int off = 32 * (kb >> 1) + 8 * (r >> 2) + 4 * (kb & 1) + (r & 3);
+      const int page = (r >> 3) ? pg[2 * (kb >> 1) + 1] : pg[2 * (kb >> 1)];
+      const bf16_t* kp = k_pages + ((size_t)page * num_kv + kvh) * head_stride +
+                         (size_t)((tile0 + off) & pmask) * head_size;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) kf[kb][ks] = *(const bf16x8*)(kp + min(32 * ks + 8 * g, dlast));
+    }
+  };
+  auto load_values = [&](const int (&pg)[4], int tile0) {
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const int page = (g >> 1) ? pg[2 * st + 1] : pg[2 * st];
+      const bf16_t* vp = v_pages + ((size_t)page * num_kv + kvh) * head_stride + ((tile0 + 32 * st + 8 * g) & pmask);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+        vf[db][st] = *(const bf16x8*)(vp + (size_t)min(16 * db + r, head_size - 1) * page_size);
+    }
+  };
+
+  int pg[4], pgn[4];
+  int tile0 = 0;
+  bool fetched = false;
+  if (window <= 0) {
+    // the first tile of this wave's share, asked for before the request's length is known: from places that
+    // are valid whatever it turns out to be, and masked afterwards
+    tile0 = split * keys_per_split + 64 * wave;
+    if (64 * wave < keys_per_split) {
+      lookup(pg, tile0);
+      load_keys(pg, tile0);
+      if (PIPE) load_values(pg, tile0);
+      fetched = true;
+    }
+  }
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int k_begin = (lo / 64) * 64 + split * keys_per_split;
   const int k_end = min(pos + 1, k_begin + keys_per_split);
-  const int dchunk = lane % CPR, kgrp = lane / CPR;
-  const size_t head_stride = (size_t)page_size * head_size;   // elements of one head of one page
-  const int kchunk = min(dchunk, cpr - 1);
+  tile0 = k_begin + 64 * wave;
 
-  float qf[8];
-  {
-    const bf16x8 qv = *(const bf16x8*)(q + (size_t)t * nq + h * head_size + kchunk * 8);
+  bf16x8 qf[NKS];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) qf[j] = dchunk < cpr ? (float)qv[j] : 0.f;
+  for (int ks = 0; ks < NKS; ++ks) {
+    const bf16x8 qv = *(const bf16x8*)(q + (size_t)t * nq + h * head_size + min(32 * ks + 8 * g, dlast));
+    qf[ks] = (32 * ks + 8 * g < head_size) ? qv : zero8;
   }
-  float m = -INFINITY, l = 0.f;
-  float acc[CPR];
+  float m = -INFINITY, l = 0.f;       // `l`: this lane's share of the sum (its own 16 keys a tile)
+  f32x4 o[NDB];
 #pragma unroll
-  for (int i = 0; i < CPR; ++i) acc[i] = 0.f;
+  for (int db = 0; db < NDB; ++db) o[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  for (int tile0 = k_begin + 64 * wave; tile0 < k_end; tile0 += 64 * NW) {
-    bf16x8 kv[CPR];
+  if (tile0 < k_end && !fetched) {
+    lookup(pg, tile0);
+    load_keys(pg, tile0);
+    if (PIPE) load_values(pg, tile0);
+  }
+  while (tile0 < k_end) {
+    const int next = tile0 + 64 * NW;
+    const bool more = next < k_end;
+    f32x4 sc[4];
 #pragma unroll
-    for (int i = 0; i < CPR; ++i) {
-      const int key = min(tile0 + i * KPI + kgrp, pos);
-      const int page = min(max(tab[key >> page_shift], 0), num_pages - 1);
-      kv[i] = *(const bf16x8*)(k_pages + ((size_t)page * num_kv + kvh) * head_stride +
-                               (size_t)(key & pmask) * head_size + kchunk * 8);
+    for (int kb = 0; kb < 4; ++kb) {
+      f32x4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks)   // a lane's chunk beyond the head's end holds the last chunk again: its query chunk is zero
+        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kb][ks], qf[ks], a, 0, 0, 0);
+      sc[kb] = a;
     }
-    float part[CPR];
-#pragma unroll
-    for (int i = 0; i < CPR; ++i) {
-      float a = 0.f;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) a = fmaf(qf[j], (float)kv[i][j], a);
-      part[i] = a;
+    if (PIPE && more) {
+      lookup(pgn, next);
+      load_keys(pgn, next);
     }
+    // sc[kb][i] of a lane is the score of key tile0 + 32 (kb / 2) + 8 g + 4 (kb % 2) + i, the same in the 16
+    // lanes of a row group
+    const bool edge = tile0 + 64 > k_end || tile0 < lo;
+    float mx = -INFINITY;
 #pragma unroll
-    for (int half = CPR / 2; half >= 1; half >>= 1) {
-      const bool upper = (dchunk & half) != 0;
+    for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-      for (int i = 0; i < half; ++i) {
-        const float keep = upper ? part[i + half] : part[i];
-        const float send = upper ? part[i] : part[i + half];
-        part[i] = keep + __shfl_xor(send, half, 64);
+      for (int i = 0; i < 4; ++i) {
+        if (edge) {
+          const int key = tile0 + 32 * (kb >> 1) + 8 * g + 4 * (kb & 1) + i;
+          if (key < lo || key >= k_end) sc[kb][i] = -INFINITY;
+        }
+        mx = fmaxf(mx, sc[kb][i]);
       }
-    }
-    // this lane now holds the score of key tile0 + dchunk * KPI + kgrp
-    const int mine = dchunk * KPI + kgrp;
-    const bool valid = tile0 + mine >= lo && tile0 + mine < k_end;
-    const float sc = valid ? part[0] : -INFINITY;
-    const float m_new = fmaxf(m, wave_max(sc));
+    mx = rows_max(mx);
+    const float m_new = fmaxf(m, mx);
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
     const float alpha = __expf(m - m_safe);
-    const float p = valid ? __expf(sc - m_safe) : 0.f;
-    l = l * alpha + wave_sum(p);
+    float sum = 0.f;
+    bf16x8 pf[2];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pr = __expf(sc[kb][i] - m_safe);
+        sum += pr;
+        pf[kb >> 1][4 * (kb & 1) + i] = (bf16_t)pr;
+      }
+    l = l * alpha + sum;
     m = m_new;
-    sm_p[wave][mine] = p;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // values of this tile: 8 keys a lane; fetched after the scores so that the registers of the keys are free
-    // again (more waves fit a SIMD, and it is other waves that hide the latency)
-    __builtin_amdgcn_sched_barrier(0);
-    const int kc = lane & 7;
-    const int vkey = min(tile0 + kc * 8, pos & ~7);
-    const int vpage = min(max(tab[vkey >> page_shift], 0), num_pages - 1);
-    const bf16_t* vbase = v_pages + ((size_t)vpage * num_kv + kvh) * head_stride + (vkey & pmask);
-    bf16x8 vv[CPR];
+    if (!PIPE) load_values(pg, tile0);
+    if (edge) {
+      // values of keys that are not the request's (beyond its end, before its window, in a page that was given
+      // back) may be anything: their probabilities are zero, and they must not be NaN
 #pragma unroll
-    for (int i = 0; i < CPR; ++i)
-      vv[i] = *(const bf16x8*)(vbase + (size_t)min(i * 8 + (lane >> 3), head_size - 1) * page_size);
-    float pv[8];
+      for (int st = 0; st < 2; ++st)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) pv[j] = sm_p[wave][kc * 8 + j];
+        for (int j = 0; j < 8; ++j) {
+          const int key = tile0 + 32 * st + 8 * g + j;
+          if (key < lo || key >= k_end) {
 #pragma unroll
-    for (int i = 0; i < CPR; ++i) {
-      float a = acc[i] * alpha;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) a += pv[j] != 0.f ? pv[j] * (float)vv[i][j] : 0.f;
-      acc[i] = a;
+            for (int db = 0; db < NDB; ++db) vf[db][st][j] = 0;
+          }
+        }
     }
-    __builtin_amdgcn_wave_barrier();
-  }
 #pragma unroll
-  for (int i = 0; i < CPR; ++i) {
-    float a = acc[i];
-    a += __shfl_xor(a, 1, 64);
-    a += __shfl_xor(a, 2, 64);
-    a += __shfl_xor(a, 4, 64);
-    if ((lane & 7) == 0) sm_o[wave][i * 8 + (lane >> 3)] = a;
+    for (int db = 0; db < NDB; ++db) {   // blocks beyond the head's end repeat its last row; they are never stored
+      f32x4 a = o[db] * alpha;
+      a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db][0], pf[0], a, 0, 0, 0);
+      a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db][1], pf[1], a, 0, 0, 0);
+      o[db] = a;
+    }
+    if (more) {
+      if (PIPE) {
+        load_values(pgn, next);
+      } else {
+        lookup(pg, next);
+        load_keys(pg, next);
+      }
+    }
+    tile0 = next;
+  }
+  // o[db][i] of a lane is element 16 db + 4 g + i of the weighted values, the same in the 16 lanes of a row group
+  l = rows_sum(l);
+  if (r == 0) {
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sm_o[wave][16 * db + 4 * g + i] = o[db][i];
   }
   if (lane == 0) {
     sm_m[wave] = m;
@@ -1066,10 +1143,11 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, 
                                               bf16_t* __restrict__ out, int num_heads, int head_size,
                                               int num_splits) {
   const int h = blockIdx.x, dz = blockIdx.y;
-  const int t = run_start[decode_runs[dz]];
+  const int run = decode_runs[dz];            // where the result goes is asked for beside the partial results
   const size_t base = ((size_t)dz * num_heads + h) * num_splits;
   float mm = -INFINITY;
   for (int s = 0; s < num_splits; ++s) mm = fmaxf(mm, part_ml[(base + s) * 2]);
+  const int t = run_start[run];
   for (int d = threadIdx.x; d < head_size; d += blockDim.x) {
     float ll = 0.f, oo = 0.f;
     for (int s = 0; s < num_splits; ++s) {
@@ -1101,29 +1179,33 @@ static int attention_decode_run(const void* q, const void* k_pages, const void* 
               "attention_decode: blocks have 4 waves, or 8 up to head size 128; not %d at head size %d", waves, head_size);
   if (num_decode <= 0) return 0;
   dim3 grid(num_splits, num_heads, num_decode);
-#define LAUNCH_DECODE_ARGS                                                                                          \
-  (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, table_width,     \
-      page_shift, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window, num_splits,     \
-      longest, head_size
-#define LAUNCH_DECODE(CPR)                                                                                         \
-  if (waves == 8)                                                                                                  \
-    attention_decode_kernel<CPR, 8><<<grid, 512, 0, stream>>>(LAUNCH_DECODE_ARGS);                                 \
-  else                                                                                                             \
-    attention_decode_kernel<CPR, 4><<<grid, 256, 0, stream>>>(LAUNCH_DECODE_ARGS)
-  // the lanes' layout is that of the next power of two; a smaller head leaves some lanes idle
-  if (head_size <= 16) {
-    LAUNCH_DECODE(2);
-  } else if (head_size <= 32) {
-    LAUNCH_DECODE(4);
-  } else if (head_size <= 64) {
-    LAUNCH_DECODE(8);
-  } else if (head_size <= 128) {
-    LAUNCH_DECODE(16);
-  } else {
-    attention_decode_kernel<32, 4><<<grid, 256, 0, stream>>>(LAUNCH_DECODE_ARGS);
-  }
-#undef LAUNCH_DECODE
-#undef LAUNCH_DECODE_ARGS
+#define LAUNCH_MFMA(NDB)                                                                                          \
+  if (waves == 8)                                                                                                 \
+    attention_decode_mfma_kernel<NDB, 8><<<grid, 512, 0, stream>>>(                                               \
+        (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table,          \
+        table_width, page_shift, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window, \
+        num_splits, longest, head_size);                                                                          \
+  else                                                                                                            \
+    attention_decode_mfma_kernel<NDB, 4><<<grid, 256, 0, stream>>>(                                               \
+        (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table,          \
+        table_width, page_shift, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window, \
+        num_splits, longest, head_size)
+    // the registers are laid out for the next of these sizes; a smaller head repeats its last chunk there
+    if (head_size <= 32) {
+      LAUNCH_MFMA(2);
+    } else if (head_size <= 64) {
+      LAUNCH_MFMA(4);
+    } else if (head_size <= 96) {
+      LAUNCH_MFMA(6);
+    } else if (head_size <= 128) {
+      LAUNCH_MFMA(8);
+    } else {
+      attention_decode_mfma_kernel<16, 4><<<grid, 256, 0, stream>>>(
+          (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table,
+          table_width, page_shift, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window,
+          num_splits, longest, head_size);
+    }
+#undef LAUNCH_MFMA
   TNX_CHECK_LAUNCH("attention_decode");
   if (num_splits > 1) {
     attention_decode_merge_kernel<<<dim3(num_heads, num_decode), head_size < 64 ? 64 : head_size, 0, stream>>>(
