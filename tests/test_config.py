@@ -122,3 +122,24 @@ def test_auto_model_picks_the_class_the_folder_names(tmp_path):
     (bad / "config.json").write_text(json.dumps(dict(TINY_A, architectures=["LlamaForCausalLM"], model_type="llama")))
     with pytest.raises(AssertionError, match="not supported"):
         NeuronAutoModelForCausalLM.from_pretrained(str(bad))
+
+
+def test_console_scripts_of_the_package_resolve():
+    """pyproject.toml names the reference's console scripts for this architecture and the trace replay."""
+    import importlib
+    import os
+    try:
+        import tomllib
+    except ImportError:
+        tomllib = pytest.importorskip("tomli")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with open(os.path.join(root, "pyproject.toml"), encoding="utf-8") as fp:
+        project = tomllib.loads(fp.read())
+    scripts = project["project"]["scripts"]
+    assert set(scripts) == {"opt_demo", "opt_gen_random_pretrained", "trace_run"}
+    for target in scripts.values():
+        module, _, name = target.partition(":")
+        assert callable(getattr(importlib.import_module(module), name))
+    for package in project["tool"]["setuptools"]["packages"]:
+        folder = package.replace("transformers_neuronx_amd", "transformers-neuronx_amd").replace(".", "/")
+        assert os.path.isfile(os.path.join(root, folder, "__init__.py")), package

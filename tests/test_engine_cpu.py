@@ -475,3 +475,34 @@ def test_model_without_the_norm_before_the_head(tmp_path):
     with_norm["model.decoder.final_layer_norm.bias"] = torch.randn(64, generator=g)
     other = plain_opt.forward_logits(with_norm, TINY_A, toks)
     assert float((other - want).abs().max()) > 1e-2
+
+
+def test_tapped_tensors_are_the_plain_intermediates(tiny_folders):
+    """Inside a debug context a step keeps the tensors the model taps: the embedded tokens, the stream after
+    every layer call, the stream between a block's halves, the logits. They are the plain implementation's."""
+    from transformers_neuronx_amd import debug
+    folder, cfg, weights = tiny_folders["A"]
+    toks = _requests(cfg["vocab_size"], [19], 2)["r0"]
+    runner, _ = _runner(folder, 64)
+    assert not debug.active()
+    with debug.debug_context() as kept:
+        assert debug.active()
+        runner.step([StepEntry("a", toks, [len(toks) - 1])])
+    assert not debug.active()
+    assert list(kept) == ["embedding", "after_mixer", "call0.layer0", "after_mixer#2", "call1.layer1", "logits"]
+    x = plain_opt.embed(torch.tensor(toks), weights, cfg)
+    assert float((kept["embedding"] - x).abs().max()) < 1e-6
+    for i in range(2):
+        x = plain_opt.block(x, weights, cfg, i)
+        assert float((kept[f"call{i}.layer{i}"] - x).abs().max()) < 1e-5
+    assert float((kept["logits"][0] - plain_opt.head(x, weights, cfg)[-1]).abs().max()) < 1e-5
+    # outside a context nothing is kept, and the step is the same
+    again = runner.step([StepEntry("b", toks, [len(toks) - 1])])
+    assert torch.equal(again, kept["logits"])
+
+
+def test_percentiles_of_the_benchmark_report():
+    from transformers_neuronx_amd.opt.demo import percentile
+    values = [5.0, 1.0, 4.0, 2.0, 3.0]
+    assert [percentile(values, q) for q in (0, 50, 90, 95, 99, 100)] == [1.0, 3.0, 5.0, 5.0, 5.0, 5.0]
+    assert percentile([7.0], 50) == 7.0 and percentile(list(range(10)), 50) == 5 and percentile(list(range(10)), 96) == 9

@@ -195,6 +195,25 @@ def test_toy_rotating_parts_on_the_gpu(dtype):
     assert "toy_norm" in hip.loaded_libraries()
 
 
+def test_benchmark_report_and_kernel_times(tiny_folders_bf16, capsys):
+    """`opt_demo run --benchmark --profile`: the reference's report (warm-up, timed generations, latency
+    percentiles) and the time of every kernel of a prompt step and a decode step."""
+    from transformers_neuronx_amd.opt import demo
+    folder = tiny_folders_bf16["C"][0]
+    assert demo.main(["--amp", "bf16", "run", folder, "--batch_size", "2", "--n_positions", "40", "--prompt_len", "9",
+                      "--top_k", "1", "--benchmark", "--profile", "--page_size", "16"]) in (0, None)
+    text = capsys.readouterr().out
+    report = json.loads(next(line for line in text.splitlines() if line.startswith("{")))
+    assert report["iterations"] == 5 and report["inferences"] == 10 and report["context_length"] == 9
+    pct = report["sequence_latency_percentiles"]
+    assert 0 < pct["sequence_latency_p0"] <= pct["sequence_latency_p50"] <= pct["sequence_latency_p100"]
+    assert report["e2e_output_token_throughput"] > 0 and report["mean_output_token_latency"] > 0
+    assert report["mean_context_encoding_latency"] > 0
+    for kernel in ("tnx_layernorm", "tnx_gemm_bf16", "tnx_attention_prefill", "tnx_attention_decode", "tnx_argmax"):
+        assert kernel in text, kernel
+    assert "prompt step" in text and "decode step" in text
+
+
 def test_trace_run_as_a_program(tiny_folders, tmp_path):
     import subprocess
     import sys

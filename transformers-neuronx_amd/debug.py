@@ -1,0 +1,82 @@
+"""Looking inside a step: intermediate tensors by name, and the time of every kernel.
+
+`tap(name, tensor)` is called by the model at fixed places (after the embedding, after every layer call,
+inside the block arrangements); it does nothing unless a `debug_context()` is open, in which case a copy
+of the tensor is kept under its name (reference: global_debugger.py:27-92, `tap` and `debug_context`,
+where a tapped tensor becomes one more output of the compiled graph; here it is simply copied). A step
+that runs inside a debug context or under a kernel timer is never replayed from a recording.
+
+`KernelTimer` brackets every launch of the HIP backend with events (reference: base.py:754-759,
+`profile`, which asks its runtime for a trace per compiled kernel).
+"""
+import contextlib
+from collections import OrderedDict
+from typing import Dict, List, Optional
+
+import torch
+
+_tapped: Optional["OrderedDict[str, torch.Tensor]"] = None
+_timer: Optional["KernelTimer"] = None
+
+
+def active() -> bool:
+    return _tapped is not None or _timer is not None
+
+
+def tap(name: str, tensor):
+    """Keep a copy of `tensor` under `name` if a debug context is open; returns the tensor."""
+    if _tapped is not None and tensor is not None:
+        key, n = name, 1
+        while key in _tapped:               # a name used again (a later step): numbered
+            n += 1
+            key = f"{name}#{n}"
+        _tapped[key] = tensor.detach().clone()
+    return tensor
+
+
+@contextlib.contextmanager
+def debug_context():
+    """`with debug_context() as tensors:` runs steps with every tapped tensor kept in `tensors`."""
+    global _tapped
+    _tapped = OrderedDict()
+    try:
+        yield _tapped
+    finally:
+        _tapped = None
+
+
+class KernelTimer:
+    """Events around every launch; `table()` sums them by kernel name after a synchronize."""
+
+    def __init__(self):
+        self.spans: List[tuple] = []
+
+    def start(self, name: str):
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        begin.record()
+        self.spans.append((name, begin, end))
+        return end
+
+    def table(self) -> Dict[str, tuple]:
+        torch.cuda.synchronize()
+        out: Dict[str, list] = {}
+        for name, begin, end in self.spans:
+            row = out.setdefault(name, [0, 0.0])
+            row[0] += 1
+            row[1] += begin.elapsed_time(end)
+        return {k: (v[0], v[1]) for k, v in sorted(out.items(), key=lambda kv: -kv[1][1])}
+
+
+def timer() -> Optional[KernelTimer]:
+    return _timer
+
+
+@contextlib.contextmanager
+def kernel_timer():
+    """`with kernel_timer() as t:` times every launch of the HIP backend; `t.table()` is {name: (calls, ms)}."""
+    global _timer
+    _timer = KernelTimer()
+    try:
+        yield _timer
+    finally:
+        _timer = None

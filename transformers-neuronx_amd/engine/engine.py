@@ -148,6 +148,23 @@ class LLMEngine:
         self._started = started
         return out
 
+    def profile(self, steps: int = 1):
+        """Run `steps` steps with events around every kernel launch (no recording, no running ahead) and
+        return ({kernel: (launches, milliseconds)}, the steps' outputs). Reference: `profile`, base.py:754-759."""
+        from .. import debug
+        ahead, self.run_ahead = self.run_ahead, False
+        outs: List[StepOutput] = []
+        try:
+            with debug.kernel_timer() as t:
+                for _ in range(steps):
+                    if not self.has_work:
+                        break
+                    outs += self.step()
+                table = t.table()
+        finally:
+            self.run_ahead = ahead
+        return table, outs
+
     def run(self, on_token: Optional[Callable[[StepOutput], None]] = None) -> None:
         """Step until every request has ended."""
         while self.has_work:

@@ -12,6 +12,7 @@ import torch
 from ..parts.base import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, CacheNeed, Stream
 from ..parts.spec import LayerSpec, ModelSpec, ParamDecl
 from ..weights.loader import load_tensors
+from .. import debug
 
 
 class _Layer:
@@ -97,10 +98,12 @@ class DecoderModel:
         first_block = self.layers[self.schedule[0][0]].block if self.schedule else None
         want_compute = bool(getattr(first_block, "reads_compute_copy", False))
         stream: Stream = self.embedding.forward(ctx, want_compute)
-        for layer, cid, writes in self.schedule:
+        debug.tap("embedding", stream.x)
+        for call, (layer, cid, writes) in enumerate(self.schedule):
             cache = caches[cid] if writes else caches[cid].reader()
             stream = self.layers[layer].block.forward(stream, ctx, cache)
-        return self.head.forward(stream, ctx)
+            debug.tap(f"call{call}.layer{layer}", stream.x)
+        return debug.tap("logits", self.head.forward(stream, ctx))
 
 
 def model_param_decls(spec: ModelSpec) -> List[ParamDecl]:

@@ -58,3 +58,27 @@ def replay(lines: Iterable[str], runner, out_dir: str, out: Optional[TextIO] = N
         print(f"done {step}", file=out, flush=True)
         n += 1
     return n
+
+
+def main(argv=None) -> int:
+    """`trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N < steps.jsonl`"""
+    import argparse
+    ap = argparse.ArgumentParser(prog="trace_run", description=__doc__,
+                                 formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
+    ap.add_argument("--out", required=True, help="folder the logits are written to")
+    ap.add_argument("--max-tokens", type=int, required=True,
+                    help="the most tokens live requests hold at a time (each request's count in whole pages)")
+    ap.add_argument("--page-size", type=int, default=64, help="tokens per cache page (divides 64 or is a multiple)")
+    ap.add_argument("--device", default="cuda:0")
+    args = ap.parse_args(argv)
+    if not os.environ.get("HOME") or not os.access(os.environ.get("HOME", "/"), os.W_OK):
+        # libraries that want a writable home get a private temporary one
+        import tempfile
+        os.environ["HOME"] = tempfile.mkdtemp(prefix="trace_run_home_")
+    print("[trace_run] loading the model ...", file=sys.stderr, flush=True)
+    runner = make_replay_runner(args.model, args.dtype, args.max_tokens, args.page_size, args.device)
+    print("[trace_run] ready", file=sys.stderr, flush=True)
+    replay(sys.stdin, runner, args.out)
+    return 0

@@ -17,6 +17,7 @@ import torch
 import numpy as np
 
 from ..cache.manager import CacheManager
+from .. import debug
 from .batch import PackedStep, StepContext, StepEntry, context_from, pack_step
 from .model import DecoderModel
 
@@ -140,7 +141,8 @@ class ModelRunner:
         their `want`; None when nothing is wanted (the step still runs)."""
         if not entries:
             return None
-        recordable = self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
+        recordable = (self.use_graphs and not debug.active()
+                      and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries))
         packed = self.prepare(entries, fixed_width=recordable, kept_allowed=kept_allowed)
         if recordable:
             key = packed.layout()

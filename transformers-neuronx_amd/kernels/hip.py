@@ -12,6 +12,7 @@ import numpy as np
 import torch
 
 from . import build
+from .. import debug
 
 _F32, _BF16 = 0, 1
 _ACT = {None: 0, "none": 0, "relu": 1, "gelu": 2, "gelu_new": 3}
@@ -164,7 +165,11 @@ class HipOps:
 
     def _call(self, module: str, fn: str, *args):
         lib = library(module)
+        timer = debug.timer()
+        end = timer.start(fn) if timer is not None else None
         rc = getattr(lib, fn)(*args)
+        if end is not None:
+            end.record()
         if rc != 0:
             raise RuntimeError(f"{fn}: {lib.tnx_last_error().decode()}")
 
@@ -380,7 +385,11 @@ class HipOps:
             return lib.tnx_gemm_library(_ptr(xa), _ptr(w), _ptr(bias), _ptr(residual), _ptr(out), _code(out.dtype),
                                         _ACT[act], m, n, k, _ptr(space), space.numel(), _ptr(flush),
                                         flush.numel() if flush is not None else 0, int(tune), _stream())
+        timer = debug.timer()
+        end = timer.start("tnx_gemm_library") if timer is not None else None
         rc = call(None, self.library_tune)
+        if end is not None:
+            end.record()
         if rc == 3:
             # the algorithms for this size are timed now, once: with memory to push the operands out of the
             # caches, as large as the last-level cache; without it, if the device has no room, nothing is timed

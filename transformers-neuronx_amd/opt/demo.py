@@ -3,7 +3,7 @@
     opt_demo [--amp f32|bf16] save DIR --random --config CONFIG.json [--seed N]
     opt_demo [--amp f32|bf16] run DIR [--batch_size 4] [--n_positions 128] [--print_latency]
              [--prompt_len N | --prompt_ids 5,6,7] [--top_k 50] [--top_p 1.0] [--temperature 1.0]
-             [--do_sample] [--max_new_tokens N] [--seed N] [--benchmark]
+             [--do_sample] [--max_new_tokens N] [--seed N] [--benchmark] [--profile]
              [--dump_logits DIR [--dump_logits_limit N]]
     opt_demo analyze -d DIR [DIR ...] GOLDEN_DIR
 
@@ -56,7 +56,11 @@ def _parser():
     run.add_argument("--dump_logits", type=str, default=None,
                      help="folder for the logits that each generated token was chosen from: <step>.pt, [batch, vocab]")
     run.add_argument("--dump_logits_limit", type=int, default=1, help="how many steps to dump; -1 for all")
-    run.add_argument("--benchmark", action="store_true")
+    run.add_argument("--benchmark", action="store_true",
+                     help="2 warm-up generations, then 5 timed ones: latency percentiles of a whole sequence, "
+                          "context encoding and output token latency, throughput")
+    run.add_argument("--profile", action="store_true",
+                     help="time every kernel of one prompt step and one decode step and print the table")
     run.add_argument("--page_size", type=int, default=64)
     return parser
 
@@ -107,13 +111,14 @@ def run(args):
                 order = sorted(range(len(requests)), key=lambda i: requests[i].req_id)
                 dumped.append(logits[order].cpu())
         model.engine.logits_hook = keep
-    if args.print_latency or args.benchmark:
+    if args.print_latency:
         model.engine.record_timings = True
     print("running model.sample")
-    start = time.time()
-    out = model.sample(input_ids, sequence_length=total, top_k=args.top_k, temperature=args.temperature,
-                       top_p=args.top_p, seed=args.seed, generation_config=gen)
-    elapsed = time.time() - start
+
+    def generate():
+        return model.sample(input_ids, sequence_length=total, top_k=args.top_k, temperature=args.temperature,
+                            top_p=args.top_p, seed=args.seed, generation_config=gen)
+    out = generate()
     print("generated_sequence=", out)
     for i, logits in enumerate(dumped):
         torch.save(logits, os.path.join(args.dump_logits, f"{i}.pt"))
@@ -123,16 +128,63 @@ def run(args):
         for rec in model.engine.timings:
             print(f"Latency: {math.ceil(rec['seconds'] * 1000)} ms ({rec['tokens']} tokens)")
     if args.benchmark:
-        t = model.engine.timings
-        prefill = [r for r in t if r["prefill_tokens"]]
-        decode = [r for r in t if not r["prefill_tokens"]]
-        new = (total - input_ids.shape[1]) * args.batch_size
-        report = {
-            "mean_context_encoding_latency_ms": 1000 * sum(r["seconds"] for r in prefill) / max(1, len(prefill)),
-            "mean_output_token_latency_ms": 1000 * sum(r["seconds"] for r in decode) / max(1, len(decode)),
-            "e2e_output_token_throughput": new / elapsed,
-        }
-        print(json.dumps(report))
+        model.engine.logits_hook = None
+        print(json.dumps(benchmark(model, generate, args.batch_size, input_ids.shape[1], total)))
+    if args.profile:
+        from ..sampling.params import SamplingParams
+        engine = model.engine
+        engine.reset()
+        for row in input_ids.tolist():
+            engine.add_request(row, SamplingParams(max_new_tokens=3, do_sample=False, ignore_eos=True))
+        for title in ("prompt step", "decode step"):
+            table, _ = engine.profile(1)
+            print(f"{title}: {sum(ms for _, ms in table.values()):.3f} ms in kernels")
+            for name, (calls, ms) in table.items():
+                print(f"  {name:32s} {calls:5d} launches {ms:9.3f} ms")
+        engine.reset()
+
+
+def percentile(values, percent):
+    """The reference's percentile of a list (generation_demo.py:96-105): the element at `len * percent / 100`,
+    rounded down unless its fraction is above one half, and never beyond the last."""
+    ordered = sorted(values)
+    pos = len(ordered) * percent / 100
+    last = len(ordered) - 1
+    low, high = min(math.floor(pos), last), min(math.ceil(pos), last)
+    return ordered[high] if pos - low > 0.5 else ordered[low]
+
+
+def benchmark(model, generate, batch_size, context_length, output_length, warmup=2, iterations=5):
+    """The reference's benchmark report (generation_demo.py:107-187): `warmup` whole generations, then
+    `iterations` timed ones; latency percentiles of a whole sequence, mean latency of the context encoding
+    (the steps that take prompts in) and of an output token, and throughput."""
+    engine = model.engine
+    print(f"Warmup ({warmup} iterations) ...")
+    for _ in range(warmup):
+        generate()
+    print(f"Benchmark loop ({iterations} iterations) ...")
+    latencies, context = [], []
+    engine.record_timings = True
+    begin = time.time()
+    for _ in range(iterations):
+        engine.timings.clear()
+        start = time.time()
+        generate()
+        latencies.append((time.time() - start) * 1000)
+        context.append(1000 * sum(r["seconds"] for r in engine.timings if r["prefill_tokens"]))
+    duration = time.time() - begin
+    engine.record_timings = False
+    new = output_length - context_length
+    return {
+        "sequence_length": output_length, "context_length": context_length, "output_length": output_length,
+        "batch_size": batch_size, "iterations": iterations, "batches": len(latencies),
+        "inferences": len(latencies) * batch_size, "total_duration_seconds": duration,
+        "mean_context_encoding_latency": sum(context) / len(context),
+        "e2e_output_token_throughput": len(latencies) * batch_size * new / duration,
+        "mean_output_token_latency": (sum(latencies) - sum(context)) / len(latencies) / max(1, new),
+        "sequence_latency_percentiles": {f"sequence_latency_p{q}": percentile(latencies, q)
+                                         for q in (0, 50, 90, 95, 99, 100)},
+    }
 
 
 def analyze(args):

@@ -1,4 +1,5 @@
 """Arrangements of a layer's parts around the residual stream."""
+from .. import debug
 from .base import Block, Stream, register_block
 
 
@@ -12,7 +13,7 @@ class PreNormBlock(Block):
 
     def forward(self, stream: Stream, ctx, cache) -> Stream:
         _, h = self.mixer_norm.forward(stream.x, False, True)
-        x = self.mixer.forward(h, ctx, cache, stream.x)
+        x = debug.tap("after_mixer", self.mixer.forward(h, ctx, cache, stream.x))
         _, h = self.feed_forward_norm.forward(x, False, True)
         x = self.feed_forward.forward(h, ctx, x)
         return Stream(x, None)
@@ -31,6 +32,7 @@ class PostNormBlock(Block):
         h = stream.compute if stream.compute is not None else self.mixer_norm.ops.cast(stream.x, self.mixer_norm.dtype)
         t = self.mixer.forward(h, ctx, cache, stream.x)
         x, h = self.mixer_norm.forward(t, True, True)
+        debug.tap("after_mixer", x)
         t = self.feed_forward.forward(h, ctx, x)
         x, h = self.feed_forward_norm.forward(t, True, True)
         return Stream(x, h)
