@@ -67,6 +67,8 @@ def main():
     ap.add_argument("--mix", action="store_true",
                     help="instead: 64 requests with prompts of 16 to 1,024 tokens and 256 new tokens each, all "
                          "queued at once (a continuous-batching workload); prints its own line")
+    ap.add_argument("--own-products", action="store_true",
+                    help="every matrix product on our own kernels (none goes to the vendor library)")
     ap.add_argument("--big-batch", type=int, default=64, help="the larger batch of `points` (cut to what fits the device at the full context)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -80,6 +82,9 @@ def main():
     from transformers_neuronx_amd.engine.factory import runner_from_random
     from transformers_neuronx_amd.sampling import SamplingParams
 
+    if args.own_products:
+        from transformers_neuronx_amd.kernels.hip import HipOps
+        HipOps.library_rows = 0
     raw = dict(MODEL)
     raw.update(OTHER_MODELS.get(args.model, {}))
     layers_full = raw["num_hidden_layers"]

@@ -66,7 +66,9 @@ def test_gather_embed_positions_cast(dtype):
 
 
 GEMM_SHAPES = [(1, 16, 8), (3, 50, 24), (8, 96, 96), (17, 1000, 48), (64, 320, 96), (65, 130, 72),
-               (130, 257, 136), (300, 96, 320), (5, 4096, 512), (40, 136, 1024), (12, 70, 1000), (16, 33, 264)]
+               (130, 257, 136), (300, 96, 320), (5, 4096, 512), (40, 136, 1024), (12, 70, 1000), (16, 33, 264),
+               # many rows, whole 64-steps of K: the wide-tile kernel, with tiles that reach beyond M and N
+               (128, 264, 64), (257, 1000, 192), (700, 520, 1024), (2048, 256, 128)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

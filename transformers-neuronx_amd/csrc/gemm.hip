@@ -1,9 +1,12 @@
 // Matrix products `out[M, N] = act(x[M, K] w[N, K]^T + bias[N]) + residual[M, N]` with float32 accumulation.
 //   gemm_f32        float32 operands, plain FMA (no matrix-core mode of reduced precision)
-//   gemm_bf16       bfloat16 operands on MFMA, 128x128 tiles staged through LDS (many rows: prompts)
+//   gemm_bf16       bfloat16 operands on MFMA, many rows (prompts): 256x256x64 tiles, operands straight from
+//                   global memory into two LDS stages, four waves of 128x128 (sizes in whole 64-steps of K);
+//                   128x128 tiles staged through registers for every other size
 //   gemm_bf16_skinny  bfloat16 operands on MFMA for M <= 64 (decoding): streams the weight once
 // bias and residual are float32 and optional; the output is float32 or bfloat16.
 #include "common.h"
+#include <type_traits>
 
 TNX_DEFINE_ERROR_API
 
@@ -283,6 +286,241 @@ gemm_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, con
     }
 }
 
+// ------------------------------------------------------------------------------------------ bfloat16, wide tiles
+
+#define WT_M 256
+#define WT_N 256
+typedef __attribute__((address_space(3))) void* lds_ptr;
+typedef const __attribute__((address_space(1))) void* glb_ptr;
+
+// out[M][N] = x[M][K] w[N][K]^T. Tiles of 64 MI x 256 x BK (MI 4: 256 rows, MI 2: 128 rows, for results too
+// narrow to give every compute unit a tile of 256), four waves (2 x 2), each 32 MI x 128 of the result as
+// MI x 4 MFMA 32x32x16 tiles (64 MI accumulator registers; a fragment read from LDS serves four products).
+// Operand tiles go from global memory straight into LDS, NSTAGE stages deep, 16-byte chunks swizzled by row
+// so that the fragment reads are free of bank conflicts (the banks repeat every 256 bytes).
+template <int BK, int NSTAGE, int MI>
+__global__ void __launch_bounds__(256, 1)
+gemm_bf16_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
+                const float* __restrict__ residual, void* __restrict__ out, int out_dtype, int act, int M, int N,
+                int K, int tiles_m, int tiles_n) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int CPR = BK / 8;                     // 16-byte chunks a row
+  constexpr int ROWB = BK * 2;                    // bytes a row
+  constexpr int TM = 64 * MI;                     // rows of x a tile takes
+  constexpr int STAGE = (TM + WT_N) * ROWB;       // bytes of one stage
+  constexpr int RPI = 64 / CPR;                   // rows a wave's load instruction covers
+  constexpr int LPA = TM / (4 * RPI);             // load instructions a wave issues for a tile of x
+  constexpr int LPT = WT_N / (4 * RPI);           // and of w
+  constexpr int KS = BK / 16;                     // k16 steps
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = (wave & 1) * 32 * MI, wn = (wave >> 1) * 128;
+  const int nb = tiles_m * tiles_n;
+  int bid = blockIdx.x;
+  if (nb % 8 == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3);
+  const int tm = bid % tiles_m, tn = bid / tiles_m;
+  const int m0 = tm * TM, n0 = tn * WT_N;
+  const int l32 = lane & 31, lhalf = lane >> 5;
+
+  f32x16 acc[MI][4];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // 16 lanes are served a cycle and the banks repeat every 256 bytes: 16 consecutive rows must put the chunk
+  // they read into 16 different 16-byte places of those 256 bytes
+  auto swz = [&](int row) { return CPR == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3); };
+  const int lrow = lane / CPR, lpos = lane % CPR;
+  const bf16_t* xsrc[LPA];
+  const bf16_t* wsrc[LPT];
+#pragma unroll
+  for (int j = 0; j < LPA; ++j) {
+    const int row = (LPA * wave + j) * RPI + lrow;
+    xsrc[j] = x + (size_t)min(m0 + row, M - 1) * K + 8 * (lpos ^ swz(row));
+  }
+#pragma unroll
+  for (int j = 0; j < LPT; ++j) {
+    const int row = (LPT * wave + j) * RPI + lrow;
+    wsrc[j] = w + (size_t)min(n0 + row, N - 1) * K + 8 * (lpos ^ swz(row));
+  }
+  auto issue_part = [&](int stage, int k0, int part, int parts) {      // loads part, part + parts, ... of a tile
+    char* a_dst = smem + stage * STAGE + (LPA * wave) * 1024;
+    char* b_dst = smem + stage * STAGE + TM * ROWB + (LPT * wave) * 1024;
+#pragma unroll
+    for (int j = 0; j < LPA; ++j)
+      if (j % parts == part)
+        __builtin_amdgcn_global_load_lds((glb_ptr)(xsrc[j] + k0), (lds_ptr)(a_dst + j * 1024), 16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < LPT; ++j)
+      if (j % parts == part)
+        __builtin_amdgcn_global_load_lds((glb_ptr)(wsrc[j] + k0), (lds_ptr)(b_dst + j * 1024), 16, 0, 0);
+  };
+  auto issue = [&](int stage, int k0) { issue_part(stage, k0, 0, 1); };
+  int a_off[MI], b_off[4];
+#pragma unroll
+  for (int i = 0; i < MI; ++i) a_off[i] = (wm + 32 * i + l32) * ROWB;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) b_off[j] = TM * ROWB + (wn + 32 * j + l32) * ROWB;
+  const int rsw = swz(l32);
+
+  const int steps = K / BK;
+#pragma unroll
+  for (int p = 0; p < NSTAGE - 1; ++p)
+    if (p < steps) issue(p, p * BK);
+  bf16x8 a[2][MI], b[2][4];
+  auto frags = [&](int slot, const char* base, int s) {
+    const int coff = ((2 * s + lhalf) ^ rsw) * 16;
+#pragma unroll
+    for (int i = 0; i < MI; ++i) a[slot][i] = *(const bf16x8*)(base + a_off[i] + coff);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) b[slot][j] = *(const bf16x8*)(base + b_off[j] + coff);
+  };
+  auto products = [&](int slot) {
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[slot][j], a[slot][i], acc[i][j], 0, 0, 0);
+  };
+  int stage = 0;
+  auto iteration = [&](int t, auto with_loads) {
+    constexpr bool more = decltype(with_loads)::value;
+    // tile t has landed when at most the loads of the NSTAGE - 2 tiles after it are still in flight
+    const int ahead = min(NSTAGE - 2, steps - 1 - t);
+    if (ahead >= 2) __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * (LPA + LPT)) & 15) | (((2 * (LPA + LPT)) >> 4) << 14));
+    else if (ahead == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | ((LPA + LPT) & 15) | (((LPA + LPT) >> 4) << 14));
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    // the stage that tile t - 1 was read from is free now: tile t + NSTAGE - 1 goes there, its loads spread
+    // over this tile's steps between the products
+    const int nstage = (stage + NSTAGE - 1) % NSTAGE, nk = (t + NSTAGE - 1) * BK;
+    const char* base = smem + stage * STAGE;
+    frags(0, base, 0);
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      // the next step's fragments are asked for first, in one run; this step's products run while they arrive
+      if (s + 1 < KS) frags((s + 1) & 1, base, s + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      if (more) {
+        issue_part(nstage, nk, s, KS);
+        products(s & 1);
+#pragma unroll
+        for (int g = 0; g < (LPA + LPT) / KS; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 4 * MI * KS / (LPA + LPT), 0);
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+      } else {
+        products(s & 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    stage = stage + 1 == NSTAGE ? 0 : stage + 1;
+  };
+  int t = 0;
+  for (; t + NSTAGE - 1 < steps; ++t) iteration(t, std::true_type{});
+  for (; t < steps; ++t) iteration(t, std::false_type{});
+  // acc[i][j][e] of a lane is out[m][n] at m = 32 i + lane % 32, n = 32 j + 8 (e / 4) + 4 (lane / 32) + e % 4 of the
+  // wave's 32 MI x 128: four consecutive n a register group. A block of 32 rows at a time goes through LDS (the
+  // stages are free now), so that rows are written to memory 16 bytes a lane, whole lines at a time.
+  __syncthreads();
+  const bool relu = act == TNX_ACT_RELU;
+  const bool wide = out_dtype == TNX_F32;
+  const int esz = wide ? 4 : 2;
+  const int rowb = 128 * esz + 16;                     // bytes of a staged row, padded against bank conflicts
+  char* mine = smem + wave * (32 * (128 * 4 + 16));
+#pragma unroll
+  for (int i = 0; i < MI; ++i) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int nl = 32 * j + 8 * q + 4 * lhalf;     // first of this lane's four columns within the wave's 128
+        const int n = n0 + wn + nl;
+        float v[4];
+        f32x4 bv = {0.f, 0.f, 0.f, 0.f};
+        if (bias) bv = *(const f32x4*)(bias + min(n, N - 4));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] = acc[i][j][4 * q + e] + bv[e];
+          if (relu) v[e] = fmaxf(v[e], 0.f);
+        }
+        char* dst = mine + l32 * rowb + nl * esz;
+        if (wide) {
+          *(f32x4*)dst = (f32x4){v[0], v[1], v[2], v[3]};
+        } else {
+          bf16x4 pk = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
+          *(bf16x4*)dst = pk;
+        }
+      }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // read back: a row of 128 outputs is 16 (bfloat16) or 32 (float32) chunks of 16 bytes
+    const int cpr_out = 128 * esz / 16;
+    const int rows_pass = 64 / cpr_out;
+    for (int r0 = 0; r0 < 32; r0 += rows_pass) {
+      const int r = r0 + lane / cpr_out, c = lane % cpr_out;
+      const int m = m0 + wm + 32 * i + r;
+      const int n = n0 + wn + c * (16 / esz);
+      f32x4 raw = *(const f32x4*)(mine + r * rowb + c * 16);
+      if (m < M && n < N) {          // N is a multiple of 8 here: a chunk is inside or outside as a whole
+        const size_t idx = (size_t)m * N + n;
+        if (wide) {
+          if (residual) {
+            const f32x4 rv = *(const f32x4*)(residual + idx);
+            raw += rv;
+          }
+          *(f32x4*)((float*)out + idx) = raw;
+        } else {
+          *(f32x4*)((bf16_t*)out + idx) = raw;
+        }
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+}
+
+
+// Where the wide-tile kernel can stand in: whole chunks of 16 bytes in every row of the result, K in steps of 64,
+// a residual only beside a float32 result, and enough rows to fill its tiles.
+static bool wide_tiles_fit(int M, int N, int K, const float* residual, int out_dtype, int act) {
+  return M >= 128 && K % 64 == 0 && N % 8 == 0 && (residual == nullptr || out_dtype == TNX_F32) &&
+         (act == TNX_ACT_NONE || act == TNX_ACT_RELU);
+}
+
+template <int MI>
+static int launch_wide_tiles(const bf16_t* x, const bf16_t* w, const float* bias, const float* residual, void* out,
+                             int out_dtype, int act, int M, int N, int K, hipStream_t stream) {
+  constexpr int TM = 64 * MI;
+  const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + WT_N - 1) / WT_N;
+  constexpr int bytes = 2 * (TM + WT_N) * 64 * 2;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_wide_kernel<64, 2, MI>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) {
+      tnx_set_error("gemm_bf16: cannot reserve %d bytes of LDS: %s", bytes, hipGetErrorString(e));
+      return 2;
+    }
+    configured = true;
+  }
+  gemm_bf16_wide_kernel<64, 2, MI><<<tiles_m * tiles_n, 256, bytes, stream>>>(x, w, bias, residual, out, out_dtype,
+                                                                             act, M, N, K, tiles_m, tiles_n);
+  return 0;
+}
+
+static int launch_wide(const bf16_t* x, const bf16_t* w, const float* bias, const float* residual, void* out,
+                       int out_dtype, int act, int M, int N, int K, hipStream_t stream) {
+  // tiles of 256 rows where they give (nearly) every compute unit one, tiles of 128 rows otherwise
+  const int full = ((M + 255) / 256) * ((N + WT_N - 1) / WT_N);
+  if (full >= 200) return launch_wide_tiles<4>(x, w, bias, residual, out, out_dtype, act, M, N, K, stream);
+  return launch_wide_tiles<2>(x, w, bias, residual, out, out_dtype, act, M, N, K, stream);
+}
+
 // ------------------------------------------------------------------------------------------ bfloat16, few rows
 
 // One block of WAVES waves makes 16 * RT columns of the output (RT tiles of 16 rows of `w`) for all
@@ -473,6 +711,13 @@ static int gemm_bf16_dispatch(const void* x, const void* w, const void* w_tiles,
 #undef SKINNY_MT
 #undef SKINNY
     TNX_CHECK_LAUNCH("gemm_bf16_skinny");
+    return 0;
+  }
+  if (!sc && force_tiled != 1 && wide_tiles_fit(M, N, K, residual, out_dtype, act) && (uintptr_t)out % 16 == 0 &&
+      (uintptr_t)residual % 16 == 0 && (uintptr_t)bias % 16 == 0) {
+    const int rc = launch_wide(xp, wp, bias, residual, out, out_dtype, act, M, N, K, stream);
+    if (rc) return rc;
+    TNX_CHECK_LAUNCH("gemm_bf16_wide");
     return 0;
   }
   dim3 grid((N + BT_N - 1) / BT_N, (M + BT_M - 1) / BT_M);

@@ -455,11 +455,13 @@ class HipOps:
         tiles = None
         if isinstance(w, PreparedWeight):
             w, tiles = w.tensor, w.tiles
-        if self.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and self._library_product(
-                ctx.num_tokens, w.shape[0], w.shape[1], w, force_tiled):
-            # many rows: the bias joins the library's float32 sums before they are rounded, once, as in the
-            # fused kernel below, so that keys and values are cached with the same rounding whichever path
-            # a token took; the queries are scaled after that
+        many = ctx.num_tokens >= 128 and w.shape[1] % 64 == 0 and w.shape[0] % 8 == 0 and not force_tiled
+        if self.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and (many or self._library_product(
+                ctx.num_tokens, w.shape[0], w.shape[1], w, force_tiled)):
+            # many rows (the vendor library, or our wide-tile kernel where sizes allow): the bias joins the
+            # product's float32 sums before they are rounded, once, as in the fused kernel below, so that keys
+            # and values are cached with the same rounding whichever path a token took; the queries are
+            # scaled after that
             return self.qkv_write(self.linear(h, w, bias), None, num_heads, num_kv_write, head_size, scale, ctx,
                                   view, k_pages, v_pages)
         if self.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
