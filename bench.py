@@ -69,6 +69,8 @@ def main():
                          "queued at once (a continuous-batching workload); prints its own line")
     ap.add_argument("--own-products", action="store_true",
                     help="every matrix product on our own kernels (none goes to the vendor library)")
+    ap.add_argument("--tune-all", action="store_true",
+                    help="time the vendor library's candidates for the many-rows products too")
     ap.add_argument("--big-batch", type=int, default=64, help="the larger batch of `points` (cut to what fits the device at the full context)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -85,6 +87,9 @@ def main():
     if args.own_products:
         from transformers_neuronx_amd.kernels.hip import HipOps
         HipOps.library_rows = 0
+    if args.tune_all:
+        from transformers_neuronx_amd.kernels.hip import HipOps
+        HipOps.library_tune = 2
     raw = dict(MODEL)
     raw.update(OTHER_MODELS.get(args.model, {}))
     layers_full = raw["num_hidden_layers"]

@@ -414,10 +414,15 @@ def run_toy_rotating_model(ops_kind, dtype, device, tol):
     spec = toy_parts.toy_spec_rotating()
     model = DecoderModel(spec)
     tensors = random_tensors(model.param_decls(), spec.init_std, 6, torch.float32)
-    assert "blocks.1.attn.wk.weight" in tensors and tensors["blocks.0.attn.wk.weight"].shape == (32, 96)
+    assert "blocks.2.attn.wk.weight" in tensors and tensors["blocks.0.attn.wk.weight"].shape == (32, 96)
+    assert tensors["blocks.1.attn.down.weight"].shape == (24, 96)
     ops = make_ops(ops_kind, dtype, device)
     model.load(TensorDict(tensors), ops, dtype, device)
     runner = ModelRunner(model, CacheManager(model.cache_needs(), 16, 12, 4, dtype, device), ops, use_graphs=True)
+    # the latent mixer's pages are of its own shape, in the same group (same page numbers) as the attention's
+    shapes = {cid: {k: tuple(v.shape) for k, v in c.pages.items()} for cid, c in runner.cache.caches.items()}
+    assert shapes[1] == {"z": (12, 16, 24)} and shapes[0] == {"k": (12, 1, 16, 32), "v": (12, 1, 32, 16)}
+    assert list(runner.cache.groups) == ["full"]
     requests = _requests(157, [70, 33, 100], 10)
     expected = {rid: toy_parts.toy_rotating_plain_logits(tensors, toks) for rid, toks in requests.items()}
     for steps, place in (schedules.whole(requests), schedules.portions(requests),
@@ -506,3 +511,34 @@ def test_percentiles_of_the_benchmark_report():
     values = [5.0, 1.0, 4.0, 2.0, 3.0]
     assert [percentile(values, q) for q in (0, 50, 90, 95, 99, 100)] == [1.0, 3.0, 5.0, 5.0, 5.0, 5.0]
     assert percentile([7.0], 50) == 7.0 and percentile(list(range(10)), 50) == 5 and percentile(list(range(10)), 96) == 9
+
+
+def test_a_step_planner_of_the_tests_rides_in_the_steps_integers(tiny_folders):
+    """A part that brings a kernel of its own can bring what that kernel launches by: a planner registered
+    from outside adds its int32 arrays to the one buffer of integers a step sends, beside the attention
+    kernels' own plan, and the model runs as before."""
+    import numpy as np
+    from transformers_neuronx_amd.engine import register_step_planner, unregister_step_planner
+
+    def even_runs(run_lens, cached, page_size):
+        chosen = np.nonzero(run_lens % 2 == 0)[0].astype(np.int32)
+        return {"toy_even_runs": chosen, "toy_totals": (run_lens + cached).astype(np.int32)}, {"toy_count": len(chosen)}
+
+    folder, cfg, weights = tiny_folders["A"]
+    toks = _requests(cfg["vocab_size"], [6, 9, 4], 5)
+    want = {rid: plain_opt.forward_logits(weights, cfg, t)[-1] for rid, t in toks.items()}
+    register_step_planner("toy", even_runs)
+    try:
+        runner, _ = _runner(folder, 128)
+        logits = runner.step([StepEntry(rid, t, [len(t) - 1]) for rid, t in toks.items()])
+        ctx = runner._last_ctx
+        assert ctx.plan["toy_even_runs"].tolist() == [0, 2] and ctx.plan["toy_totals"].tolist() == [6, 9, 4]
+        assert ctx.plan_host["toy_count"] == 2
+        assert ctx.decode_runs.numel() == 0 and ctx.tile_run.tolist() == [1, 0, 2]     # the longest run first
+        for i, rid in enumerate(toks):
+            assert float((logits[i] - want[rid]).abs().max()) < 1e-5
+    finally:
+        unregister_step_planner("toy")
+    runner, _ = _runner(folder, 128)
+    runner.step([StepEntry("a", toks["r0"], [0])])
+    assert "toy_even_runs" not in runner._last_ctx.plan

@@ -110,8 +110,8 @@ def test_attention_part_in_two_steps(dtype, heads, kv, hs, bias, window):
     assert (need.kind, need.kv_heads, need.head_size, need.window) == ("paged", kv, hs, window)
     ps, pages = 16, 8
     cache = LayerCache(0, "full", True,
-                       torch.full((pages, kv, ps, hs), float("nan"), device=DEV, dtype=dtype),
-                       torch.full((pages, kv, hs, ps), float("nan"), device=DEV, dtype=dtype))
+                       {"k": torch.full((pages, kv, ps, hs), float("nan"), device=DEV, dtype=dtype),
+                        "v": torch.full((pages, kv, hs, ps), float("nan"), device=DEV, dtype=dtype)})
     n0, n1, other = 37, 9, 21
     h = (torch.randn(n0 + n1, width, device=DEV, generator=g)).to(dtype)
     ho = (torch.randn(other, width, device=DEV, generator=g)).to(dtype)
@@ -188,8 +188,8 @@ def test_block_arrangements(dtype, order):
     ops = _ops(dtype)
     for part, prefix in named:
         part.load(t, prefix, ops, dtype)
-    cache = LayerCache(0, "full", True, torch.zeros(3, heads, ps, hs, device=DEV, dtype=dtype),
-                       torch.zeros(3, heads, hs, ps, device=DEV, dtype=dtype))
+    cache = LayerCache(0, "full", True, {"k": torch.zeros(3, heads, ps, hs, device=DEV, dtype=dtype),
+                                         "v": torch.zeros(3, heads, hs, ps, device=DEV, dtype=dtype)})
     ctx = build_context([StepEntry("a", [0] * n, [])], [0], [0], {"full": np.array([[2, 0]], dtype=np.int32)}, ps, DEV)
     x = torch.randn(n, width, device=DEV, generator=g)
     out = block.forward(Stream(x, ops.cast(x, dtype)), ctx, cache)

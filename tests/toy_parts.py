@@ -306,24 +306,67 @@ class ToyScaleNorm(Norm):
         return (out_f32 if want_f32 else None), ((out_f32 if same else out_cd) if want_compute else None)
 
 
+@register_mixer("toy_latent")
+class ToyLatentMixer(Mixer):
+    """Keeps one small vector per token in pages of its own shape, z_t = h_t W_in^T (a paged cache that is
+    no pair of keys and values), and returns the mean of the vectors so far through W_out: y_t = mean_{j<=t}
+    z_j W_out^T. Torch operations and a loop over requests: a toy."""
+
+    def __init__(self, width: int, latent: int):
+        self.width, self.latent = width, latent
+
+    def cache_need(self):
+        return CacheNeed("paged", page_tensors=(("z", ("page", self.latent)),))
+
+    def param_decls(self, prefix):
+        return [ParamDecl(prefix + "down.weight", (self.latent, self.width)),
+                ParamDecl(prefix + "up.weight", (self.width, self.latent))]
+
+    def load(self, tensors, prefix, ops, dtype):
+        super().load(tensors, prefix, ops, dtype)
+        self.down, self.up = tensors[prefix + "down.weight"], tensors[prefix + "up.weight"]
+
+    def forward(self, h, ctx, cache, residual):
+        z = self.ops.linear(h, self.down, None, out_f32=True)
+        pages = cache.pages["z"]                                  # [pages, page_size, latent]
+        view = ctx.groups[cache.group]
+        table = view.block_table.cpu()
+        ps = view.page_size
+        means = torch.empty_like(z)
+        start = 0
+        for r in range(ctx.num_requests):
+            n, have = int(ctx.run_lens_host[r]), int(ctx.cached_lens_host[r])
+            for i in range(n):                                    # store, token by token
+                pos = have + i
+                pages[int(table[r, pos // ps]), pos % ps] = z[start + i].to(pages.dtype)
+            blocks = [int(b) for b in table[r, :-(-(have + n) // ps)]]
+            so_far = pages[blocks].reshape(-1, self.latent)[:have + n].float()
+            sums = torch.cumsum(so_far, dim=0)[have:]
+            means[start:start + n] = sums / torch.arange(have + 1, have + n + 1, device=z.device)[:, None]
+            start += n
+        return self.ops.linear(means.to(self.dtype), self.up, None, residual=residual, out_f32=True)
+
+
 def toy_spec_rotating(width=96, heads=3, kv_heads=1, inner=72, vocab=157, positions=150, eps=1e-3, base=100.0):
-    """Two layers of attention whose queries and keys are turned by their positions (no encoding at the
-    input), grouped heads, a scale-only norm with its own kernel, names of its own for every tensor."""
+    """Attention whose queries and keys are turned by their positions (no encoding at the input), grouped
+    heads, between two such layers one whose mixer keeps a paged cache of another shape; a scale-only norm
+    with its own kernel, names of its own for every tensor."""
     hs = width // heads
     norm = PartSpec("toy_scale_norm", dict(width=width, eps=eps))
     mixer = PartSpec("attention", dict(width=width, num_heads=heads, head_size=hs, num_kv_heads=kv_heads, bias=False,
                                        names=("wq", "wk", "wv", "wo"), rotation=PartSpec("toy_rotation", dict(base=base))))
     ffn = PartSpec("dense", dict(width=width, inner=inner, activation="gelu", bias=False, up_name="up", down_name="down"))
-    layers = tuple(LayerSpec(prefix=f"blocks.{i}.", block="pre_norm", mixer=mixer, feed_forward=ffn, mixer_norm=norm,
-                             feed_forward_norm=norm, mixer_name="attn.", feed_forward_name="mlp.",
-                             mixer_norm_name="attn_norm", feed_forward_norm_name="mlp_norm") for i in range(2))
+    latent = PartSpec("toy_latent", dict(width=width, latent=24))
+    layers = tuple(LayerSpec(prefix=f"blocks.{i}.", block="pre_norm", mixer=latent if i == 1 else mixer, feed_forward=ffn,
+                             mixer_norm=norm, feed_forward_norm=norm, mixer_name="attn.", feed_forward_name="mlp.",
+                             mixer_norm_name="attn_norm", feed_forward_norm_name="mlp_norm") for i in range(3))
     embedding = PartSpec("token_table", dict(vocab=vocab, embed_width=width, width=width, position=PartSpec("none", {}),
                                              table_name="tokens.weight", projection_name=None, position_name=None))
     head = PartSpec("vocab_projection", dict(vocab=vocab, embed_width=width, width=width, norm=norm,
                                              weight_name="out.weight", tied_to=None, projection_name=None,
                                              norm_name="out_norm"))
     return ModelSpec(hidden_size=width, vocab_size=vocab, max_positions=positions, embedding=embedding, layers=layers,
-                     schedule=ModelSpec.sequential(2), head=head, init_std=0.1)
+                     schedule=ModelSpec.sequential(3), head=head, init_std=0.1)
 
 
 def toy_rotating_plain_logits(w, tokens, width=96, heads=3, kv_heads=1, eps=1e-3, base=100.0, first_position=0):
@@ -344,9 +387,17 @@ def toy_rotating_plain_logits(w, tokens, width=96, heads=3, kv_heads=1, eps=1e-3
         t = t.reshape(n, nh, hs // 2, 2)
         return torch.stack([t[..., 0] * cos - t[..., 1] * sin, t[..., 0] * sin + t[..., 1] * cos], -1).reshape(n, nh * hs)
 
-    for i in range(2):
+    for i in range(3):
         p = f"blocks.{i}."
         h = norm(x, p + "attn_norm")
+        if i == 1:                                  # the layer that keeps a small vector per token and averages them
+            z = plain_opt.linear(h, w[p + "attn.down.weight"])
+            means = torch.cumsum(z, dim=0) / torch.arange(1, n + 1, dtype=torch.float32)[:, None]
+            x = x + plain_opt.linear(means, w[p + "attn.up.weight"])
+            h = norm(x, p + "mlp_norm")
+            x = x + plain_opt.linear(plain_opt.activation(plain_opt.linear(h, w[p + "mlp.up.weight"]), "gelu"),
+                                     w[p + "mlp.down.weight"])
+            continue
         q = turn(plain_opt.linear(h, w[p + "attn.wq.weight"]), heads)
         k = turn(plain_opt.linear(h, w[p + "attn.wk.weight"]), kv_heads)
         v = plain_opt.linear(h, w[p + "attn.wv.weight"])

@@ -2,8 +2,10 @@
 one set of pages per group of layers with the same needs, and slots of
 fixed-size state.
 
-Storage of a paged cache (one pair per cache id, that is per writing call of the
-run order): keys `[pages, kv_heads, page_size, head_size]`, values
+Storage of a paged cache (one set of tensors per cache id, that is per writing
+call of the run order): whatever the mixer's `CacheNeed` names, each tensor with
+the page number in front and the page size where the need says "page". Attention
+keeps keys `[pages, kv_heads, page_size, head_size]` and values
 `[pages, kv_heads, head_size, page_size]` (values are kept transposed inside a
 page: the kernels contract over the tokens of a page). Caches of one group share
 page numbers, so one block table serves all of them. The reference's paged
@@ -30,12 +32,19 @@ class LayerCache:
     cache_id: int
     group: Optional[str]            # name of the page group (None for state-only caches)
     writes: bool = True
-    k_pages: Optional[torch.Tensor] = None
-    v_pages: Optional[torch.Tensor] = None
+    pages: Dict[str, torch.Tensor] = field(default_factory=dict)   # name -> [pages, *shape with the page size in it]
     state: Dict[str, torch.Tensor] = field(default_factory=dict)   # name -> [slots, *shape]
 
+    @property
+    def k_pages(self) -> Optional[torch.Tensor]:
+        return self.pages.get("k")
+
+    @property
+    def v_pages(self) -> Optional[torch.Tensor]:
+        return self.pages.get("v")
+
     def reader(self) -> "LayerCache":
-        return LayerCache(self.cache_id, self.group, False, self.k_pages, self.v_pages, self.state)
+        return LayerCache(self.cache_id, self.group, False, self.pages, self.state)
 
 
 @dataclass
@@ -85,9 +94,9 @@ class CacheManager:
                 g.cache_ids.append(cid)
                 lc = LayerCache(cid, g.name)
                 if allocate:
-                    n = g.pool.num_pages
-                    lc.k_pages = torch.empty(n, need.kv_heads, page_size, need.head_size, dtype=dtype, device=device)
-                    lc.v_pages = torch.empty(n, need.kv_heads, need.head_size, page_size, dtype=dtype, device=device)
+                    for name, shape in need.tensors_of_a_page():
+                        dims = [page_size if d == "page" else d for d in shape]
+                        lc.pages[name] = torch.empty(g.pool.num_pages, *dims, dtype=dtype, device=device)
                 self.caches[cid] = lc
             elif need.kind == "state":
                 lc = LayerCache(cid, None)
@@ -104,8 +113,16 @@ class CacheManager:
     @staticmethod
     def bytes_per_page(needs: Dict[int, CacheNeed], page_size: int, dtype: torch.dtype) -> int:
         item = torch.empty(0, dtype=dtype).element_size()
-        return sum(2 * n.kv_heads * n.head_size * page_size * item
-                   for n in needs.values() if n is not None and n.kind == "paged")
+        total = 0
+        for n in needs.values():
+            if n is None or n.kind != "paged":
+                continue
+            for _, shape in n.tensors_of_a_page():
+                count = 1
+                for d in shape:
+                    count *= page_size if d == "page" else d
+                total += count * item
+        return total
 
     # ---------------------------------------------------------------- requests
 

@@ -817,7 +817,7 @@ struct LibraryCall {              // the operands of one product, as the library
   size_t workspace_bytes;
   hipStream_t stream;
 };
-constexpr int MAX_DEVICES = 64, CANDIDATES = 6, TUNED_ROWS = 256;
+constexpr int MAX_DEVICES = 64, CANDIDATES = 16, FEW_CANDIDATES = 6, TUNED_ROWS = 256;
 LibraryApi library_api;
 hipblasLtHandle_t library_handles[MAX_DEVICES] = {};
 std::map<std::tuple<int, int, int, int, int>, LibraryPlan> library_plans;     // device, M, N, K, what follows
@@ -887,7 +887,7 @@ float library_time(hipblasLtHandle_t handle, const LibraryPlan& p, const hipblas
 // The plan of one product: descriptors and an algorithm. Row-major out[M][N] = x[M][K] w[N][K]^T is, in the
 // library's column-major terms, D[N x M] = op_T(w as K x N) (x as K x M).
 LibraryPlan make_plan(hipblasLtHandle_t handle, int M, int N, int K, const float* bias, bool relu, bool out_f32,
-                      const LibraryCall& call, void* flush, size_t flush_bytes) {
+                      const LibraryCall& call, void* flush, size_t flush_bytes, int candidates) {
   LibraryPlan p;
   const LibraryApi& a = library_api;
   if (a.desc_create(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return p;
@@ -916,11 +916,11 @@ LibraryPlan make_plan(hipblasLtHandle_t handle, int M, int N, int K, const float
   int count = 0;
   const size_t room = call.workspace_bytes;
   if (a.pref_set(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &room, sizeof(room)) != HIPBLAS_STATUS_SUCCESS ||
-      a.heuristic(handle, p.desc, p.w, p.x, p.c, p.c, pref, CANDIDATES, found, &count) != HIPBLAS_STATUS_SUCCESS)
+      a.heuristic(handle, p.desc, p.w, p.x, p.c, p.c, pref, candidates, found, &count) != HIPBLAS_STATUS_SUCCESS)
     count = 0;
   a.pref_destroy(pref);
   int fits[CANDIDATES], n_fit = 0;
-  for (int i = 0; i < count && i < CANDIDATES; ++i)
+  for (int i = 0; i < count && i < candidates; ++i)
     if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= room) fits[n_fit++] = i;
   if (n_fit == 0) return p;
   int pick = fits[0];
@@ -971,7 +971,8 @@ extern "C" int tnx_gemm_library(const void* x, const void* w, const float* bias,
   const auto key = std::make_tuple(device, M, N, K, what);
   auto it = library_plans.find(key);
   if (it == library_plans.end()) {
-    bool timed = tune && M <= TUNED_ROWS;
+    // `tune` 1: up to TUNED_ROWS rows, the first few of the ranking; 2: every product, more of the ranking
+    bool timed = tune >= 2 || (tune && M <= TUNED_ROWS);
     if (timed) {
       // nothing is timed inside a recording: the first choice of the library's ranking stands in there
       hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
@@ -979,7 +980,8 @@ extern "C" int tnx_gemm_library(const void* x, const void* w, const float* bias,
     }
     if (timed && (flush == nullptr || flush_bytes == 0)) return 3;
     it = library_plans.emplace(key, make_plan(library_handles[device], M, N, K, bias, act == TNX_ACT_RELU,
-                                              out_dtype == TNX_F32, call, timed ? flush : nullptr, flush_bytes)).first;
+                                              out_dtype == TNX_F32, call, timed ? flush : nullptr, flush_bytes,
+                                              tune >= 2 ? CANDIDATES : FEW_CANDIDATES)).first;
   }
   const LibraryPlan& p = it->second;
   if (!p.usable || p.workspace > workspace_bytes) return 2;

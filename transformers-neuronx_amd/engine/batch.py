@@ -15,6 +15,43 @@ import torch
 
 QUERY_TILE = 128    # queries of one run that one block of the prompt attention kernel takes
 
+# What a kernel wants to know about a step beyond its tokens, as int32 arrays that travel in the step's one
+# buffer of integers: a planner is `fn(run_lens, cached, page_size) -> ({name: int32 array}, {name: host value})`,
+# registered under a name; the arrays of all planners are laid out behind the step's own pieces and reach the
+# kernels as `ctx.plan[name]`, the host values as `ctx.plan_host[name]`. The attention kernels' planner below
+# is registered like any other; a part that brings a kernel of its own can bring a planner with it.
+_PLANNERS: Dict[str, object] = {}
+
+
+def register_step_planner(name: str, fn) -> None:
+    _PLANNERS[name] = fn
+
+
+def unregister_step_planner(name: str) -> None:
+    _PLANNERS.pop(name, None)
+
+
+def attention_plan(run_lens: np.ndarray, cached: np.ndarray, page_size: int):
+    """What the attention kernels launch by: the runs of one token (each attends with one query) and the
+    most keys one of them reads; for every tile of QUERY_TILE queries of the longer runs its run and its first
+    query, those that see the most keys first (a kernel that takes them in this order starts its longest
+    blocks first)."""
+    single = run_lens == 1
+    decode_runs = np.nonzero(single)[0].astype(np.int32)
+    longest = int((cached[single] + 1).max()) if single.any() else 0
+    tiles = []
+    for i in np.nonzero(run_lens > 1)[0]:
+        for q0 in range(0, int(run_lens[i]), QUERY_TILE):
+            tiles.append((-(int(cached[i]) + min(q0 + QUERY_TILE, int(run_lens[i]))), int(i), q0))
+    tiles.sort()
+    arrays = {"decode_runs": decode_runs, "tile_run": np.array([t[1] for t in tiles], dtype=np.int32),
+              "tile_start": np.array([t[2] for t in tiles], dtype=np.int32),
+              "longest_decode": np.array([longest], dtype=np.int32)}
+    return arrays, {"longest_decode": longest}
+
+
+register_step_planner("attention", attention_plan)
+
 
 @dataclass
 class StepEntry:
@@ -46,16 +83,13 @@ class StepContext:
     slots: torch.Tensor             # int32 [R], state slot of each request
     logits_rows: torch.Tensor       # int32 [M], tokens whose logits are wanted
     groups: Dict[str, GroupView]
-    decode_runs: torch.Tensor = None     # int32, the runs of one token (each attends with one query)
-    tile_run: torch.Tensor = None        # int32, for every tile of QUERY_TILE queries of the longer runs: its run
-    tile_start: torch.Tensor = None      # int32, and its first query within the run
-    query_tile: int = QUERY_TILE         # queries of a tile
-    longest_decode: torch.Tensor = None  # int32 [1], the most keys a one-token run of this step reads
+    plan: Dict[str, torch.Tensor] = field(default_factory=dict)   # int32 arrays of the registered step planners
+    plan_host: Dict[str, object] = field(default_factory=dict)    # and what they say on the host
+    query_tile: int = QUERY_TILE         # queries of a tile of the attention plan
     # int32 [slots]: the token last chosen for the request in each slot, on the device. A token id -1 - s
     # in `token_ids` stands for `kept_tokens[s]`: a step can be started before the host has read the
     # tokens that the step before it chose.
     kept_tokens: Optional[torch.Tensor] = None
-    longest_decode_host: int = 0
     # When a step is recorded for replay, nothing in its launches may depend on the lengths of this
     # particular step: `length_bound` then stands in for them where a launch is sized.
     length_bound: Optional[int] = None
@@ -64,6 +98,27 @@ class StepContext:
     cached_lens_host: np.ndarray = None
     slots_host: np.ndarray = None
     plans: Dict = field(default_factory=dict)    # launch plans the kernel backend keeps per step
+
+    # the attention kernels' plan under the names they use
+    @property
+    def decode_runs(self) -> torch.Tensor:
+        return self.plan["decode_runs"]
+
+    @property
+    def tile_run(self) -> torch.Tensor:
+        return self.plan["tile_run"]
+
+    @property
+    def tile_start(self) -> torch.Tensor:
+        return self.plan["tile_start"]
+
+    @property
+    def longest_decode(self) -> torch.Tensor:
+        return self.plan["longest_decode"]
+
+    @property
+    def longest_decode_host(self) -> int:
+        return self.plan_host["longest_decode"]
 
     @property
     def max_run(self) -> int:
@@ -88,7 +143,8 @@ class PackedStep:
     run_lens: np.ndarray
     cached: np.ndarray
     slots: np.ndarray
-    longest_decode: int
+    plan_names: List[str]
+    plan_host: Dict[str, object]
 
     def layout(self):
         """What two steps must share for one to reuse the other's device buffer and views."""
@@ -96,7 +152,7 @@ class PackedStep:
                 tuple(self.group_names), tuple(sorted(self.widths.items())), self.page_size)
 
 
-_FIXED_PIECES = 11   # pieces before the per-group ones, see pack_step
+_FIXED_PIECES = 7    # the step's own pieces, before the planners' and the per-group ones, see pack_step
 
 
 def pack_step(entries: List[StepEntry], cached: List[int], slots: List[int], tables: Dict[str, np.ndarray],
@@ -116,22 +172,17 @@ def pack_step(entries: List[StepEntry], cached: List[int], slots: List[int], tab
                 raise ValueError(f"request {e.req!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
             rows.append(run_start[i] + w)
     rows = np.array(rows, dtype=np.int32)
-    single = run_lens == 1
-    decode_runs = np.nonzero(single)[0].astype(np.int32)
-    longest = int((cached_np[single] + 1).max()) if single.any() else 0
-    # Tiles of the longer runs, those that see the most keys first: a kernel that takes them in this order
-    # starts its longest blocks first.
-    tiles = []
-    for i in np.nonzero(run_lens > 1)[0]:
-        for q0 in range(0, int(run_lens[i]), QUERY_TILE):
-            tiles.append((-(int(cached_np[i]) + min(q0 + QUERY_TILE, int(run_lens[i]))), int(i), q0))
-    tiles.sort()
-    tile_run = [t[1] for t in tiles]
-    tile_start = [t[2] for t in tiles]
-    pieces = [token_ids, positions, token_request, run_start, cached_np, np.array(slots, dtype=np.int32), rows,
-              decode_runs, np.array(tile_run, dtype=np.int32), np.array(tile_start, dtype=np.int32),
-              np.array([longest], dtype=np.int32)]
+    pieces = [token_ids, positions, token_request, run_start, cached_np, np.array(slots, dtype=np.int32), rows]
     assert len(pieces) == _FIXED_PIECES
+    plan_names, plan_host = [], {}
+    for planner in _PLANNERS.values():
+        arrays, host = planner(run_lens, cached_np, page_size)
+        for name, array in arrays.items():
+            if name in plan_names:
+                raise ValueError(f"two step planners name an array {name!r}")
+            plan_names.append(name)
+            pieces.append(np.ascontiguousarray(array, dtype=np.int32).reshape(-1))
+        plan_host.update(host)
     names = list(tables)
     pieces += [tables[g].reshape(-1) for g in names]
     for g in names:
@@ -150,7 +201,7 @@ def pack_step(entries: List[StepEntry], cached: List[int], slots: List[int], tab
         flat[off:off + p.size] = p
     return PackedStep(flat, offsets, [p.size for p in pieces], t, r, names,
                       {g: tables[g].shape[1] for g in names}, page_size, run_lens, cached_np,
-                      np.array(slots, dtype=np.int32), longest)
+                      np.array(slots, dtype=np.int32), plan_names, plan_host)
 
 
 def context_from(packed: PackedStep, dev: torch.Tensor) -> StepContext:
@@ -158,14 +209,15 @@ def context_from(packed: PackedStep, dev: torch.Tensor) -> StepContext:
     views = [dev[off:off + n] for off, n in zip(packed.offsets, packed.sizes)]
     groups = {}
     n = len(packed.group_names)
+    first = _FIXED_PIECES + len(packed.plan_names)        # the per-group pieces follow the planners'
     for i, g in enumerate(packed.group_names):
         width = packed.widths[g]
-        groups[g] = GroupView(views[_FIXED_PIECES + i].view(packed.num_requests, width), packed.page_size, width,
-                              token_page=views[_FIXED_PIECES + n + i], token_offset=views[_FIXED_PIECES + 2 * n])
+        groups[g] = GroupView(views[first + i].view(packed.num_requests, width), packed.page_size, width,
+                              token_page=views[first + n + i], token_offset=views[first + 2 * n])
+    plan = {name: views[_FIXED_PIECES + i] for i, name in enumerate(packed.plan_names)}
     return StepContext(packed.num_tokens, packed.num_requests, views[0], views[1], views[2], views[3], views[4],
-                       views[5], views[6], groups, decode_runs=views[7], tile_run=views[8], tile_start=views[9],
-                       longest_decode=views[10], run_lens_host=packed.run_lens, cached_lens_host=packed.cached,
-                       slots_host=packed.slots, longest_decode_host=packed.longest_decode)
+                       views[5], views[6], groups, plan=plan, plan_host=dict(packed.plan_host),
+                       run_lens_host=packed.run_lens, cached_lens_host=packed.cached, slots_host=packed.slots)
 
 
 def build_context(entries: List[StepEntry], cached: List[int], slots: List[int],

@@ -373,7 +373,7 @@ class HipOps:
         return out
 
     library_direct = True   # many-rows products as calls of the vendor library itself, with what follows them
-    library_tune = True     # and its algorithms timed once for products of few rows
+    library_tune = 1        # and its algorithms timed once: 1, for products of few rows; 2, for every product
     _workspaces: Dict[str, torch.Tensor] = {}
 
     def _library_call(self, xa, w, bias, residual, out, act, m, n, k) -> bool:
@@ -397,7 +397,7 @@ class HipOps:
                 flush = torch.empty(256 << 20, dtype=torch.uint8, device=xa.device)
             except torch.OutOfMemoryError:
                 flush = None
-            rc = call(flush, flush is not None)
+            rc = call(flush, int(self.library_tune) if flush is not None else 0)
         if rc == 1:
             raise RuntimeError(f"tnx_gemm_library: {lib.tnx_last_error().decode()}")
         return rc == 0

@@ -16,11 +16,14 @@ from .spec import ParamDecl, PartSpec
 class CacheNeed:
     """What a mixer keeps per request between steps.
 
-    kind 'paged': grows with the tokens. `shapes` names per-token tensors as
-         {name: (layout, dims...)}; `window` (tokens) lets pages be given back
-         once every later query is past them, None keeps them all.
-    kind 'state': fixed size per request. `shapes` is {name: dims}; a slot is
-         zeroed when a request gets it.
+    kind 'paged': grows with the tokens, in pages. What a page holds is a set of named tensors,
+         `page_tensors` = ((name, shape), ...), where the place of the page's tokens in a shape is the
+         string "page" (the manager puts its page size there and the page number in front). Left empty,
+         it is what attention keeps: keys `(kv_heads, "page", head_size)` and values
+         `(kv_heads, head_size, "page")`. `window` (tokens) lets pages be given back once every later
+         query is past them, None keeps them all.
+    kind 'state': fixed size per request. `state_shapes` is ((name, dims), ...); a slot is zeroed when a
+         request gets it.
     """
     kind: str
     kv_heads: int = 0
@@ -28,10 +31,16 @@ class CacheNeed:
     window: Optional[int] = None
     state_shapes: Tuple[Tuple[str, Tuple[int, ...]], ...] = ()
     state_dtype: str = "float32"
+    page_tensors: Tuple[Tuple[str, Tuple], ...] = ()
 
     def group_key(self):
         """Layers with equal keys share a page table."""
         return (self.kind, self.window)
+
+    def tensors_of_a_page(self) -> Tuple[Tuple[str, Tuple], ...]:
+        if self.page_tensors:
+            return self.page_tensors
+        return (("k", (self.kv_heads, "page", self.head_size)), ("v", (self.kv_heads, self.head_size, "page")))
 
 
 class Part:
