@@ -546,15 +546,20 @@ class HipOps:
                        _stream())
         return out
 
+    # What the choice between one and two sets of waves a block rests on: the time of one 64-key step of a
+    # block, in microseconds, measured on an MI355X at head size 128 (a block alone on its compute unit, two
+    # blocks that share one, a block of two sets, and what a second round of blocks adds). Only the ratios
+    # matter; another chip or head size changes which of two close estimates wins, not the results.
+    prefill_step_cost = dict(alone=2.6, shared=3.9, two_sets=4.1, second_round=7.0)
+
     def _prefill_sets(self, ctx, num_heads, window) -> int:
         """How the staged prompt kernel runs this step: 0, two sets of four waves a block that halve a tile's
         keys between them, or 2, one set. One set lets two blocks share a compute unit and overlap each other's
         waits; two sets halve the time of the tile that sees the most keys, which the launch waits for when the
-        blocks are few or uneven. The choice compares the two estimates below, in the time one 64-key step
-        of a block takes (measured at head size 128: 2.6 us for a block alone on its unit, 3.9 us for two that
-        share it, 4.1 us for a block of two sets, 7 us for a second round of blocks)."""
+        blocks are few or uneven. The choice compares two estimates made from `prefill_step_cost`."""
         plan = ctx.plans.get(("prefill_sets", window))
         if plan is None:
+            cost = self.prefill_step_cost
             lens, cached = ctx.run_lens_host, ctx.cached_lens_host
             steps = []
             for i in np.nonzero(lens > 1)[0]:
@@ -565,10 +570,10 @@ class HipOps:
             steps = np.array(steps)
             halves = (steps + 1) // 2
             units = self.compute_units
-            one = max(steps.max() * 2.6, steps.sum() * num_heads / units * 1.95)
-            two = max(halves.max() * 4.1, halves.sum() * num_heads / units * 4.1)
+            one = max(steps.max() * cost["alone"], steps.sum() * num_heads / units * cost["shared"] / 2)
+            two = max(halves.max() * cost["two_sets"], halves.sum() * num_heads / units * cost["two_sets"])
             if len(steps) * num_heads > units:
-                two += 7.0
+                two += cost["second_round"]
             plan = ctx.plans[("prefill_sets", window)] = 0 if two < one else 2
         return plan
 
