@@ -699,7 +699,13 @@ static int gemm_bf16_dispatch(const void* x, const void* w, const void* w_tiles,
     case 3: SKINNY(3, WV, 1); break;         \
     default: SKINNY(4, WV, 1); break;        \
   }
-    if (two_tiles && M <= 16) {
+    if (force_tiled == 3 && M <= 16) {
+      SKINNY(1, 4, 3);
+    } else if (force_tiled == 5 && M <= 16) {
+      SKINNY(1, 8, 2);
+    } else if (force_tiled == 6 && M <= 16) {
+      SKINNY(1, 8, 3);
+    } else if (two_tiles && M <= 16) {
       SKINNY(1, 4, 2);
     } else if (two_tiles && M <= 32) {
       SKINNY(2, 4, 2);
