@@ -458,16 +458,28 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict_
 
 // The same computation with the keys and values of a tile staged through LDS, once for the four waves of a
 // block, and the next tile's global loads in flight while the current one is computed (two LDS buffers, one
-// barrier a tile). Page sizes that are powers of two. K is staged as [key][head_size + 8] and V^T as
-// [head_size][64 + 8] (the padding spreads the rows over the LDS banks).
+// barrier a tile). Page sizes that are powers of two. K is staged as [key][head_size + pad] and V^T as
+// [head_size][64 + pad].
 // FAST is the case of a head size of exactly 16 * NDB and pages of 64 keys or more: a tile then lies within
 // one page, whose number is one scalar lookup, every thread's place within the tile is fixed, and no part of
 // the inner loops depends on a size known only at run time.
+// Where the rows lie in LDS is chosen by measurement of the fragment reads (16 rows by 4 chunks of 16 bytes
+// a wave): rows of 16 (2 n + 1) bytes, the usual padding, take twice the time of rows of 32 (2 n + 1) bytes,
+// which are read at the full rate, as are unpadded 256-byte rows whose chunk c lies at c ^ (row's index among
+// the 16 that are read together). The 8-byte reads of the general case's values want 16 (2 n + 1).
 // With GROUPS = 2 a block has two such sets of four waves for the same 128 queries: the first takes the
 // first half of the key tiles and the second the rest, each through LDS buffers of its own, and their
 // partial results (maximum, sum, weighted values, float32) meet in LDS at the end. The tile of the last
 // queries of a long prompt, which sees the most keys, then takes half as long, and it is that tile which the
 // launch waits for.
+template <int NDB, bool FAST>
+struct PrefillTileLayout {
+  static constexpr int DMAX = 16 * NDB;
+  static constexpr bool SWIZZLED = FAST && NDB == 8;            // 256-byte key rows, chunks exchanged
+  static constexpr int KSTR = SWIZZLED ? DMAX : DMAX + 16;      // elements per staged key row
+  static constexpr int VSTR = FAST ? 64 + 16 : 64 + 8;          // per staged value row (one element, 64 keys)
+  static constexpr int KBUF = 64 * KSTR, VBUF = DMAX * VSTR;
+};
 template <int NDB, bool FAST, int GROUPS>
 __global__ void __launch_bounds__(256 * GROUPS, (NDB <= 8 && GROUPS == 1 ? 2 : 1))
 attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
@@ -478,9 +490,9 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
                              int head_size, int window) {
   constexpr int NKS = (NDB + 1) / 2;
   constexpr int DMAX = 16 * NDB;
-  constexpr int KSTR = DMAX + 8;            // elements per staged key row
-  constexpr int VSTR = 64 + 8;              // elements per staged value row (one head-size element, 64 keys)
-  constexpr int KBUF = 64 * KSTR, VBUF = DMAX * VSTR;
+  using Layout = PrefillTileLayout<NDB, FAST>;
+  constexpr bool SWZ = Layout::SWIZZLED;
+  constexpr int KSTR = Layout::KSTR, VSTR = Layout::VSTR, KBUF = Layout::KBUF, VBUF = Layout::VBUF;
   constexpr int KCH = (64 * DMAX / 8 + 255) / 256;   // 16-byte chunks a thread stages per tile, keys
   constexpr int VCH = (DMAX * 8 + 255) / 256;        // and values
   extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
@@ -606,7 +618,12 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
     bf16_t* vd = vs_buf + buf * VBUF;
 #pragma unroll
     for (int j = 0; j < KCH; ++j)
-      if (tid + 256 * j < k_chunks) *(bf16x8*)(kd + kc_key[j] * KSTR + kc_dc[j] * 8) = kreg[j];
+      if (tid + 256 * j < k_chunks) {
+        // swizzled: chunk c of key row k lies at c ^ (4 ((k / 8) % 4) + k % 4), the row's index among the 16
+        // that a fragment read takes together (see `read_keys`)
+        const int dc = SWZ ? (kc_dc[j] ^ ((((kc_key[j] >> 3) & 3) << 2) | (kc_key[j] & 3))) : kc_dc[j];
+        *(bf16x8*)(kd + kc_key[j] * KSTR + dc * 8) = kreg[j];
+      }
 #pragma unroll
     for (int j = 0; j < VCH; ++j) {
       if (tid + 256 * j < v_chunks) {
@@ -652,11 +669,16 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
     constexpr int KA = NDB <= 8 ? 2 : 1;
     f32x4 s[4][2];
     bf16x8 kf[KA][NKS];
+    // FAST: row r of key block kb is key 32 (kb / 2) + 8 (r / 4) + 4 (kb % 2) + r % 4 of the tile, so that the
+    // probabilities a lane holds are those of 8 consecutive keys and the values are read 16 bytes a lane;
+    // otherwise key 16 kb + r, the values being read in two halves in the accumulators' order
     auto read_keys = [&](int kb, bf16x8* dst) {
-      const bf16_t* krow = kd + (16 * kb + r) * KSTR + 8 * g;
+      const int row = FAST ? 32 * (kb >> 1) + 8 * (r >> 2) + 4 * (kb & 1) + (r & 3) : 16 * kb + r;
+      const bf16_t* krow = kd + row * KSTR;
+      const int flip = SWZ ? r : 0;
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks)
-        dst[ks] = (32 * ks + 8 * g < head_size) ? *(const bf16x8*)(krow + 32 * ks) : zero8;
+        dst[ks] = (32 * ks + 8 * g < head_size) ? *(const bf16x8*)(krow + ((4 * ks + g) ^ flip) * 8) : zero8;
     };
     if (KA == 2) read_keys(0, kf[0]);
 #pragma unroll
@@ -686,7 +708,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
         for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const int key = tile0 + 16 * kb + 4 * g + i;
+            const int key = FAST ? tile0 + 32 * (kb >> 1) + 8 * g + 4 * (kb & 1) + i : tile0 + 16 * kb + 4 * g + i;
             const bool ok = key <= qpos[qb] && (window <= 0 || key > qpos[qb] - window);
             if (!ok) s[kb][qb][i] = -INFINITY;
           }
@@ -733,6 +755,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
         for (int j = 0; j < 8; ++j) pb[qb][j] = (bf16_t)s[2 * t + (j >> 2)][qb][j & 3];
       // the values of 16 head-size elements are read while the products of the 16 before them run
       auto read_values = [&](int db) {
+        if (FAST) return *(const bf16x8*)(vd + (16 * db + r) * VSTR + 32 * t + 8 * g);
         const bf16_t* vrow = vd + (16 * db + r) * VSTR + 32 * t + 4 * g;
         const bf16x4 lo4 = *(const bf16x4*)(vrow);
         const bf16x4 hi4 = *(const bf16x4*)(vrow + 16);
@@ -820,7 +843,9 @@ static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, co
                               const int* tile_q0, bf16_t* out, int num_heads, int num_kv, int head_size,
                               int window) {
   constexpr int DMAX = 16 * NDB;
-  constexpr size_t bytes = GROUPS * 2 * (size_t)(64 * (DMAX + 8) + DMAX * (64 + 8)) * sizeof(bf16_t);
+  using Layout = PrefillTileLayout<NDB, FAST>;
+  constexpr size_t bytes = GROUPS * 2 * (size_t)(Layout::KBUF + Layout::VBUF) * sizeof(bf16_t);
+  static_assert(bytes <= 160 * 1024, "the staging buffers must fit the 160 KB of LDS");
   static_assert(GROUPS == 1 || bytes >= (4 * NDB * 2 * 4 * 64 + 4 * 2 * 2 * 64) * sizeof(float),
                 "the partial results of the second set of waves must fit the staging buffers");
   static bool configured = false;
