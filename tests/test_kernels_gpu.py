@@ -265,6 +265,39 @@ def test_attention_finds_a_far_key():
                                torch.full_like(out_in, 5.0).float(), rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("sets", [2, 3])
+@pytest.mark.parametrize("hs", [64, 128])
+def test_prompt_attention_when_the_maximum_jumps(sets, hs):
+    """The pipelined prompt kernel moves a query's reference maximum only when a score exceeds it by more than
+    2^8: a key that stands out by less leaves probabilities above one in play, a key that stands out by much
+    more makes all sums so far shrink. Both in the middle of a long prompt, against the torch rendition."""
+    dtype = torch.bfloat16
+    hip, ref = _ops(dtype)
+    hip.prefill_direct = sets
+    heads, ps, n = 2, 64, 600
+    num_pages = -(-n // ps) + 2
+    ctx = _make_step([n], [0], ps, num_pages, seed=21)
+    view = ctx.groups["full"]
+    g = torch.Generator(device=DEV).manual_seed(33)
+    kp = (torch.randn(num_pages, heads, ps, hs, device=DEV, generator=g) * 0.05).to(dtype)
+    vp = (torch.randn(num_pages, heads, hs, ps, device=DEV, generator=g) * 0.1).to(dtype)
+    direction = torch.randn(hs, device=DEV, generator=g)
+    direction /= direction.norm()
+    # every query has a component of 2 along `direction`; key 200 has 2 along it (score + 4: e^4, no rescale),
+    # key 400 has 10 (score + 20), key 401 has 9.5 (one below the new maximum)
+    q = (torch.randn(n, heads, hs, device=DEV, generator=g) * 0.3 + 2 * direction).reshape(n, heads * hs).to(dtype)
+    for key, size, value in ((200, 2.0, 1.0), (400, 10.0, -2.0), (401, 9.5, 3.0)):
+        page = int(view.block_table[0, key // ps])
+        kp[page, :, key % ps, :] = (direction * size).to(dtype)
+        vp[page, :, :, key % ps] = value
+    got = hip.attention(q, heads, heads, hs, ctx, view, kp, vp, None)
+    want = ref.attention(q, heads, heads, hs, ctx, view, kp, vp, None)
+    torch.testing.assert_close(got.float(), want.float(), rtol=2e-2, atol=2e-2)
+    # queries before key 200 see none of the three, those from 400 on are ruled by keys 400 and 401
+    assert got[:200].float().abs().max() < 0.5
+    assert (got[450:].float().mean() - (-2 * 0.731 + 3 * 0.269)).abs() < 0.1      # weights e^0 : e^-1
+
+
 @pytest.mark.parametrize("mode", ["staged", "direct", "plain"])
 def test_windowed_attention_over_pages_given_back(mode):
     """A windowed group gives back the pages its queries have passed: their table entries are -1, and the
@@ -395,6 +428,11 @@ FAST_CASES = [
     (3, 3, 32, 16, [1, 1, 2], [0, 1, 0]),
     (2, 2, 16, 64, [1, 260], [900, 3]),
     (2, 2, 96, 16, [150, 33], [10, 0]),
+    # long prompts on pages of 64 keys or more at head sizes 64 and 128: the pipelined prompt kernel, whose
+    # waves take several whole tiles before the one the positions mask
+    (4, 2, 128, 64, [700, 130, 1], [0, 333, 50]),
+    (6, 2, 64, 128, [513, 64], [1000, 17]),
+    (2, 2, 128, 256, [1000], [37]),
 ]
 
 
@@ -418,7 +456,9 @@ def test_bfloat16_attention_kernels_agree(case, window):
     direct.prefill_direct = True                  # the prompt kernel that reads the pages without staging
     o_direct = direct.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)
     torch.testing.assert_close(o_direct.float(), o_plain.float(), rtol=2e-2, atol=2e-2)
-    for sets in (2, 3):                           # the staged prompt kernel with one set of waves a block, and two
+    # the prompt kernels that stage tiles in LDS with one set of waves a block and with two: 2 and 3 (the
+    # pipelined kernel where it applies), 7 and 6 (never the pipelined one)
+    for sets in (2, 3, 6, 7):
         forced = HipOps(torch.bfloat16, DEV)
         forced.prefill_direct = sets
         o_forced = forced.attention(q, heads, kv, hs, ctx, ctx.groups["full"], kp, vp, window)

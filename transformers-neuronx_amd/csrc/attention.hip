@@ -864,6 +864,521 @@ static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, co
   return 0;
 }
 
+
+// The staged computation once more for the FAST case (see above) without a window, arranged so that the
+// matrix unit and the vector unit work at the same time within a wave: the scores of tile i + 1 are multiplied
+// while the softmax of tile i is computed (the two are independent, and a wave issues vector instructions
+// while its matrix instruction runs; measured, a matrix instruction costs a wave the time of two vector
+// instructions to issue and the unit that of four to run, so two vector instructions to a product keep both
+// busy). The keys therefore run one tile ahead of the values in LDS. What keeps the vector unit's share small:
+//  - the sums so far are rescaled only when some query's maximum has moved far (see `softmax_maximum`);
+//  - the sum of a query's probabilities comes from the matrix unit (a block of ones beside the values);
+//  - tiles go from the pages to LDS without passing through registers (`load_to_lds`: a wave instruction
+//    fills 1 KB of LDS in lane order, so the layout's exchange of chunks is applied to the global addresses),
+//    one load at a time between the products: issued together they held every wave of the block at the
+//    memory pipeline's queue.
+// Rows lie unpadded in LDS, chunk c of key row k at c ^ (k's index among the 16 rows read together) and chunk
+// c of value row d at c ^ (d % 8), which the fragment reads take without bank conflicts. What a load brings
+// of keys beyond the request is zeroed in LDS by the lane that asked for it (values only: their probabilities
+// are zero, and zero times a stale NaN is not). Measured at 32 heads of size 128 and a prompt of 2,048: 54.6 us
+// against 64.3 for the kernel above (per 64-key step of a block: 0.97 us is what the 136 matrix instructions of
+// its two waves a SIMD take, 1.8 us is what the step takes; LDS reads and the tile loads account for most of
+// the rest).
+template <int NDB, int GROUPS>
+__global__ void __launch_bounds__(256 * GROUPS, GROUPS == 1 ? 2 : 1)
+attention_prefill_pipelined_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
+                                   const bf16_t* __restrict__ v_pages, const int* __restrict__ run_start,
+                                   const int* __restrict__ cached_lens, const int* __restrict__ table,
+                                   int table_width, int page_shift, int num_pages,
+                                   const int* __restrict__ tile_run, const int* __restrict__ tile_q0,
+                                   bf16_t* __restrict__ out, int num_heads, int num_kv) {
+  static_assert(NDB == 4 || NDB == 8, "head sizes 64 and 128");
+  constexpr int NKS = NDB / 2, DH = 16 * NDB, CPR = 2 * NDB;   // CPR: 16-byte chunks of a key row
+  constexpr int TILE_BYTES = 64 * DH * 2;                       // 64 keys, and as many values
+  constexpr int NLD = TILE_BYTES / 4096;                        // 1 KB loads of a wave for a tile
+  extern __shared__ __attribute__((aligned(16))) char pipelined_smem[];
+  const int grp = GROUPS == 1 ? 0 : __builtin_amdgcn_readfirstlane(threadIdx.x >> 8);
+  char* kbuf = pipelined_smem + grp * 4 * TILE_BYTES;           // [2][TILE_BYTES]
+  char* vbuf = kbuf + 2 * TILE_BYTES;                           // [2][TILE_BYTES]
+  const unsigned kbuf_lds = (unsigned)(size_t)(__attribute__((address_space(3))) char*)kbuf;
+  const unsigned vbuf_lds = kbuf_lds + 2 * TILE_BYTES;
+  const int tid = threadIdx.x & 255, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, g = lane >> 4;
+  const int tile = blockIdx.x / num_heads, h = blockIdx.x % num_heads;
+  const int run = tile_run[tile];
+  const int kvh = h / (num_heads / num_kv);
+  const int t0 = run_start[run], qlen = run_start[run + 1] - t0, cached = cached_lens[run];
+  const int q0 = tile_q0[tile];
+  const int qw0 = q0 + 32 * wave;
+  const bool wave_on = qw0 < qlen;
+  const int nq = num_heads * DH;
+  const int* tab = table + (size_t)run * table_width;
+  const int total = cached + qlen;
+  const int page_size = 1 << page_shift, pmask = page_size - 1;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const size_t head_stride = (size_t)page_size * DH;
+
+  bf16x8 qf[2][NKS];
+  int qpos[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int qi = qw0 + 16 * qb + r;
+    qpos[qb] = cached + qi;
+#pragma unroll
+    for (int s = 0; s < NKS; ++s)
+      qf[qb][s] = qi < qlen ? *(const bf16x8*)(q + (size_t)(t0 + qi) * nq + h * DH + 32 * s + 8 * g) : zero8;
+  }
+  const int blk_last = cached + min(q0 + PREFILL_Q_TILE - 1, qlen - 1);
+  const int last_q = cached + min(qw0 + 31, qlen - 1);
+  const int first_q = cached + qw0;
+
+  // What each lane asks for: place p = (4 j + wave) * 64 + lane of a tile, in chunks. The offsets of the NLD
+  // loads differ by a constant and, for the keys, by which two bits the chunk is exchanged with; they are made
+  // from one register each when they are needed (and hidden from the compiler, which would keep them all).
+  //   keys: row (4 j + wave) (64 / CPR) + lane / CPR, stored chunk lane % CPR -> chunk (lane % CPR) ^ swizzle(row)
+  //   values: row 32 j + 8 wave + lane / 8, stored chunk lane % 8 -> chunk (lane % 8) ^ (row % 8)
+  unsigned kbase, vbase;      // bytes from the tile's first key within its page, for j = 0 (keys: bits 2-3 of the
+                              // exchange left out)
+  {
+    const int krow = wave * (64 / CPR) + lane / CPR;
+    kbase = (krow * DH + ((lane % CPR) ^ (krow & 3)) * 8) * 2;
+    const int d = 8 * wave + (lane >> 3);
+    vbase = (d * page_size + ((lane & 7) ^ (d & 7)) * 8) * 2;
+  }
+  const int vkey = ((lane & 7) ^ ((lane >> 3) & 7)) * 8;     // the first key of the lane's value chunks
+  auto key_offset = [&](int j) -> unsigned {
+    // bits 3-4 of the row (head size 128: rows 16 j + 4 wave + ..) or bit 3 (head size 64: rows 32 j + 8 wave
+    // + ..) go to bits 2-3 of the chunk number, bits 6-7 of the byte offset
+    const int high = NDB == 8 ? ((2 * j + (wave >> 1)) & 3) : (wave & 1);
+    unsigned base = kbase;
+    asm volatile("" : "+v"(base));
+    return (base ^ (high << 6)) + j * 4096;
+  };
+  auto value_offset = [&](int j) -> unsigned {
+    unsigned base = vbase;
+    asm volatile("" : "+v"(base));
+    return base + j * 32 * page_size * 2;
+  };
+  auto lookup = [&](int tile0) { return tab[min(tile0, total - 1) >> page_shift]; };
+  auto key_source = [&](int tile0, int page) -> const bf16_t* {
+    const int pg = min(max(page, 0), num_pages - 1);
+    return k_pages + ((size_t)pg * num_kv + kvh) * head_stride + (size_t)(tile0 & pmask) * DH;
+  };
+  auto value_source = [&](int tile0, int page) -> const bf16_t* {
+    const int pg = min(max(page, 0), num_pages - 1);
+    return v_pages + ((size_t)pg * num_kv + kvh) * head_stride + (tile0 & pmask);
+  };
+  auto issue_key_load = [&](int j, int buf, const bf16_t* src) {
+    load_to_lds(src, key_offset(j), kbuf_lds + buf * TILE_BYTES + wave * 1024 + j * 4096);
+  };
+  auto issue_value_load = [&](int j, int buf, const bf16_t* src) {
+    load_to_lds(src, value_offset(j), vbuf_lds + buf * TILE_BYTES + wave * 1024 + j * 4096);
+  };
+  auto issue_keys = [&](int buf, int tile0, int page) {
+    const bf16_t* src = key_source(tile0, page);
+#pragma unroll
+    for (int j = 0; j < NLD; ++j) issue_key_load(j, buf, src);
+  };
+  auto issue_values = [&](int buf, int tile0, int page) {
+    const bf16_t* src = value_source(tile0, page);
+#pragma unroll
+    for (int j = 0; j < NLD; ++j) issue_value_load(j, buf, src);
+  };
+  // after the lane's own loads have landed: zero what must not be seen
+  auto clear_values = [&](int buf, int tile0) {
+    if (tile0 + 64 <= total) return;
+#pragma unroll
+    for (int j = 0; j < NLD; ++j) {
+      const int k0 = tile0 + vkey;
+      if (k0 + 8 > total) {
+        bf16x8* at = (bf16x8*)(vbuf + buf * TILE_BYTES + ((4 * j + wave) * 64 + lane) * 16);
+        bf16x8 v = *at;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (k0 + e >= total) v[e] = 0;
+        *at = v;
+      }
+    }
+  };
+
+  // the block's key tiles in equal shares for its sets of waves, as in the kernel above
+  const int share = (blk_last / 64 + GROUPS) / GROUPS;
+  const int tile_begin = grp * share * 64;
+  const int tile_last = min(blk_last, tile_begin + share * 64 - 1);
+  const int n_live = tile_last >= tile_begin ? (tile_last - tile_begin) / 64 + 1 : 0;     // tiles of this set
+  // the tiles of this wave: those that some query of it sees
+  int it_b = last_q >= tile_begin ? min(n_live - 1, (last_q - tile_begin) >> 6) : -1;
+  if (!wave_on) it_b = -1;
+  it_b = __builtin_amdgcn_readfirstlane(it_b);
+
+  float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
+  f32x4 o[NDB][2];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) o[db][qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  // fragment reads: byte offsets of this lane, to which the block of rows adds a constant
+  const int swr = NDB == 8 ? r : (r & 7);
+  const int krow_off = (8 * (r >> 2) + (r & 3)) * CPR * 16;
+  int kchunk[NKS], vchunk[2];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) kchunk[ks] = krow_off + (((4 * ks + g) ^ swr) & (CPR - 1)) * 16;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) vchunk[t] = r * 128 + ((4 * t + g) ^ (r & 7)) * 16;
+
+  // S^T = K Q^T of one tile: row r of key block kb is key 32 (kb / 2) + 8 (r / 4) + 4 (kb % 2) + r % 4
+  auto read_keys = [&](const char* kd, int kb, bf16x8* dst) {
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks)
+      dst[ks] = *(const bf16x8*)(kd + (32 * (kb >> 1) + 4 * (kb & 1)) * CPR * 16 + kchunk[ks]);
+  };
+  auto multiply_keys = [&](const bf16x8* kf, f32x4 (&s)[2]) {
+    f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[0][ks], a0, 0, 0, 0);
+      a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[1][ks], a1, 0, 0, 0);
+    }
+    s[0] = a0;
+    s[1] = a1;
+  };
+  auto scores = [&](int buf, f32x4 (&s)[4][2]) {
+    const char* kd = kbuf + buf * TILE_BYTES;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      bf16x8 kf[NKS];
+      read_keys(kd, kb, kf);
+      multiply_keys(kf, s[kb]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto mask = [&](int tile0, f32x4 (&s)[4][2]) {
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = tile0 + 32 * (kb >> 1) + 8 * g + 4 * (kb & 1) + i;
+          if (key > qpos[qb]) s[kb][qb][i] = -INFINITY;
+        }
+  };
+  // The softmax of a tile in parts, so that each can be set beside a quarter of the next tile's score
+  // products. The scores become probabilities in place.
+  // The reference maximum m of a query (probabilities are e^(score - m)) follows the true maximum lazily: it
+  // moves, for all queries of the wave at once, when some query meets a score more than RESCALE_AT powers of
+  // two above its own m. Between such moves no sum needs rescaling and a probability is at most 2^RESCALE_AT,
+  // which changes nothing in the quotient of the sums. `moved` tells the caller to multiply the sums so far
+  // by `alpha`.
+  constexpr float RESCALE_AT = 8.f;
+  float m_log2[2] = {0.f, 0.f};
+  auto softmax_maximum = [&](const f32x4 (&s)[4][2], float (&alpha)[2]) -> bool {
+    float mx[2];
+    bool jump = false;
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      float x = -INFINITY;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x = fmaxf(x, s[kb][qb][i]);
+      mx[qb] = rows_max(x);
+      jump = jump || (mx[qb] - m[qb]) * LOG2E > RESCALE_AT;     // false where both are -inf
+    }
+    const bool moved = __builtin_amdgcn_ballot_w64(jump) != 0;
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      const float m_new = moved ? fmaxf(m[qb], mx[qb]) : m[qb];
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      // e^(x - m) as 2^(x log2 e - m log2 e): one multiply-add and the hardware's 2^x
+      m_log2[qb] = m_safe * LOG2E;
+      alpha[qb] = __builtin_amdgcn_exp2f((m[qb] - m_safe) * LOG2E);
+      m[qb] = m_new;
+    }
+    return moved;
+  };
+  // the probabilities of four keys (one block of four registers)
+  auto exponentials = [&](f32x4 (&s)[4][2], int kb, int qb) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s[kb][qb][i] = __builtin_amdgcn_exp2f(fmaf(s[kb][qb][i], LOG2E, -m_log2[qb]));
+  };
+  // the probabilities of keys 32 t .. 32 t + 31 of the tile as the B operands of the value products
+  auto rounded = [&](const f32x4 (&s)[4][2], int t, bf16x8 (&pb)[2]) {
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pb[qb][j] = (bf16_t)s[2 * t + (j >> 2)][qb][j & 3];
+  };
+  // The sums of the probabilities come from the matrix unit as well: a block of ones in the place of the
+  // values gives every lane the sum over the keys for its query, of the probabilities as they are multiplied
+  // (rounded), with no addition or exchange between lanes on the vector unit.
+  f32x4 lsum[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+  bf16x8 ones;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) ones[j] = (bf16_t)1.f;
+  auto rescale = [&](const float (&alpha)[2]) {
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[db][qb][i] *= alpha[qb];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) lsum[qb][i] *= alpha[qb];
+    }
+  };
+  // O^T += V^T P^T, and the second half of the softmax. The probabilities of the tile's first 32 keys are
+  // there; those of the other 32 are made between the products of the first, and `next`, if asked, takes the
+  // place of the probabilities between the products of the second half: some two vector instructions to a
+  // matrix instruction everywhere, as beside the score products, so that neither unit waits for the other
+  // for long. The values of 16 head-size elements are read two steps before their products.
+  auto weighted_values = [&](int buf, f32x4 (&s)[4][2], const f32x4 (&next)[4][2], bool take_next) {
+    const char* vd = vbuf + buf * TILE_BYTES;
+    auto read_values = [&](int j) { return *(const bf16x8*)(vd + 16 * (j % NDB) * 128 + vchunk[j / NDB]); };
+    constexpr int AHEAD = 2;
+    bf16x8 vf[AHEAD + 1], pb[2];
+#pragma unroll
+    for (int j = 0; j < AHEAD; ++j) vf[j] = read_values(j);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 2 * NDB; ++j) {
+      const int db = j % NDB;
+      if (j + AHEAD < 2 * NDB) vf[(j + AHEAD) % (AHEAD + 1)] = read_values(j + AHEAD);
+      if (db == 0) {
+        rounded(s, j / NDB, pb);
+        lsum[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[0], lsum[0], 0, 0, 0);
+        lsum[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[1], lsum[1], 0, 0, 0);
+      }
+      o[db][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j % (AHEAD + 1)], pb[0], o[db][0], 0, 0, 0);
+      o[db][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j % (AHEAD + 1)], pb[1], o[db][1], 0, 0, 0);
+      // the vector work of this step: 4 * NDB / ... pieces of four registers over the NDB steps of a half
+      constexpr int PER = 4 / (NDB / 2 > 4 ? 4 : NDB / 2);     // blocks of four registers a step: 1 (NDB 8), 2 (NDB 4)
+#pragma unroll
+      for (int c = PER * db; c < PER * db + PER; ++c) {
+        if (c >= 4) break;
+        if (j < NDB) {
+          exponentials(s, 2 + (c >> 1), c & 1);
+        } else if (take_next) {
+          s[c >> 1][c & 1] = next[c >> 1][c & 1];
+          s[2 + (c >> 1)][c & 1] = next[2 + (c >> 1)][c & 1];
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto softmax_and_values = [&](int buf, f32x4 (&s)[4][2], const f32x4 (&next)[4][2], bool take_next) {
+    float alpha[2];
+    const bool moved = softmax_maximum(s, alpha);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) exponentials(s, c >> 1, c & 1);
+    __builtin_amdgcn_sched_barrier(0);
+    if (moved) rescale(alpha);
+    weighted_values(buf, s, next, take_next);
+  };
+  // The scores of the next tile beside the softmax of the current one: after each product a few vector
+  // instructions of the softmax part that stands beside this quarter of the products.
+  // The loads of the step (the values of the next tile, the keys of the one after it) are issued one at a
+  // time between the quarters, not together at the step's start, where every wave of the block would wait
+  // for room in the queue of the memory pipeline with the matrix unit idle.
+  auto scores_beside_softmax = [&](int buf, f32x4 (&next)[4][2], f32x4 (&cur)[4][2], float (&alpha)[2],
+                                   int load_buf_v, const bf16_t* vsrc, int load_buf_k, const bf16_t* ksrc) -> bool {
+    const char* kd = kbuf + buf * TILE_BYTES;
+    // One set of key fragments: half of the next block's are asked for when the first half of this block's
+    // products has been issued, the rest after the second (the registers do not hold two sets).
+    bf16x8 kf[NKS];
+    bool moved = false;
+    read_keys(kd, 0, kf);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+#pragma unroll
+        for (int ks = half * NKS / 2; ks < (half + 1) * NKS / 2; ++ks) {
+          a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[0][ks], a0, 0, 0, 0);
+          a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[1][ks], a1, 0, 0, 0);
+        }
+        if (kb < 3) {
+#pragma unroll
+          for (int ks = half * NKS / 2; ks < (half + 1) * NKS / 2; ++ks)
+            kf[ks] = *(const bf16x8*)(kd + (32 * ((kb + 1) >> 1) + 4 * ((kb + 1) & 1)) * CPR * 16 + kchunk[ks]);
+        }
+        // the maximum beside the first two blocks of products, the first half's probabilities beside the rest
+        if (kb == 0 && half == 0) moved = softmax_maximum(cur, alpha);
+        if (kb >= 2) exponentials(cur, kb - 2, half);
+#pragma unroll
+        for (int i = 0; i < NKS; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (kb < 2) __builtin_amdgcn_sched_group_barrier(0x002, 12 / NKS, 0);
+          else __builtin_amdgcn_sched_group_barrier(0x002, 8 / NKS, 0);
+        }
+        if (kb < 3) __builtin_amdgcn_sched_group_barrier(0x100, NKS / 2, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        {
+          constexpr int PER = NLD / 4 > 0 ? NLD / 4 : 1;       // loads a half-quarter: 2 NLD loads over 8 of them
+          const int slot = 2 * kb + half;
+          if (NLD == 4 || slot % 2 == 0) {
+            const int j = NLD == 4 ? slot : slot / 2;          // 0 .. 2 NLD - 1
+            if (j < NLD) issue_value_load(j, load_buf_v, vsrc);
+            else issue_key_load(j - NLD, load_buf_k, ksrc);
+          }
+          (void)PER;
+        }
+      }
+      next[kb][0] = a0;
+      next[kb][1] = a1;
+    }
+    return moved;
+  };
+
+  f32x4 s_even[4][2], s_odd[4][2];
+  int page1, page2;       // pages of the tiles one and two after the current one
+  {
+    const int page0 = lookup(tile_begin);
+    page1 = lookup(tile_begin + 64);
+    page2 = lookup(tile_begin + 128);
+    if (n_live > 0) {
+      issue_keys(0, tile_begin, page0);
+      issue_values(0, tile_begin, page0);
+    }
+    if (n_live > 1) issue_keys(1, tile_begin + 64, page1);
+    wait_for_loads();                                 // this lane's loads are in LDS
+    if (n_live > 0) clear_values(0, tile_begin);
+    __syncthreads();
+    if (it_b >= 0) scores(0, s_even);
+  }
+  // Step `it`: LDS holds the keys of tile it + 1 and the values of tile it; `cur` holds the scores of tile it.
+  // Every step passes one barrier, whichever loop below it belongs to: the waves of a block take different
+  // numbers of steps in the first loop and the same number in both together.
+  auto begin_step = [&](int it, bool with_loads) {
+    __syncthreads();      // every wave is done with tile it - 1; tile it's values and tile it + 1's keys are there
+    const int tile0 = tile_begin + 64 * it;
+    if (with_loads) {
+      if (it + 1 < n_live) issue_values((it + 1) & 1, tile0 + 64, page1);
+      if (it + 2 < n_live) issue_keys(it & 1, tile0 + 128, page2);
+    }
+  };
+  auto end_step = [&](int it) {
+    // the page of the tile after the next two is looked up here, where the wave waits anyway
+    page1 = page2;
+    page2 = lookup(tile_begin + 64 * it + 192);
+    wait_for_loads();
+    if (it + 1 < n_live) clear_values((it + 1) & 1, tile_begin + 64 * it + 64);
+  };
+  // the tiles that every query of the wave sees whole and that another tile of the wave follows
+  const int n_full = first_q + 1 > tile_begin ? (first_q + 1 - tile_begin) >> 6 : 0;
+  const int n_hot = __builtin_amdgcn_readfirstlane(max(0, min(it_b, n_full)));
+  f32x4 (&cur)[4][2] = s_even, (&next)[4][2] = s_odd;
+  int it = 0;
+  for (; it < n_hot; ++it) {
+    begin_step(it, false);
+    float alpha[2];
+    // a tile beyond the set's last is not read by anyone: its loads bring the last tile once more
+    const int tile_v = tile_begin + 64 * min(it + 1, n_live - 1), tile_k = tile_begin + 64 * min(it + 2, n_live - 1);
+    const bool moved = scores_beside_softmax((it + 1) & 1, next, cur, alpha, (it + 1) & 1, value_source(tile_v, page1),
+                                             it & 1, key_source(tile_k, it + 2 < n_live ? page2 : page1));
+    if (moved) rescale(alpha);
+    weighted_values(it & 1, cur, next, true);
+    end_step(it);
+  }
+  // the wave's last tiles, which the positions mask, and the steps in which it only loads and waits
+  for (; it < share; ++it) {
+    begin_step(it, true);
+    const int tile0 = tile_begin + 64 * it;
+    const bool has_cur = it <= it_b, has_next = it + 1 <= it_b;
+    if (has_next) scores((it + 1) & 1, next);
+    if (has_cur) {
+      if (tile0 + 63 > first_q) mask(tile0, cur);
+      softmax_and_values(it & 1, cur, next, has_next);
+    }
+    end_step(it);
+  }
+
+  l[0] = lsum[0][0];
+  l[1] = lsum[1][0];
+  if (GROUPS == 2) {
+    // the second set leaves what it has in LDS (every lane its own words, lanes side by side), the first adds it
+    float* po = (float*)pipelined_smem;                         // [4 waves][NDB][2][4][64]
+    float* pml = po + 4 * NDB * 2 * 4 * 64;                     // [4 waves][2][2][64]
+    __syncthreads();                                            // the staged tiles are done with
+    if (grp == 1 && wave_on) {
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) {
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) po[(((wave * NDB + db) * 2 + qb) * 4 + i) * 64 + lane] = o[db][qb][i];
+        pml[((wave * 2 + qb) * 2 + 0) * 64 + lane] = m[qb];
+        pml[((wave * 2 + qb) * 2 + 1) * 64 + lane] = l[qb];
+      }
+    }
+    __syncthreads();
+    if (grp == 1) return;
+    if (wave_on) {
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) {
+        const float m1 = pml[((wave * 2 + qb) * 2 + 0) * 64 + lane];
+        const float l1 = pml[((wave * 2 + qb) * 2 + 1) * 64 + lane];
+        const float m_all = fmaxf(m[qb], m1);
+        const float m_safe = m_all == -INFINITY ? 0.f : m_all;
+        const float a0 = __builtin_amdgcn_exp2f((m[qb] - m_safe) * LOG2E);
+        const float a1 = __builtin_amdgcn_exp2f((m1 - m_safe) * LOG2E);
+        l[qb] = l[qb] * a0 + l1 * a1;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            o[db][qb][i] = o[db][qb][i] * a0 + po[(((wave * NDB + db) * 2 + qb) * 4 + i) * 64 + lane] * a1;
+      }
+    }
+  }
+  if (!wave_on) return;
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int qi = qw0 + 16 * qb + r;
+    if (qi >= qlen) continue;
+    const float inv = 1.f / l[qb];
+    bf16_t* orow = out + (size_t)(t0 + qi) * nq + h * DH;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+      bf16x4 v4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v4[i] = (bf16_t)(o[db][qb][i] * inv);
+      *(bf16x4*)(orow + 16 * db + 4 * g) = v4;
+    }
+  }
+}
+
+template <int NDB, int GROUPS>
+static int launch_prefill_pipelined(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k_pages,
+                                    const bf16_t* v_pages, const int* run_start, const int* cached_lens,
+                                    const int* table, int table_width, int page_shift, int num_pages,
+                                    const int* tile_run, const int* tile_q0, bf16_t* out, int num_heads, int num_kv,
+                                    int head_size, int window) {
+  constexpr size_t bytes = GROUPS * 4 * (size_t)(64 * 16 * NDB * 2);
+  static_assert(bytes <= 160 * 1024, "the staging buffers must fit the 160 KB of LDS");
+  static_assert(GROUPS == 1 || bytes >= (4 * NDB * 2 * 4 * 64 + 4 * 2 * 2 * 64) * sizeof(float),
+                "the partial results of the second set of waves must fit the staging buffers");
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)attention_prefill_pipelined_kernel<NDB, GROUPS>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) {
+      tnx_set_error("attention_prefill: cannot reserve %zu bytes of LDS: %s", bytes, hipGetErrorString(e));
+      return 2;
+    }
+    configured = true;
+  }
+  (void)head_size;
+  (void)window;
+  attention_prefill_pipelined_kernel<NDB, GROUPS><<<grid, 256 * GROUPS, bytes, stream>>>(
+      q, k_pages, v_pages, run_start, cached_lens, table, table_width, page_shift, num_pages, tile_run, tile_q0, out,
+      num_heads, num_kv);
+  return 0;
+}
+
 extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const void* v_pages, const int* run_start,
                                      const int* cached_lens, const int* table, int table_width, int page_size,
                                      int num_pages, const int* tile_run, const int* tile_q0, int num_tiles, void* out,
@@ -883,10 +1398,14 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
   // that run longest start first and the short ones fill in behind them.
   dim3 grid((unsigned)num_tiles * num_heads);
   if ((page_size & (page_size - 1)) == 0 && direct != 1) {
-    const int sets = direct == 2 ? 1 : 2;       // `direct` 2: one set of waves a block; 0 or 3: two
+    // `direct` 0 or 3: two sets of waves a block; 2: one set; 6 and 7: the same with the staged kernel where the
+    // pipelined one would run (head sizes 64 and 128, pages of 64 keys or more, no window)
+    const int sets = (direct == 2 || direct == 7) ? 1 : 2;
+    const bool pipelined = direct != 6 && direct != 7 && window <= 0 && page_size >= 64 &&
+                           (head_size == 64 || head_size == 128);
     int page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
-    int rc;
+    int rc = -1;
 #define LDS_ARGS                                                                                                 \
   grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, \
       table_width, page_shift, num_pages, tile_run, tile_q0, (bf16_t*)out, num_heads, num_kv, head_size, window
@@ -899,7 +1418,12 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
     else                                                                                                         \
       rc = fast ? launch_prefill_lds<NDB, true, G>(LDS_ARGS) : launch_prefill_lds<NDB, false, G>(LDS_ARGS);      \
   }
-    if (head_size <= 64) {
+    if (pipelined) {
+      if (head_size == 64)
+        rc = sets == 2 ? launch_prefill_pipelined<4, 2>(LDS_ARGS) : launch_prefill_pipelined<4, 1>(LDS_ARGS);
+      else
+        rc = sets == 2 ? launch_prefill_pipelined<8, 2>(LDS_ARGS) : launch_prefill_pipelined<8, 1>(LDS_ARGS);
+    } else if (head_size <= 64) {
       LAUNCH_LDS(4);
     } else if (head_size <= 128) {
       LAUNCH_LDS(8);

@@ -157,3 +157,27 @@ __device__ __forceinline__ float apply_act(float x, int act) {
       return x;
   }
 }
+
+// ---- loads from global memory straight into LDS (`global_load_lds_dwordx4`)
+// 16 bytes a lane from `base + offset` (offset in bytes, per lane) to LDS at `lds + 16 * lane` (the same for the
+// whole wave). Written as assembly so that the compiler does not know of it: with such a load in flight it
+// makes every wait for an LDS read a wait for all LDS reads, and the reads of the next fragments could not
+// stay in flight during the products of these. The caller waits (`wait_for_loads`) before anyone reads.
+__device__ __forceinline__ void load_to_lds(const void* base, unsigned offset, unsigned lds) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds), "v"(offset), "s"(base)
+               : "memory");
+}
+// the same from a pointer of the lane's own
+__device__ __forceinline__ void load_to_lds(const void* address, unsigned lds) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(lds), "v"(address)
+               : "memory");
+}
+__device__ __forceinline__ void wait_for_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// the address of a place in LDS as such a load wants it
+__device__ __forceinline__ unsigned lds_offset(const void* p) {
+  return (unsigned)(size_t)(const __attribute__((address_space(3))) char*)p;
+}

@@ -351,11 +351,11 @@ gemm_bf16_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w
 #pragma unroll
     for (int j = 0; j < LPA; ++j)
       if (j % parts == part)
-        __builtin_amdgcn_global_load_lds((glb_ptr)(xsrc[j] + k0), (lds_ptr)(a_dst + j * 1024), 16, 0, 0);
+        load_to_lds(xsrc[j] + k0, lds_offset(a_dst + j * 1024));
 #pragma unroll
     for (int j = 0; j < LPT; ++j)
       if (j % parts == part)
-        __builtin_amdgcn_global_load_lds((glb_ptr)(wsrc[j] + k0), (lds_ptr)(b_dst + j * 1024), 16, 0, 0);
+        load_to_lds(wsrc[j] + k0, lds_offset(b_dst + j * 1024));
   };
   auto issue = [&](int stage, int k0) { issue_part(stage, k0, 0, 1); };
   int a_off[MI], b_off[4];
