@@ -1184,41 +1184,47 @@ attention_prefill_pipelined_kernel(const bf16_t* __restrict__ q, const bf16_t* _
   auto scores_beside_softmax = [&](int buf, f32x4 (&next)[4][2], f32x4 (&cur)[4][2], float (&alpha)[2],
                                    int load_buf_v, const bf16_t* vsrc, int load_buf_k, const bf16_t* ksrc) -> bool {
     const char* kd = kbuf + buf * TILE_BYTES;
-    // One set of key fragments: half of the next block's are asked for when the first half of this block's
-    // products has been issued, the rest after the second (the registers do not hold two sets).
-    bf16x8 kf[NKS];
+    // The fragments of half a block of keys (NKS / 2 steps of 32 over the head size) at a time, three such sets
+    // in turn: a set is asked for two half-blocks (eight products) before it is used; the registers do not
+    // hold more.
+    constexpr int HK = NKS / 2;
+    bf16x8 kf[3][HK];
     bool moved = false;
-    read_keys(kd, 0, kf);
+    auto read_half = [&](int slot, bf16x8* dst) {      // half-block `slot` of the tile: key block slot / 2
+      const int kb = slot >> 1, half = slot & 1;
+#pragma unroll
+      for (int i = 0; i < HK; ++i)
+        dst[i] = *(const bf16x8*)(kd + (32 * (kb >> 1) + 4 * (kb & 1)) * CPR * 16 + kchunk[half * HK + i]);
+    };
+    read_half(0, kf[0]);
+    read_half(1, kf[1]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
       f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
+        const int slot = 2 * kb + half;
+        if (slot + 2 < 8) read_half(slot + 2, kf[(slot + 2) % 3]);
 #pragma unroll
-        for (int ks = half * NKS / 2; ks < (half + 1) * NKS / 2; ++ks) {
-          a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[0][ks], a0, 0, 0, 0);
-          a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[1][ks], a1, 0, 0, 0);
-        }
-        if (kb < 3) {
-#pragma unroll
-          for (int ks = half * NKS / 2; ks < (half + 1) * NKS / 2; ++ks)
-            kf[ks] = *(const bf16x8*)(kd + (32 * ((kb + 1) >> 1) + 4 * ((kb + 1) & 1)) * CPR * 16 + kchunk[ks]);
+        for (int i = 0; i < HK; ++i) {
+          const int ks = half * HK + i;
+          a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[slot % 3][i], qf[0][ks], a0, 0, 0, 0);
+          a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[slot % 3][i], qf[1][ks], a1, 0, 0, 0);
         }
         // the maximum beside the first two blocks of products, the first half's probabilities beside the rest
         if (kb == 0 && half == 0) moved = softmax_maximum(cur, alpha);
         if (kb >= 2) exponentials(cur, kb - 2, half);
+        if (slot + 2 < 8) __builtin_amdgcn_sched_group_barrier(0x100, HK, 0);
 #pragma unroll
         for (int i = 0; i < NKS; ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           if (kb < 2) __builtin_amdgcn_sched_group_barrier(0x002, 12 / NKS, 0);
           else __builtin_amdgcn_sched_group_barrier(0x002, 8 / NKS, 0);
         }
-        if (kb < 3) __builtin_amdgcn_sched_group_barrier(0x100, NKS / 2, 0);
         __builtin_amdgcn_sched_barrier(0);
         {
           constexpr int PER = NLD / 4 > 0 ? NLD / 4 : 1;       // loads a half-quarter: 2 NLD loads over 8 of them
-          const int slot = 2 * kb + half;
           if (NLD == 4 || slot % 2 == 0) {
             const int j = NLD == 4 ? slot : slot / 2;          // 0 .. 2 NLD - 1
             if (j < NLD) issue_value_load(j, load_buf_v, vsrc);
