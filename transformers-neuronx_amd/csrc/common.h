@@ -163,6 +163,8 @@ __device__ __forceinline__ float apply_act(float x, int act) {
 // whole wave). Written as assembly so that the compiler does not know of it: with such a load in flight it
 // makes every wait for an LDS read a wait for all LDS reads, and the reads of the next fragments could not
 // stay in flight during the products of these. The caller waits (`wait_for_loads`) before anyone reads.
+// M0 is written here behind the compiler's back (it does not take M0 in a clobber list): a kernel that uses
+// these loads must have no other instruction that reads M0, which holds for every kernel of ours.
 __device__ __forceinline__ void load_to_lds(const void* base, unsigned offset, unsigned lds) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :

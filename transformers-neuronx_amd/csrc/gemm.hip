@@ -316,6 +316,9 @@ gemm_bf16_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w
   constexpr int LPA = TM / (4 * RPI);             // load instructions a wave issues for a tile of x
   constexpr int LPT = WT_N / (4 * RPI);           // and of w
   constexpr int KS = BK / 16;                     // k16 steps
+  // the k16 steps of a tile between whose products the next tile's loads are issued: the first two, so that the
+  // last load has half a tile's time to land before the barrier (over all four: 3 to 8% slower; in the first: 2%)
+  constexpr int LOAD_STEPS = KS < 2 ? KS : 2;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = (wave & 1) * 32 * MI, wn = (wave >> 1) * 128;
   const int nb = tiles_m * tiles_n;
@@ -373,7 +376,8 @@ gemm_bf16_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w
 #pragma unroll
   for (int p = 0; p < NSTAGE - 1; ++p)
     if (p < steps) issue(p, p * BK);
-  bf16x8 a[2][MI], b[2][4];
+  constexpr int AHEAD = 1;                        // k16 steps between asking for fragments and using them (2: 3% slower)
+  bf16x8 a[AHEAD + 1][MI], b[AHEAD + 1][4];
   auto frags = [&](int slot, const char* base, int s) {
     const int coff = ((2 * s + lhalf) ^ rsw) * 16;
 #pragma unroll
@@ -402,21 +406,23 @@ gemm_bf16_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w
     const int nstage = (stage + NSTAGE - 1) % NSTAGE, nk = (t + NSTAGE - 1) * BK;
     const char* base = smem + stage * STAGE;
     frags(0, base, 0);
+    if (AHEAD == 2 && KS > 1) frags(1, base, 1);
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
-      // the next step's fragments are asked for first, in one run; this step's products run while they arrive
-      if (s + 1 < KS) frags((s + 1) & 1, base, s + 1);
+      // the fragments of the step after next are asked for first, in one run; this step's products run
+      // while they arrive
+      if (s + AHEAD < KS) frags((s + AHEAD) % (AHEAD + 1), base, s + AHEAD);
       __builtin_amdgcn_sched_barrier(0);
-      if (more) {
-        issue_part(nstage, nk, s, KS);
-        products(s & 1);
+      if (more && s < LOAD_STEPS) {
+        issue_part(nstage, nk, s, LOAD_STEPS);
+        products(s % (AHEAD + 1));
 #pragma unroll
-        for (int g = 0; g < (LPA + LPT) / KS; ++g) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 4 * MI * KS / (LPA + LPT), 0);
+        for (int g = 0; g < (LPA + LPT) / LOAD_STEPS; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 4 * MI * LOAD_STEPS / (LPA + LPT), 0);
           __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
       } else {
-        products(s & 1);
+        products(s % (AHEAD + 1));
       }
       __builtin_amdgcn_sched_barrier(0);
     }
