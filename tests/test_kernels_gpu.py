@@ -593,3 +593,88 @@ def test_fused_projection_from_the_tile_ordered_copy():
     assert torch.equal(torch.isnan(kp), torch.isnan(kp_r)) and torch.equal(torch.isnan(vp), torch.isnan(vp_r))
     torch.testing.assert_close(torch.nan_to_num(kp.float()), torch.nan_to_num(kp_r.float()), rtol=2e-2, atol=2e-2)
     torch.testing.assert_close(torch.nan_to_num(vp.float()), torch.nan_to_num(vp_r.float()), rtol=2e-2, atol=2e-2)
+
+
+# ------------------------------------------------------------------ a LayerNorm folded into the product after it
+
+def _float32_norm_then_product(x, gamma, beta, eps, w, bias, act):
+    """What the folded product must give, in float32 from the stored (bfloat16) matrix."""
+    h = torch.nn.functional.layer_norm(x, (x.shape[1],), gamma, beta, eps)
+    y = h @ w.float().T + (bias if bias is not None else 0)
+    return torch.relu(y) if act == "relu" else y
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 48, 128), (8, 12288, 4096), (16, 16384, 4096), (17, 160, 256),
+                                   (32, 16384, 4096), (5, 1024, 2048), (2, 4096, 4096), (3, 16, 1152)])
+@pytest.mark.parametrize("act", [None, "relu"])
+def test_product_of_normalised_rows(m, n, k, act):
+    """`linear` on the deferred output of a LayerNorm, with the norm folded into the matrix, against the norm
+    and the product in float32: every wave count, tile count and row count of the few-rows kernel. The rows
+    carry a common part a hundred times their spread, which the kernel takes out before it rounds."""
+    from transformers_neuronx_amd.kernels.hip import DeferredNorm
+    hip, _ = _ops(torch.bfloat16)
+    g = torch.Generator(device=DEV).manual_seed(m * 7 + n)
+    x = torch.randn(m, k, device=DEV, generator=g) * torch.rand(m, 1, device=DEV, generator=g) * 3
+    x += torch.randn(m, 1, device=DEV, generator=g) * 100
+    gamma = 1 + 0.2 * torch.randn(k, device=DEV, generator=g)
+    beta = 0.3 * torch.randn(k, device=DEV, generator=g)
+    w = (torch.randn(n, k, device=DEV, generator=g) / k ** 0.5).to(torch.bfloat16)
+    bias = torch.randn(n, device=DEV, generator=g) * 0.2
+    eps = 1e-5
+    pw = hip.prepare_weight(w)
+    assert hip.fold_norm(pw, gamma, beta) and pw.tiles is None and pw.folded is not None
+    h = hip.layernorm_deferred(x, gamma, beta, eps, torch.bfloat16)
+    assert isinstance(h, DeferredNorm)
+    got = hip.linear(h, pw, bias, act=act)
+    want = _float32_norm_then_product(x, gamma, beta, eps, w, bias, act)
+    torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2)
+    # and the same through the norm's own kernel and the plain product (another matrix object: not folded)
+    plain = hip.linear(hip.layernorm(x, gamma, beta, eps, torch.bfloat16, False, True)[1], hip.prepare_weight(w),
+                       bias, act=act)
+    torch.testing.assert_close(got.float(), plain.float(), rtol=2e-2, atol=3e-2)
+    # a deferred norm that meets a matrix it was not folded into is carried out by its own kernel
+    other = hip.linear(h, hip.prepare_weight(w), bias, act=act)
+    assert torch.equal(other, plain)
+
+
+def test_product_of_normalised_rows_without_weight_and_bias():
+    hip, _ = _ops(torch.bfloat16)
+    g = torch.Generator(device=DEV).manual_seed(3)
+    x = torch.randn(4, 256, device=DEV, generator=g)
+    w = (torch.randn(64, 256, device=DEV, generator=g) / 16).to(torch.bfloat16)
+    pw = hip.prepare_weight(w)
+    assert hip.fold_norm(pw, None, None)
+    got = hip.linear(hip.layernorm_deferred(x, None, None, 1e-3, torch.bfloat16), pw, None)
+    want = _float32_norm_then_product(x, None, None, 1e-3, w, None, None)
+    torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2)
+
+
+def test_projection_of_normalised_rows_into_the_cache():
+    """The fused projection on a deferred LayerNorm: queries, and keys and values in their pages, as from
+    the norm's own kernel and the projection after it."""
+    hip, ref = _ops(torch.bfloat16)
+    heads, kv, hs, ps = 4, 2, 32, 16
+    runs, cached = [1, 1, 3, 1], [40, 0, 7, 15]
+    num_pages = 10
+    ctx = _make_step(runs, cached, ps, num_pages, seed=2)
+    view = ctx.groups["full"]
+    width, total = 256, (heads + 2 * kv) * hs
+    g = torch.Generator(device=DEV).manual_seed(4)
+    x = torch.randn(ctx.num_tokens, width, device=DEV, generator=g) * 2 + 5
+    gamma = 1 + 0.2 * torch.randn(width, device=DEV, generator=g)
+    beta = 0.3 * torch.randn(width, device=DEV, generator=g)
+    w = (torch.randn(total, width, device=DEV, generator=g) / 16).to(torch.bfloat16)
+    bias = torch.randn(total, device=DEV, generator=g) * 0.2
+    kp_r = torch.full((num_pages, kv, ps, hs), float("nan"), device=DEV, dtype=torch.bfloat16)
+    vp_r = torch.full((num_pages, kv, hs, ps), float("nan"), device=DEV, dtype=torch.bfloat16)
+    kp, vp = kp_r.clone(), vp_r.clone()
+    h_r = ref.layernorm(x, gamma, beta, 1e-5, torch.bfloat16, False, True)[1]
+    q_r = ref.qkv_project(h_r, w, bias, heads, kv, hs, 0.25, ctx, view, kp_r, vp_r)
+    pw = hip.prepare_weight(w)
+    assert hip.fold_norm(pw, gamma, beta)
+    q = hip.qkv_project(hip.layernorm_deferred(x, gamma, beta, 1e-5, torch.bfloat16), pw, bias, heads, kv, hs, 0.25,
+                        ctx, view, kp, vp)
+    torch.testing.assert_close(q.float(), q_r.float(), rtol=2e-2, atol=2e-2)
+    assert torch.equal(torch.isnan(kp), torch.isnan(kp_r)) and torch.equal(torch.isnan(vp), torch.isnan(vp_r))
+    torch.testing.assert_close(torch.nan_to_num(kp.float()), torch.nan_to_num(kp_r.float()), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(torch.nan_to_num(vp.float()), torch.nan_to_num(vp_r.float()), rtol=2e-2, atol=2e-2)

@@ -158,6 +158,19 @@ __device__ __forceinline__ float apply_act(float x, int act) {
   }
 }
 
+// the compute units of the current device (asked once a device)
+inline int tnx_compute_units() {
+  static int known[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (known[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    known[dev] = n;
+  }
+  return known[dev];
+}
+
 // ---- loads from global memory straight into LDS (`global_load_lds_dwordx4`)
 // 16 bytes a lane from `base + offset` (offset in bytes, per lane) to LDS at `lds + 16 * lane` (the same for the
 // whole wave). Written as assembly so that the compiler does not know of it: with such a load in flight it

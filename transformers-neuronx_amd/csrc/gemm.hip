@@ -546,12 +546,28 @@ static int launch_wide(const bf16_t* x, const bf16_t* w, const float* bias, cons
 // With SHUF the weight is read from a copy laid out for this kernel: [N/16][K/128][4][16 rows][4][8], that is
 // tile after tile in the order the loads take it, so that a block streams one contiguous run of memory and
 // each load of a wave covers 1 KB of it (N a multiple of 16, K of 128).
-template <int MT, int WAVES, bool QKV, bool SHUF, int RT>
+// With NORMED the rows of `x` are those of a LayerNorm's float32 input and the product is that of the
+// normalised rows, without a kernel for the norm: with W' = W diag(gamma), c = W' 1 and d = W beta,
+//     W (gamma (x - mean) rstd + beta) = rstd (W' (x - x0) - (mean - x0) c) + d
+// for any x0. The block's waves read every element of the rows between them anyway (they share K), so the sums
+// of x - x0 and of its square cost no load; x0 is the median of three elements of the row (one of them may be
+// an outlier), so that what is rounded to bfloat16 for the products is small where the row has a large common
+// part. `w` is W' here (tile order), `nf.c`
+// and `nf.d` come with it; K is a multiple of 128.
+struct NormFold {
+  const float* x;      // [M][K] float32
+  const float* c;      // [N]
+  const float* d;      // [N]
+  float eps;
+};
+
+template <int MT, int WAVES, bool QKV, bool SHUF, int RT, bool NORMED = false>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
                         const float* __restrict__ residual, void* __restrict__ out, int out_dtype, int act, int M,
-                        int N, int K, QkvScatter sc) {
+                        int N, int K, QkvScatter sc, NormFold nf) {
   __shared__ float red[WAVES][MT][RT][4][64];
+  __shared__ float stat[WAVES][MT][2][16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 16 * RT;     // RT tiles of 16 weight rows a block; tile j begins at n0 + 16 j
@@ -569,8 +585,16 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
 #pragma unroll
     for (int j = 0; j < RT; ++j) acc[t][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
   const bf16_t* xrow[MT];
+  const float* xfrow[MT];
+  float x0[MT], s1[MT], s2[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) xrow[t] = x + (size_t)min(t * 16 + r, M - 1) * K + 8 * g;
+  for (int t = 0; t < MT; ++t) {
+    const size_t row = (size_t)min(t * 16 + r, M - 1) * K;
+    xrow[t] = NORMED ? nullptr : x + row + 8 * g;
+    xfrow[t] = NORMED ? nf.x + row + 8 * g : nullptr;
+    x0[t] = NORMED ? __builtin_amdgcn_fmed3f(nf.x[row], nf.x[row + K / 2], nf.x[row + K - 1]) : 0.f;
+    s1[t] = s2[t] = 0.f;
+  }
   constexpr int STRIDE = WAVES * 128;
   const int k_full = K & ~127;          // whole steps end here
   const int k_last = k_full - 128;      // the last whole step (negative if there is none)
@@ -587,12 +611,47 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
 #pragma unroll
         for (int s = 0; s < 4; ++s) wf[slot][j][s] = *(const bf16x8*)(wrow[j] + (size_t)k * W_STEP + W_LOAD * s);
     };
+    // NORMED: the float32 elements wait in registers as they came and are shifted, summed and rounded when
+    // their step is multiplied, a step after they were asked for (used at once they would make the wave
+    // wait for every load before them, the weights' among them)
+    f32x4 xr[NORMED ? 2 : 1][MT][4][2];
     auto fetch_x = [&](int slot, int kc) {
       const int k = min(kc, k_last);
+      if (NORMED) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+#pragma unroll
+          for (int s = 0; s < 4; ++s) {
+            xr[slot][t][s][0] = *(const f32x4*)(xfrow[t] + k + 32 * s);
+            xr[slot][t][s][1] = *(const f32x4*)(xfrow[t] + k + 32 * s + 4);
+          }
+        }
+        return;
+      }
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) xf[slot][t][s] = *(const bf16x8*)(xrow[t] + k + 32 * s);
+      }
+    };
+    auto round_x = [&](int slot) {
 #pragma unroll
       for (int t = 0; t < MT; ++t)
 #pragma unroll
-        for (int s = 0; s < 4; ++s) xf[slot][t][s] = *(const bf16x8*)(xrow[t] + k + 32 * s);
+        for (int s = 0; s < 4; ++s) {
+          bf16x8 b;
+          float a1 = 0.f, a2 = 0.f;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float v = xr[slot][t][s][e >> 2][e & 3] - x0[t];
+            a1 += v;
+            a2 = fmaf(v, v, a2);
+            b[e] = (bf16_t)v;
+          }
+          xf[slot][t][s] = b;
+          s1[t] += a1;
+          s2[t] += a2;
+        }
     };
     auto product = [&](int wslot, int xslot) {
 #pragma unroll
@@ -615,6 +674,7 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
           fetch_x((u + 1) & 1, kc + STRIDE);
           fetch_w((u + 2) % 3, kc + 2 * STRIDE);
           __builtin_amdgcn_sched_barrier(0);
+          if (NORMED) round_x(u & 1);
           product(u % 3, u & 1);
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -643,6 +703,17 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
     for (int j = 0; j < RT; ++j)
 #pragma unroll
       for (int i = 0; i < 4; ++i) red[wave][t][j][i][lane] = acc[t][j][i];
+  if (NORMED) {
+    // a row's elements lie with the four lanes that share lane % 16, of every wave
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const float a1 = rows_sum(s1[t]), a2 = rows_sum(s2[t]);
+      if (g == 0) {
+        stat[wave][t][0][r] = a1;
+        stat[wave][t][1][r] = a2;
+      }
+    }
+  }
   __syncthreads();
   // acc[t][j][i] of lane l is output column n0 + 16*j + 4*(l/16) + i, row 16*t + l%16.
   for (int idx = tid; idx < MT * RT * 256; idx += WAVES * 64) {
@@ -651,6 +722,17 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
 #pragma unroll
     for (int wv = 0; wv < WAVES; ++wv) v += red[wv][t][j][i][l];
     const int n = n0 + 16 * j + 4 * (l >> 4) + i, m = t * 16 + (l & 15);
+    if (NORMED && n < N) {
+      float a1 = 0.f, a2 = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv) {
+        a1 += stat[wv][t][0][l & 15];
+        a2 += stat[wv][t][1][l & 15];
+      }
+      const float mean = a1 / (float)K;                       // of x - x0
+      const float var = fmaxf(a2 / (float)K - mean * mean, 0.f);
+      v = rsqrtf(var + nf.eps) * (v - mean * nf.c[n]) + nf.d[n];
+    }
     if (n < N && m < M) {
       if (QKV)
         qkv_store(v, m, n, bias, sc);
@@ -663,27 +745,47 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
 template <int MT, int WAVES, int RT>
 static void launch_skinny(const bf16_t* xp, const bf16_t* wp, const bf16_t* ws, const float* bias,
                           const float* residual, void* out, int out_dtype, int act, int M, int N, int K,
-                          const QkvScatter* sc, hipStream_t stream) {
+                          const QkvScatter* sc, const NormFold* nf, hipStream_t stream) {
   const dim3 grid((N + 16 * RT - 1) / (16 * RT)), block(WAVES * 64);
   const QkvScatter none{};
+  const NormFold plain{};
+  if (nf) {           // the dispatcher has seen to it that there is a tile-ordered weight and MT <= 2
+    if constexpr (MT <= 2) {
+      if (sc)
+        gemm_bf16_skinny_kernel<MT, WAVES, true, true, RT, true><<<grid, block, 0, stream>>>(
+            nullptr, ws, bias, residual, out, out_dtype, act, M, N, K, *sc, *nf);
+      else
+        gemm_bf16_skinny_kernel<MT, WAVES, false, true, RT, true><<<grid, block, 0, stream>>>(
+            nullptr, ws, bias, residual, out, out_dtype, act, M, N, K, none, *nf);
+    }
+    return;
+  }
   if (ws && sc)
     gemm_bf16_skinny_kernel<MT, WAVES, true, true, RT><<<grid, block, 0, stream>>>(xp, ws, bias, residual, out,
-                                                                                out_dtype, act, M, N, K, *sc);
+                                                                                out_dtype, act, M, N, K, *sc, plain);
   else if (ws)
     gemm_bf16_skinny_kernel<MT, WAVES, false, true, RT><<<grid, block, 0, stream>>>(xp, ws, bias, residual, out,
-                                                                                 out_dtype, act, M, N, K, none);
+                                                                                 out_dtype, act, M, N, K, none, plain);
   else if (sc)
     gemm_bf16_skinny_kernel<MT, WAVES, true, false, RT><<<grid, block, 0, stream>>>(xp, wp, bias, residual, out,
-                                                                                 out_dtype, act, M, N, K, *sc);
+                                                                                 out_dtype, act, M, N, K, *sc, plain);
   else
     gemm_bf16_skinny_kernel<MT, WAVES, false, false, RT><<<grid, block, 0, stream>>>(xp, wp, bias, residual, out,
-                                                                                  out_dtype, act, M, N, K, none);
+                                                                                  out_dtype, act, M, N, K, none, plain);
 }
 
 static int gemm_bf16_dispatch(const void* x, const void* w, const void* w_tiles, const float* bias,
                               const float* residual, void* out, int out_dtype, int act, int M, int N, int K,
-                              int force_tiled, const QkvScatter* sc, hipStream_t stream) {
+                              int force_tiled, const QkvScatter* sc, hipStream_t stream,
+                              const NormFold* nf = nullptr) {
   TNX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
+  if (nf) {
+    TNX_REQUIRE(w_tiles != nullptr && M <= 32 && K % 128 == 0 && N % 16 == 0 && force_tiled != 1,
+                "gemm_bf16: a product of normalised rows takes up to 32 rows and a tile-ordered weight, K a "
+                "multiple of 128 and N of 16; got M=%d N=%d K=%d", M, N, K);
+    TNX_REQUIRE(((uintptr_t)nf->x | (uintptr_t)w_tiles) % 16 == 0, "gemm_bf16: operands must be 16-byte aligned");
+    x = w = w_tiles;          // what the checks below look at
+  }
   TNX_REQUIRE(K % 8 == 0, "gemm_bf16: the inner size K=%d must be a multiple of 8", K);
   TNX_REQUIRE(((uintptr_t)x | (uintptr_t)w) % 16 == 0, "gemm_bf16: operands must be 16-byte aligned");
   if (M == 0) return 0;
@@ -699,9 +801,21 @@ static int gemm_bf16_dispatch(const void* x, const void* w, const void* w_tiles,
     // enough to share (more bytes in flight for each of the few blocks). Two weight tiles a block for wide
     // matrices. force_tiled 4 or 8 picks the wave count and 2 the two tiles, for measurements and tests.
     const int waves = force_tiled == 4 || force_tiled == 8 ? force_tiled : (N < 4096 && K >= 2048 ? 8 : 4);
-    const bool two_tiles = force_tiled == 2 || (force_tiled == 0 && waves == 4 && N >= 16384 && M <= 32);
+    // Two or three tiles of weight rows a block where the blocks still fill the chip in whole rounds: every
+    // block reads all of `x`, so fewer blocks read less (up to 16 rows, 12,288 columns on 256 compute
+    // units: 21.2 -> 20.5 us with three tiles, and 27.8 -> 22.7 for normalised rows, which are float32)
+    int tiles_per_block = 1;
+    if (force_tiled == 0 && waves == 4 && M <= 32) {
+      const int units = tnx_compute_units();
+      for (int rt = (M <= 16 ? 3 : 2); rt >= 2 && tiles_per_block == 1; --rt) {
+        const int blocks = (N + 16 * rt - 1) / (16 * rt), rounds = (blocks + units - 1) / units;
+        if (blocks >= 4 * units || (blocks >= units && blocks * 20 >= rounds * units * 19)) tiles_per_block = rt;
+      }
+    }
+    const bool two_tiles = force_tiled == 2 || tiles_per_block == 2;
+    const bool three_tiles = tiles_per_block == 3;
 #define SKINNY(MT, WV, RT) \
-  launch_skinny<MT, WV, RT>(xp, wp, ws, bias, residual, out, out_dtype, act, M, N, K, sc, stream)
+  launch_skinny<MT, WV, RT>(xp, wp, ws, bias, residual, out, out_dtype, act, M, N, K, sc, nf, stream)
 #define SKINNY_MT(WV)                        \
   switch ((M + 15) / 16) {                   \
     case 1: SKINNY(1, WV, 1); break;         \
@@ -709,7 +823,7 @@ static int gemm_bf16_dispatch(const void* x, const void* w, const void* w_tiles,
     case 3: SKINNY(3, WV, 1); break;         \
     default: SKINNY(4, WV, 1); break;        \
   }
-    if (force_tiled == 3 && M <= 16) {
+    if ((force_tiled == 3 || three_tiles) && M <= 16) {
       SKINNY(1, 4, 3);
     } else if (force_tiled == 5 && M <= 16) {
       SKINNY(1, 8, 2);
@@ -779,6 +893,41 @@ extern "C" int tnx_gemm_bf16_qkv(const void* x, const void* w, const void* w_til
   const int N = sc.nq + 2 * sc.nk;
   return gemm_bf16_dispatch(x, w, w_tiles, bias, nullptr, nullptr, TNX_BF16, TNX_ACT_NONE, M, N, K, force_tiled, &sc,
                             stream);
+}
+
+// The same two for the rows of a LayerNorm's input (float32), the norm folded into the product (see `NormFold`):
+// `w_folded` is W diag(gamma) in tile order, `fold_c` its row sums, `fold_d` W beta.
+extern "C" int tnx_gemm_bf16_normed(const float* x, const void* w_folded, const float* fold_c, const float* fold_d,
+                                    float eps, const float* bias, void* out, int out_dtype, int act, int M, int N,
+                                    int K, int force_tiled, hipStream_t stream) {
+  const NormFold nf{x, fold_c, fold_d, eps};
+  return gemm_bf16_dispatch(nullptr, nullptr, w_folded, bias, nullptr, out, out_dtype, act, M, N, K, force_tiled,
+                            nullptr, stream, &nf);
+}
+
+extern "C" int tnx_gemm_bf16_qkv_normed(const float* x, const void* w_folded, const float* fold_c,
+                                        const float* fold_d, float eps, const float* bias, int M, int K,
+                                        const int* token_page, const int* token_off, void* q_out, void* k_pages,
+                                        void* v_pages, float scale, int num_heads, int num_kv, int head_size,
+                                        int page_size, int num_pages, int force_tiled, hipStream_t stream) {
+  TNX_REQUIRE(num_heads > 0 && num_kv >= 0 && head_size > 0 && page_size > 0, "gemm_bf16_qkv: bad sizes");
+  QkvScatter sc;
+  sc.token_page = token_page;
+  sc.token_off = token_off;
+  sc.q_out = (bf16_t*)q_out;
+  sc.k_pages = (bf16_t*)k_pages;
+  sc.v_pages = (bf16_t*)v_pages;
+  sc.scale = scale;
+  sc.nq = num_heads * head_size;
+  sc.nk = num_kv * head_size;
+  sc.head_size = head_size;
+  sc.num_kv = num_kv;
+  sc.page_size = page_size;
+  sc.num_pages = num_pages;
+  const int N = sc.nq + 2 * sc.nk;
+  const NormFold nf{x, fold_c, fold_d, eps};
+  return gemm_bf16_dispatch(nullptr, nullptr, w_folded, bias, nullptr, nullptr, TNX_BF16, TNX_ACT_NONE, M, N, K,
+                            force_tiled, &sc, stream, &nf);
 }
 
 // ------------------------------------------------------------------------------------- the vendor library

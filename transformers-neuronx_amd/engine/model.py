@@ -37,6 +37,7 @@ class _Layer:
     def load(self, tensors, ops, dtype):
         for part, prefix in self._named():
             part.load(tensors, prefix, ops, dtype)
+        self.block.after_load()
 
 
 def _spec_of(kind):

@@ -42,6 +42,11 @@ _SIGNATURES = {
                               _c_int, _c_void_p],
         "tnx_gemm_library": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                              _c_int, _c_void_p, ctypes.c_size_t, _c_void_p, ctypes.c_size_t, _c_int, _c_void_p],
+        "tnx_gemm_bf16_normed": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_int,
+                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_gemm_bf16_qkv_normed": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int,
+                                     _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int,
+                                     _c_int, _c_int, _c_int, _c_int, _c_void_p],
     },
     "attention": {
         "tnx_qkv_write": [_c_void_p, _c_int, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
@@ -82,10 +87,11 @@ class PreparedWeight:
     `[out/16][in/128][4][16][4][8]`: each block then reads one contiguous run of memory. The copy doubles
     the memory of the matrices; it is what decoding reads, the plain tensor is what prompts read."""
 
-    __slots__ = ("tensor", "tiles")
+    __slots__ = ("tensor", "tiles", "folded")
 
     def __init__(self, tensor: torch.Tensor, tiles: Optional[torch.Tensor]):
         self.tensor, self.tiles = tensor, tiles
+        self.folded: Optional["FoldedNorm"] = None
 
     @property
     def shape(self):
@@ -94,6 +100,54 @@ class PreparedWeight:
     @property
     def dtype(self):
         return self.tensor.dtype
+
+
+class FoldedNorm:
+    """A matrix with the LayerNorm in front of it folded in, for the few-rows kernel: `tiles` is
+    W diag(gamma) in tile order, `c` its row sums (of the rounded values, which are what is multiplied),
+    `d` = W beta; `key` names the norm's tensors it was made from."""
+
+    __slots__ = ("tiles", "c", "d", "key", "_with_bias")
+
+    def __init__(self, tiles, c, d, key):
+        self.tiles, self.c, self.d, self.key = tiles, c, d, key
+        self._with_bias = {}
+
+    def d_with(self, bias):
+        """`d + bias`: what a plain product of the folded copy with rows that are normalised but not yet
+        scaled adds (made once a bias vector)."""
+        if bias is None:
+            return self.d
+        k = bias.data_ptr()
+        if k not in self._with_bias:
+            self._with_bias[k] = (self.d + bias).contiguous()
+        return self._with_bias[k]
+
+
+class DeferredNorm:
+    """The input of a LayerNorm whose output only a matrix product reads: the product of few rows applies the
+    norm itself (`HipOps.linear`, `HipOps.qkv_project`); whoever else gets one calls `materialize()`."""
+
+    __slots__ = ("ops", "x", "weight", "bias", "eps", "dtype")
+
+    def __init__(self, ops, x, weight, bias, eps, dtype):
+        self.ops, self.x, self.weight, self.bias, self.eps, self.dtype = ops, x, weight, bias, eps, dtype
+
+    @property
+    def shape(self):
+        return self.x.shape
+
+    @property
+    def key(self):
+        return (self.weight.data_ptr() if self.weight is not None else 0,
+                self.bias.data_ptr() if self.bias is not None else 0)
+
+    def materialize(self):
+        return self.ops.layernorm(self.x, self.weight, self.bias, self.eps, self.dtype, False, True)[1]
+
+    def normalised(self):
+        """`(x - mean) rstd` alone, for a product with a folded copy."""
+        return self.ops.layernorm(self.x, None, None, self.eps, self.dtype, False, True)[1]
 
 
 def tile_order(w: torch.Tensor) -> torch.Tensor:
@@ -308,6 +362,45 @@ class HipOps:
                    _ptr(out_cd), _code(dtype), t, width, _stream())
         return (out_f32 if want_f32 else None), ((out_f32 if same else out_cd) if want_compute else None)
 
+    # Steps of few rows: a LayerNorm that only a matrix product reads is done by that product (`fold_norm`,
+    # `layernorm_deferred`). Up to `fuse_norm_rows` rows the few-rows kernel reads the float32 rows itself
+    # (measured at 4,096 -> 12,288: 23.0 us against 24.4 for norm and product at 8 rows, but 25.8 against 25.2 at
+    # 16 and twice the time at 32: every block reads all rows, and these are float32); beyond that, as far as
+    # the few-rows kernel goes, the norm's kernel normalises and the folded copy does the rest.
+    fuse_norm = True
+    fuse_norm_rows = 8
+    few_rows = 32           # the few-rows kernel takes up to this many rows
+
+    def fold_norm(self, w, weight, bias) -> bool:
+        """Called once when a layer has its tensors, for a matrix `w` that reads a LayerNorm's output and
+        nothing else does: keeps, in the place of its tile-ordered copy, the copy with the norm's weight
+        folded in and the two vectors that go with it (see `FoldedNorm`). False if this matrix has no such
+        copy (then the norm stays a kernel of its own)."""
+        if not (self.fuse_norm and self.dtype == torch.bfloat16 and isinstance(w, PreparedWeight)
+                and w.tiles is not None and w.tensor.dtype == torch.bfloat16):
+            return False
+        full = w.tensor.float()
+        scaled = (full * weight.float()[None, :] if weight is not None else full).to(torch.bfloat16)
+        c = scaled.float().sum(dim=1).contiguous()
+        d = (full @ bias.float() if bias is not None else torch.zeros_like(c)).contiguous()
+        key = (weight.data_ptr() if weight is not None else 0, bias.data_ptr() if bias is not None else 0)
+        w.folded = FoldedNorm(tile_order(scaled), c, d, key)
+        w.tiles = None          # the few-rows steps read the folded copy; the memory stays what it was
+        return True
+
+    def layernorm_deferred(self, x, weight, bias, eps, dtype):
+        """The compute-dtype output of the norm, or, in steps of few rows, a `DeferredNorm`."""
+        if self.fuse_norm and dtype == torch.bfloat16 and self.dtype == torch.bfloat16 \
+                and x.shape[0] <= self.few_rows and x.shape[1] % 128 == 0 and not debug.active():
+            return DeferredNorm(self, x, weight, bias, eps, dtype)
+        return self.layernorm(x, weight, bias, eps, dtype, False, True)[1]
+
+    def _folded_for(self, h, w):
+        """The folded copy of `w` that fits the deferred norm `h`, or None."""
+        if isinstance(w, PreparedWeight) and w.folded is not None and w.folded.key == h.key:
+            return w.folded
+        return None
+
     # ---------------------------------------------------------------- matrix products
 
     decode_copies = True    # keep a tile-ordered copy of every matrix for the few-rows kernel
@@ -321,6 +414,34 @@ class HipOps:
         return PreparedWeight(w, tiles)
 
     def linear(self, x, w, bias=None, act=None, residual=None, out_f32=False, force_tiled=False):
+        if isinstance(x, DeferredNorm):
+            folded = self._folded_for(x, w) if (residual is None and not out_f32 and force_tiled != 1) else None
+            if folded is not None and self._library_product(x.shape[0], w.tensor.shape[0], w.tensor.shape[1],
+                                                              w.tensor, force_tiled):
+                folded = None
+            if folded is None:
+                x = x.materialize()
+            elif x.shape[0] > self.fuse_norm_rows:
+                # the norm's kernel without weight and bias, then the plain product of the folded copy
+                m, k = x.shape
+                n = w.tensor.shape[0]
+                out = torch.empty(m, n, dtype=self.dtype, device=x.x.device)
+                rows, shift = x.normalised(), folded.d_with(bias)     # held until the launch is made
+                self._call("gemm", "tnx_gemm_bf16", _ptr(rows), _ptr(w.tensor), _ptr(folded.tiles), _ptr(shift), None,
+                           _ptr(out), _code(self.dtype), _ACT[act], m, n, k, int(force_tiled), _stream())
+                return out
+            else:
+                if act not in _ACT:
+                    raise ValueError(f"unknown activation {act!r}")
+                m, k = x.shape
+                n = w.tensor.shape[0]
+                if bias is not None:
+                    _want(bias, "bias", torch.float32, (n,))
+                out = torch.empty(m, n, dtype=self.dtype, device=x.x.device)
+                self._call("gemm", "tnx_gemm_bf16_normed", _ptr(x.x), _ptr(folded.tiles), _ptr(folded.c),
+                           _ptr(folded.d), float(x.eps), _ptr(bias), _ptr(out), _code(self.dtype), _ACT[act], m, n, k,
+                           int(force_tiled), _stream())
+                return out
         tiles = None
         if isinstance(w, PreparedWeight):
             w, tiles = w.tensor, w.tiles
@@ -452,6 +573,36 @@ class HipOps:
                     force_tiled=0):
         """Queries, keys and values of the step's tokens: one matrix product whose epilogue scales the
         queries and stores keys and values in their pages (bfloat16), or product and `qkv_write` apart."""
+        if isinstance(h, DeferredNorm):
+            folded = self._folded_for(h, w) if force_tiled != 1 else None
+            if folded is not None and (ctx.num_tokens >= 128 or self._library_product(
+                    ctx.num_tokens, w.tensor.shape[0], w.tensor.shape[1], w.tensor, force_tiled)):
+                folded = None
+            if folded is None:
+                h = h.materialize()
+            elif h.shape[0] > self.fuse_norm_rows:
+                # the norm's kernel without weight and bias, then the fused projection of the folded copy
+                h, w, bias = h.normalised(), PreparedWeight(w.tensor, folded.tiles), folded.d_with(bias)
+            else:
+                t = ctx.num_tokens
+                total = (num_heads + 2 * num_kv_write) * head_size
+                _want(h.x, "x", torch.float32, (t, w.tensor.shape[1]))
+                if tuple(w.tensor.shape) != (total, h.x.shape[1]):
+                    raise ValueError(f"w is {tuple(w.tensor.shape)}, the projections need {(total, h.x.shape[1])}")
+                if bias is not None:
+                    _want(bias, "qkv bias", torch.float32, (total,))
+                num_pages = 0
+                if num_kv_write:
+                    num_pages = self._check_pages(k_pages, v_pages, num_kv_write, head_size, view.page_size)
+                _want(view.token_page, "token pages", torch.int32, (t,))
+                _want(view.token_offset, "token offsets", torch.int32, (t,))
+                q = torch.empty(t, num_heads * head_size, dtype=self.dtype, device=h.x.device)
+                self._call("gemm", "tnx_gemm_bf16_qkv_normed", _ptr(h.x), _ptr(folded.tiles), _ptr(folded.c),
+                           _ptr(folded.d), float(h.eps), _ptr(bias), t, h.x.shape[1], _ptr(view.token_page),
+                           _ptr(view.token_offset), _ptr(q), _ptr(k_pages) if num_kv_write else None,
+                           _ptr(v_pages) if num_kv_write else None, float(scale), num_heads, num_kv_write, head_size,
+                           view.page_size, num_pages, int(force_tiled), _stream())
+                return q
         tiles = None
         if isinstance(w, PreparedWeight):
             w, tiles = w.tensor, w.tiles

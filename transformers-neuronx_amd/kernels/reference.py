@@ -74,6 +74,14 @@ class ReferenceOps:
 
     # ---------------------------------------------------------------- matrix products
 
+    def layernorm_deferred(self, x, weight, bias, eps, dtype):
+        """The norm's output for a part that only multiplies it; a backend may hand back something a
+        product resolves instead (`HipOps.layernorm_deferred`)."""
+        return self.layernorm(x, weight, bias, eps, dtype, False, True)[1]
+
+    def fold_norm(self, w, weight, bias) -> bool:
+        return False
+
     def prepare_weight(self, w):
         """Matrices are used as they are here."""
         return w

@@ -77,12 +77,22 @@ class Mixer(Part):
     def forward(self, h, ctx, cache, residual):
         raise NotImplementedError
 
+    def first_weight(self):
+        """The matrix that `h` is multiplied by, if that product is all this part does with `h` and it goes
+        through `ops.linear` or `ops.qkv_project`; None otherwise. A block may then hand `h` over as
+        what `Norm.deferred` returns and let the product apply the norm."""
+        return None
+
 
 class FeedForward(Part):
     """forward(h, ctx, residual) -> float32 `[T, hidden]`: residual + f(h), token by token."""
 
     def forward(self, h, ctx, residual):
         raise NotImplementedError
+
+    def first_weight(self):
+        """As `Mixer.first_weight`."""
+        return None
 
 
 class Norm(Part):
@@ -91,6 +101,16 @@ class Norm(Part):
 
     def forward(self, x, want_f32: bool, want_compute: bool):
         raise NotImplementedError
+
+    def fold_into(self, w) -> bool:
+        """Asked once, after loading, by a block whose next part only multiplies this norm's output by `w`:
+        True if the backend has folded the norm into `w`, so that `deferred` may be used for that part."""
+        return False
+
+    def deferred(self, x):
+        """The compute-dtype output for a part whose `first_weight` this norm was folded into: the output
+        itself, or what the backend's products take in its place."""
+        return self.forward(x, False, True)[1]
 
 
 class PositionEncoding(Part):
@@ -118,6 +138,9 @@ class Block(Part):
         self.feed_forward = feed_forward
         self.mixer_norm = mixer_norm
         self.feed_forward_norm = feed_forward_norm
+
+    def after_load(self) -> None:
+        """Called when the four parts have their tensors."""
 
     def forward(self, stream, ctx, cache):
         raise NotImplementedError

@@ -11,10 +11,23 @@ class PreNormBlock(Block):
 
     recordable = True
 
+    fold_mixer_norm = fold_feed_forward_norm = False
+
+    def after_load(self) -> None:
+        # Each norm's output goes to one part only; where that part does nothing with it but one matrix
+        # product, the backend may do the norm inside the product (the few-rows products of decode steps:
+        # one launch less for each half of a layer).
+        w = self.mixer.first_weight()
+        self.fold_mixer_norm = w is not None and self.mixer_norm.fold_into(w)
+        w = self.feed_forward.first_weight()
+        self.fold_feed_forward_norm = w is not None and self.feed_forward_norm.fold_into(w)
+
     def forward(self, stream: Stream, ctx, cache) -> Stream:
-        _, h = self.mixer_norm.forward(stream.x, False, True)
+        h = (self.mixer_norm.deferred(stream.x) if self.fold_mixer_norm
+             else self.mixer_norm.forward(stream.x, False, True)[1])
         x = debug.tap("after_mixer", self.mixer.forward(h, ctx, cache, stream.x))
-        _, h = self.feed_forward_norm.forward(x, False, True)
+        h = (self.feed_forward_norm.deferred(x) if self.fold_feed_forward_norm
+             else self.feed_forward_norm.forward(x, False, True)[1])
         x = self.feed_forward.forward(h, ctx, x)
         return Stream(x, None)
 

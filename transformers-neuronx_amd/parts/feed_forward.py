@@ -32,6 +32,9 @@ class DenseFeedForward(FeedForward):
         self.b1 = tensors.get(f"{prefix}{self.up_name}.bias") if self.has_bias else None
         self.b2 = tensors.get(f"{prefix}{self.down_name}.bias") if self.has_bias else None
 
+    def first_weight(self):
+        return self.w1
+
     def forward(self, h, ctx, residual):
         inner = self.ops.linear(h, self.w1, self.b1, act=self.activation)
         return self.ops.linear(inner, self.w2, self.b2, residual=residual, out_f32=True)

@@ -83,6 +83,9 @@ class Attention(Mixer):
         if self.rotation is not None:
             self.rotation.load(tensors, prefix + "rotation", ops, dtype)
 
+    def first_weight(self):
+        return self.w_qkv
+
     def forward(self, h, ctx, cache, residual):
         if cache.writes != self.own_kv:
             raise ValueError("an attention mixer with own_kv writes its cache; one without reads another's")

@@ -31,3 +31,9 @@ class LayerNorm(Norm):
 
     def forward(self, x, want_f32: bool, want_compute: bool):
         return self.ops.layernorm(x, self.weight, self.bias, self.eps, self.dtype, want_f32, want_compute)
+
+    def fold_into(self, w) -> bool:
+        return self.ops.fold_norm(w, self.weight, self.bias)
+
+    def deferred(self, x):
+        return self.ops.layernorm_deferred(x, self.weight, self.bias, self.eps, self.dtype)
