@@ -37,8 +37,11 @@ _ARCHITECTURES: Dict[str, Architecture] = {}
 
 # Packages that register an architecture when they are imported. Another architecture is another package
 # that calls `register_architecture`, and its name here (or a call of `add_architecture_package`, or just
-# its import before a model folder is read).
+# its import before a model folder is read). A program that is started apart (a command line) learns of
+# packages from outside through the environment: TNX_ARCHITECTURE_PACKAGES holds module names, separated
+# by commas, that are importable from where it runs.
 ARCHITECTURE_PACKAGES: List[str] = ["transformers_neuronx_amd.opt"]
+PACKAGES_VARIABLE = "TNX_ARCHITECTURE_PACKAGES"
 
 
 def add_architecture_package(module: str) -> None:
@@ -58,8 +61,14 @@ def known_architectures():
 
 
 def _load_builtin():
-    for module in ARCHITECTURE_PACKAGES:
-        importlib.import_module(module)
+    named = [m.strip() for m in os.environ.get(PACKAGES_VARIABLE, "").split(",") if m.strip()]
+    for module in ARCHITECTURE_PACKAGES + named:
+        try:
+            importlib.import_module(module)
+        except ImportError as e:
+            if module in ARCHITECTURE_PACKAGES:
+                raise
+            raise ConfigError(f"{PACKAGES_VARIABLE} names '{module}', which cannot be imported: {e}") from e
 
 
 def resolve(raw: Dict[str, Any]) -> Architecture:
