@@ -453,3 +453,54 @@ def test_command_line_dump_and_analyze(tiny_folders, tmp_path, capsys):
         torch.save(t, os.path.join(bad, name))
     assert demo.main(["analyze", "-d", bad, dirs["f32"]]) == 1
     assert "step 3" in capsys.readouterr().out
+
+
+def _drawn_case(seed):
+    """A configuration, a precision, a page size, requests and a way of cutting them, all drawn from `seed`."""
+    rng = np.random.default_rng(seed)
+    hs = int(rng.choice([16, 32, 48, 64, 64, 64, 80, 96, 128, 128, 128, 160, 256]))
+    heads = max(1, min(int(rng.integers(1, 7)), 768 // hs))
+    hidden = heads * hs
+    raw = dict(architectures=["OPTForCausalLM"], model_type="opt", vocab_size=int(rng.integers(40, 1500)),
+               hidden_size=hidden, num_hidden_layers=int(rng.integers(1, 4)), num_attention_heads=heads,
+               ffn_dim=int(rng.choice([8, 72, 128, 200, 256, 384, 520, 1024])),
+               max_position_embeddings=int(rng.choice([300, 700])),
+               word_embed_proj_dim=int(rng.choice([hidden, hidden, 48, 136])),
+               do_layer_norm_before=bool(rng.random() < 0.7),
+               activation_function=str(rng.choice(["relu", "gelu", "gelu_new"])),
+               enable_bias=bool(rng.random() < 0.7), layer_norm_elementwise_affine=bool(rng.random() < 0.7),
+               layer_norm_eps=float(rng.choice([1e-5, 1e-3])), init_std=float(rng.choice([0.02, 0.03, 0.05])))
+    dtype = "bfloat16" if rng.random() < 0.7 else "float32"
+    page = int(rng.choice([16, 32, 48, 64, 64, 128]))
+    most = raw["max_position_embeddings"] - 2
+    lengths = [int(min(most, rng.choice([rng.integers(1, 40), rng.integers(40, 300), rng.integers(200, 698)])))
+               for _ in range(int(rng.integers(2, 13)))]
+    max_live = int(rng.integers(1, 13))
+    tail = int(rng.choice([4, 16, 40]))
+    requests = _requests(raw, lengths, seed)
+    rounded = sorted((-(-n // page) * page for n in lengths), reverse=True)
+    kind = str(rng.choice(["mixed", "mixed", "portions", "singles"]))
+    if kind == "mixed":
+        max_tokens = sum(rounded[:max(1, max_live // 2)]) + page
+        steps, place = schedules.mixed(requests, max_tokens=max_tokens, page=page, seed=seed, tail=tail,
+                                       max_live=max_live)
+    else:
+        max_tokens = rounded[0] + page
+        steps, place = (schedules.portions(requests) if kind == "portions"
+                        else schedules.head_then_singles(requests, tail=tail))
+    return raw, dtype, page, requests, max_tokens, steps, place
+
+
+@pytest.mark.parametrize("seed", range(100, 124))
+def test_drawn_configurations_and_schedules(tmp_path, seed):
+    """Sizes, options, precision, page size, up to twelve requests of up to 698 tokens, up to twelve of them
+    live, and the way they are cut into steps: all drawn from the seed, against the plain implementation."""
+    from safetensors.torch import load_file
+    from transformers_neuronx_amd.opt.config import OPTConfig
+    from transformers_neuronx_amd.weights import write_random_model
+    raw, dtype, page, requests, max_tokens, steps, place = _drawn_case(seed)
+    folder = write_random_model(OPTConfig.from_dict(raw), str(tmp_path / "model"), seed, dtype=dtype)
+    weights = load_file(os.path.join(folder, "model.safetensors"))
+    expected = _expected(weights, raw, requests)
+    out, _ = _run(folder, dtype, steps, max_tokens, page, tmp_path, "drawn")
+    _compare(out, place, expected, raw["vocab_size"], dtype)
