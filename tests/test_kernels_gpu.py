@@ -524,7 +524,9 @@ def test_library_product_and_own_product_agree(m, n, k):
     w = (torch.randn(n, k, device=DEV, generator=g) / math.sqrt(k)).to(torch.bfloat16)
     bias = torch.randn(n, device=DEV, generator=g)
     res = torch.randn(m, n, device=DEV, generator=g)
-    for kwargs in (dict(act="relu"), dict(act="gelu"), dict(residual=res, out_f32=True), dict(bias=None)):
+    # (an activation comes before the residual, also where the library, whose own ReLU comes last, makes the product)
+    for kwargs in (dict(act="relu"), dict(act="gelu"), dict(residual=res, out_f32=True), dict(bias=None),
+                   dict(act="relu", residual=res, out_f32=True), dict(act="gelu_new", residual=res, out_f32=True)):
         b = kwargs.pop("bias", bias)
         want = ref.linear(x, w, b, **kwargs).float()
         for ops in (lib, own):

@@ -1122,6 +1122,7 @@ extern "C" int tnx_gemm_library(const void* x, const void* w, const float* bias,
               "gemm_library: operands must be 16-byte aligned");
   TNX_REQUIRE(out != (const void*)residual, "gemm_library: the sum is not made in place");
   if (act != TNX_ACT_NONE && act != TNX_ACT_RELU) return 2;
+  if (act != TNX_ACT_NONE && residual) return 2;   // the library's ReLU comes after the residual sum, ours before it
   std::lock_guard<std::mutex> lock(library_mutex);
   if (!library_ready()) return 2;
   int device = 0;

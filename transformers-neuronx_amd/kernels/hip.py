@@ -463,7 +463,10 @@ class HipOps:
             # library can do that itself: bias and ReLU before it rounds a bfloat16 result, or bias and the
             # residual added to its float32 sums for a float32 result. The float32 head keeps our kernel.
             xa = self.cast(x, torch.bfloat16)
-            if self.library_direct and act in (None, "none", "relu") and (residual is None or out_f32):
+            # (its ReLU comes after everything it adds, so a product with both ReLU and a residual is not its)
+            plain_act = act in (None, "none")
+            if self.library_direct and (plain_act or (act == "relu" and residual is None)) \
+                    and (residual is None or out_f32):
                 out = torch.empty(m, n, dtype=out_dtype, device=x.device)
                 if self._library_call(xa, w, bias, residual, out, act, m, n, k):
                     return out
