@@ -354,8 +354,10 @@ def test_argmax_and_sampling(vocab):
     rows = 24
     logits = torch.randn(rows, vocab, device=DEV, generator=g) * 3
     logits[3, 17] = logits[3, 400 % vocab] = logits[3].max() + 1     # a tie: the lower id wins
+    logits[4] = -1 - logits[4].abs()                                  # -0 and +0 tie as well
+    logits[4, 7], logits[4, 9] = -0.0, 0.0
     assert torch.equal(hip.argmax(logits), ref.argmax(logits))
-    assert int(hip.argmax(logits)[3]) == 17
+    assert int(hip.argmax(logits)[3]) == 17 and int(hip.argmax(logits)[4]) == 7
     temp = torch.tensor([0.0, 1.0, 0.7, 1.3] * 6, device=DEV)
     top_k = torch.tensor([0, 50, 1, 5, 0, vocab + 5] * 4, device=DEV, dtype=torch.int32)
     top_p = torch.tensor([1.0, 1.0, 0.9, 0.5, 0.3, 0.99, 1.0, 0.05] * 3, device=DEV)

@@ -15,6 +15,7 @@ TNX_DEFINE_ERROR_API
 
 __device__ __forceinline__ uint64_t order_key(float x, int idx) {
   if (x != x) x = -INFINITY;  // NaN orders last
+  if (x == 0.f) x = 0.f;      // -0 and +0 are one value: the lower token id decides between them
   uint32_t u = __float_as_uint(x);
   u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
   return ((uint64_t)u << 32) | (uint32_t)(~(uint32_t)idx);
