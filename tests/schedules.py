@@ -100,3 +100,14 @@ def mixed(requests, max_tokens, page=64, seed=0, tail=32, max_live=4):
             del live[rid]
         steps.append({"step": len(steps), "entries": entries, "end": end})
     return _finish(steps)
+
+
+def only_last(made):
+    """The same steps with logits wanted at the last token of each request alone: every other entry wants
+    nothing, and many a step wants nothing at all."""
+    steps, _ = made
+    out = []
+    for rec in steps:
+        entries = [dict(e, want=[len(e["tokens"]) - 1] if e["id"] in rec["end"] else []) for e in rec["entries"]]
+        out.append(dict(rec, entries=entries))
+    return _finish(out)

@@ -81,6 +81,22 @@ def test_schedules_agree_with_plain(tiny_folders, tiny_folders_bf16, tmp_path, d
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_steps_that_want_nothing(tiny_folders, tiny_folders_bf16, tmp_path, dtype, name):
+    """Portions and decoded tokens whose logits nobody asks for: the steps run, leave their keys and values,
+    write no file, and the one row wanted at each request's end is right."""
+    folder, cfg, weights = (tiny_folders if dtype == "float32" else tiny_folders_bf16)[name]
+    requests = _requests(cfg, [5, 40, 77, 120], seed=3)
+    expected = _expected(weights, cfg, requests)
+    for made in (schedules.portions(requests), schedules.mixed(requests, max_tokens=256, page=16, seed=4)):
+        steps, place = schedules.only_last(made)
+        assert len(place) == len(requests) and any(not any(e["want"] for e in s["entries"]) for s in steps)
+        out, _ = _run(folder, dtype, steps, 256, 16, tmp_path, f"last_{len(steps)}")
+        assert sorted(os.listdir(out)) == sorted(f"{step}.f32" for step, _ in place)
+        _compare(out, place, expected, cfg["vocab_size"], dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(tiny_folders, tiny_folders_bf16, tmp_path, dtype):
     """A short prompt, then 240 tokens one by one, across many pages."""
     folder, cfg, weights = (tiny_folders if dtype == "float32" else tiny_folders_bf16)["B"]

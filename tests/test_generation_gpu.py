@@ -60,10 +60,12 @@ def _check_exact(outs, prompts, params, weights, cfg):
 WORKLOADS = {
     "A": dict(lengths=[5, 17, 31], new=16, chunk=None, temperature=0.0),
     "B": dict(lengths=[1, 9, 40, 77, 120], new=14, chunk=32, temperature=0.8),
+    # the model with the norm before the head, its prompts in portions: steps that ask nothing of the head
+    "C": dict(lengths=[3, 64, 65, 150], new=10, chunk=32, temperature=0.0),
 }
 
 
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 @pytest.mark.parametrize("run_ahead", [False, True])
 def test_generation_with_few_pages_float32(tiny_folders, name, run_ahead):
     from transformers_neuronx_amd.sampling import SamplingParams
@@ -138,7 +140,7 @@ def test_late_end_of_sequence_and_arrivals_float32(tiny_folders, prompts_first):
                 assert first[i][1][k] < 1e-5, (i, outs[i], want[i])
 
 
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_generation_with_few_pages_bfloat16(tiny_folders_bf16, name):
     """In bfloat16 a choice may part from the float32 one where two logits are a rounding apart: every
     greedy token must be within the rounding of the best one under the plain implementation, given the

@@ -182,8 +182,8 @@ extern "C" int tnx_layernorm(const float* x, const float* weight, const float* b
                              void* out_cd, int cd_dtype, int tokens, int width, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && width > 0, "layernorm: bad sizes tokens=%d width=%d", tokens, width);
   TNX_REQUIRE(eps > 0.f, "layernorm: eps must be positive");
-  TNX_REQUIRE(out_f32 != x, "layernorm: the float32 output may not alias the input");
   if (tokens == 0) return 0;
+  TNX_REQUIRE(out_f32 != x, "layernorm: the float32 output may not alias the input");
   const bool affine = weight != nullptr;
   TNX_REQUIRE((weight != nullptr) == (bias != nullptr), "layernorm: weight and bias come together or not at all");
   const bool vec = width % 4 == 0 && width <= 1024 * 16 && (cd_dtype == TNX_BF16 || out_cd == nullptr);

@@ -1,6 +1,8 @@
 """Input and output ends of the decoder."""
 from typing import Dict, List, Optional
 
+import torch
+
 from .base import (EMBEDDINGS, HEADS, NORMS, POSITIONS, Part, Stream, register_embedding, register_head)
 from .spec import ParamDecl, PartSpec
 
@@ -75,6 +77,8 @@ class VocabHead(Part):
             self.norm.load(tensors, self.norm_name, ops, dtype)
 
     def forward(self, stream: Stream, ctx):
+        if ctx.logits_rows.numel() == 0:      # a step of prompt portions alone: nothing is asked of the head
+            return torch.empty(0, self.vocab, dtype=torch.float32, device=stream.x.device)
         rows = self.ops.gather_rows(stream.x, ctx.logits_rows)
         if self.norm is not None:
             _, h = self.norm.forward(rows, False, True)
