@@ -406,6 +406,11 @@ ODD = [
     _odd(4099, 6, 64, 1, 1000, None, True, "relu", True, True, 1e-5),
     _odd(96, 2, 128, 1, 136, None, True, "relu", True, True, 1e-5),
     _odd(513, 11, 16, 3, 176, 8, True, "relu", False, False, 1e-3),
+    # inner sizes of products that are no multiple of 8 (bfloat16 rows are read 16 bytes at a time; such
+    # matrices are filled up when they are loaded) and embedding rows of an odd number of elements
+    _odd(211, 2, 32, 2, 37, 33, True, "gelu", True, True, 1e-5),
+    _odd(97, 3, 16, 1, 1, 1, False, "relu", False, False, 1e-4),
+    _odd(300, 4, 64, 2, 1001, 127, True, "relu", True, True, 1e-5),
 ]
 
 

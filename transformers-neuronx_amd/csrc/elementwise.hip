@@ -3,28 +3,33 @@
 
 TNX_DEFINE_ERROR_API
 
-// out[m, :] = src[idx[m], :], rows of `row_bytes` bytes (a multiple of 4). An index -1 - k stands for
+// out[m, :] = src[idx[m], :], rows of `row_bytes` bytes, moved in words of 4 bytes, or of 2 where a row is no
+// whole number of those (bfloat16 rows of odd length). An index -1 - k stands for
 // `indirect[k]`: a row number that an earlier kernel left in device memory (a token that was chosen on the
 // device and has not been read by the host yet).
-__global__ void gather_rows_kernel(const uint32_t* __restrict__ src, const int* __restrict__ idx,
-                                   uint32_t* __restrict__ out, int words, int src_rows,
-                                   const int* __restrict__ indirect, int indirect_size) {
+template <typename W>
+__global__ void gather_rows_kernel(const W* __restrict__ src, const int* __restrict__ idx, W* __restrict__ out,
+                                   int words, int src_rows, const int* __restrict__ indirect, int indirect_size) {
   const int m = blockIdx.x;
   int r = idx[m];
   if (r < 0 && indirect && -1 - r < indirect_size) r = indirect[-1 - r];
   if (r < 0 || r >= src_rows) return;  // the host checks ids; an id out of range writes nothing
-  const uint32_t* s = src + (size_t)r * words;
-  uint32_t* o = out + (size_t)m * words;
+  const W* s = src + (size_t)r * words;
+  W* o = out + (size_t)m * words;
   for (int i = threadIdx.x; i < words; i += blockDim.x) o[i] = s[i];
 }
 
 extern "C" int tnx_gather_rows(const void* src, const int* idx, void* out, int m, int row_bytes, int src_rows,
                                const int* indirect, int indirect_size, hipStream_t stream) {
-  TNX_REQUIRE(row_bytes > 0 && row_bytes % 4 == 0, "gather_rows: row of %d bytes is not a multiple of 4", row_bytes);
+  TNX_REQUIRE(row_bytes > 0 && row_bytes % 2 == 0, "gather_rows: row of %d bytes is not a multiple of 2", row_bytes);
   TNX_REQUIRE(m >= 0 && src_rows > 0, "gather_rows: bad sizes m=%d rows=%d", m, src_rows);
   if (m == 0) return 0;
-  gather_rows_kernel<<<m, 256, 0, stream>>>((const uint32_t*)src, idx, (uint32_t*)out, row_bytes / 4, src_rows,
-                                            indirect, indirect ? indirect_size : 0);
+  if (row_bytes % 4 == 0)
+    gather_rows_kernel<uint32_t><<<m, 256, 0, stream>>>((const uint32_t*)src, idx, (uint32_t*)out, row_bytes / 4,
+                                                         src_rows, indirect, indirect ? indirect_size : 0);
+  else
+    gather_rows_kernel<uint16_t><<<m, 256, 0, stream>>>((const uint16_t*)src, idx, (uint16_t*)out, row_bytes / 2,
+                                                         src_rows, indirect, indirect ? indirect_size : 0);
   TNX_CHECK_LAUNCH("gather_rows");
   return 0;
 }

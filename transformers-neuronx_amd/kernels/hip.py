@@ -87,15 +87,19 @@ class PreparedWeight:
     `[out/16][in/128][4][16][4][8]`: each block then reads one contiguous run of memory. The copy doubles
     the memory of the matrices; it is what decoding reads, the plain tensor is what prompts read."""
 
-    __slots__ = ("tensor", "tiles", "folded")
+    __slots__ = ("tensor", "tiles", "folded", "inner")
 
-    def __init__(self, tensor: torch.Tensor, tiles: Optional[torch.Tensor]):
+    def __init__(self, tensor: torch.Tensor, tiles: Optional[torch.Tensor], inner: Optional[int] = None):
         self.tensor, self.tiles = tensor, tiles
         self.folded: Optional["FoldedNorm"] = None
+        # the matrix's own inner size where `tensor` carries columns of zeros after it (bfloat16 rows are
+        # read 16 bytes at a time: an inner size that is no multiple of 8 is filled up once, here, and the
+        # rows that meet it are filled up as they come)
+        self.inner = tensor.shape[1] if inner is None else inner
 
     @property
     def shape(self):
-        return self.tensor.shape
+        return torch.Size((self.tensor.shape[0], self.inner))
 
     @property
     def dtype(self):
@@ -411,6 +415,9 @@ class HipOps:
         if (self.decode_copies and self.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 2
                 and w.shape[0] % 16 == 0 and w.shape[1] % 128 == 0):
             tiles = tile_order(w)
+        if self.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] % 8:
+            inner = w.shape[1]
+            return PreparedWeight(torch.nn.functional.pad(w, (0, 8 - inner % 8)).contiguous(), None, inner)
         return PreparedWeight(w, tiles)
 
     def linear(self, x, w, bias=None, act=None, residual=None, out_f32=False, force_tiled=False):
@@ -444,6 +451,8 @@ class HipOps:
                 return out
         tiles = None
         if isinstance(w, PreparedWeight):
+            if w.inner != w.tensor.shape[1] and x.shape[1] == w.inner:
+                x = torch.nn.functional.pad(x, (0, w.tensor.shape[1] - w.inner))
             w, tiles = w.tensor, w.tiles
         _want(x, "x")
         _want(w, "w")
