@@ -32,12 +32,13 @@ def unregister_step_planner(name: str) -> None:
 
 
 def attention_plan(run_lens: np.ndarray, cached: np.ndarray, page_size: int):
-    """What the attention kernels launch by: the runs of one token (each attends with one query) and the
-    most keys one of them reads; for every tile of QUERY_TILE queries of the longer runs its run and its first
+    """What the attention kernels launch by: the runs of one token (each attends with one query), those with
+    the most keys first, and the most keys one of them reads; for every tile of QUERY_TILE queries of the longer runs its run and its first
     query, those that see the most keys first (a kernel that takes them in this order starts its longest
     blocks first)."""
     single = run_lens == 1
-    decode_runs = np.nonzero(single)[0].astype(np.int32)
+    decode_runs = np.nonzero(single)[0]
+    decode_runs = decode_runs[np.argsort(-cached[decode_runs], kind="stable")].astype(np.int32)
     longest = int((cached[single] + 1).max()) if single.any() else 0
     tiles = []
     for i in np.nonzero(run_lens > 1)[0]:
