@@ -682,3 +682,49 @@ def test_projection_of_normalised_rows_into_the_cache():
     assert torch.equal(torch.isnan(kp), torch.isnan(kp_r)) and torch.equal(torch.isnan(vp), torch.isnan(vp_r))
     torch.testing.assert_close(torch.nan_to_num(kp.float()), torch.nan_to_num(kp_r.float()), rtol=2e-2, atol=2e-2)
     torch.testing.assert_close(torch.nan_to_num(vp.float()), torch.nan_to_num(vp_r.float()), rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("m,n,k", [(33, 4096, 512), (48, 64, 128), (64, 2560, 1024), (65, 48, 384), (100, 1040, 640),
+                                   (128, 4096, 2048), (7, 16, 128)])
+def test_product_of_some_rows(m, n, k):
+    """The kernel for 33 to 128 rows (it takes fewer too) against float32 torch: every count of row tiles, shares
+    of K that divide its steps unevenly or are cut to what there is, one to four steps in flight (two beyond 64
+    rows), weight tiles beyond the last, float32 and bfloat16 results; and `linear`, which sends the
+    float32-result products of such row counts there."""
+    from transformers_neuronx_amd.kernels.hip import HipOps, _ACT, _code, _ptr, _stream
+    hip = HipOps(torch.bfloat16, DEV)
+    g = torch.Generator(device=DEV).manual_seed(m + n + k)
+    x = torch.randn(m, k, device=DEV, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, device=DEV, generator=g) / math.sqrt(k)).to(torch.bfloat16)
+    bias = torch.randn(n, device=DEV, generator=g)
+    res = torch.randn(m, n, device=DEV, generator=g)
+    pw = hip.prepare_weight(w)
+    assert pw.tiles is not None
+    space = torch.empty(4 << 20, dtype=torch.float32, device=DEV)
+    exact = x.float() @ w.float().t()
+    for shares, ahead in ((0, 0), (1, 1), (2, 2), (3, 3), (7, 4), (64, 0)):
+        for act, b, r, wide in ((None, bias, res, True), ("relu", bias, None, False), ("gelu", None, res, True),
+                                (None, None, None, True)):
+            out = torch.full((m, n), float("nan"), device=DEV, dtype=torch.float32 if wide else torch.bfloat16)
+            hip.call("gemm", "tnx_gemm_bf16_mid", _ptr(x), _ptr(pw.tiles), _ptr(b), _ptr(r), _ptr(out), _code(out.dtype),
+                     _ACT[act], m, n, k, _ptr(space), space.numel(), shares, ahead, _stream())
+            want = exact + (b if b is not None else 0)
+            want = {None: want, "relu": torch.relu(want), "gelu": torch.nn.functional.gelu(want)}[act]
+            want = want + (r if r is not None else 0)
+            tol = dict(rtol=1e-3, atol=1e-3) if wide else dict(rtol=2e-2, atol=2e-2)
+            torch.testing.assert_close(out.float(), want, **tol)
+    # without a workspace the sum over K is not shared out
+    out = torch.empty(m, n, device=DEV)
+    hip.call("gemm", "tnx_gemm_bf16_mid", _ptr(x), _ptr(pw.tiles), None, None, _ptr(out), _code(out.dtype), 0, m, n, k,
+             None, 0, 4, 0, _stream())
+    torch.testing.assert_close(out, exact, rtol=1e-3, atol=1e-3)
+    if m > 32:
+        seen = []
+        inner = hip._call
+        hip._call = lambda module, fn, *a: (seen.append(fn), inner(module, fn, *a))[1]
+        got = hip.linear(x, pw, bias, residual=res, out_f32=True)
+        assert seen == ["tnx_gemm_bf16_mid"]
+        torch.testing.assert_close(got, exact + bias + res, rtol=1e-3, atol=1e-3)
+    with pytest.raises(RuntimeError, match="1 to 128 rows"):
+        hip.call("gemm", "tnx_gemm_bf16_mid", _ptr(x), _ptr(pw.tiles), None, None, _ptr(out), _code(out.dtype), 0, 129,
+                 n, k, None, 0, 0, 0, _stream())

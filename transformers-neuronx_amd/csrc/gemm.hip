@@ -930,6 +930,196 @@ extern "C" int tnx_gemm_bf16_qkv_normed(const float* x, const void* w_folded, co
                             force_tiled, &sc, stream, &nf);
 }
 
+// ------------------------------------------------------------------------------------------ bfloat16, some rows
+//
+// Decode batches beyond the few-rows kernel (33 to 128 rows): the product is still the weight read once, but
+// every block of the few-rows kernel would read all of `x` again, and the vendor library's kernels for such
+// sizes leave much of the memory's rate unused where the output is small and K long (the products that end
+// in the residual sum). Here a block of four waves takes 64 weight rows (each wave a tile of 16, from the
+// tile-ordered copy in runs of 1 KB) and one share of K. Everything comes straight from global memory into
+// LDS, AHEAD steps of 128 before it is used: the rows of `x` once a block, 16-byte chunks swizzled over the
+// 256 bytes of a row, and each wave's weights into a place of its own, where a lane finds the 16 bytes it
+// asked for (row lane % 16, chunk lane / 16 of the tile's step). No load lands in a register, so the only waits are the ones written here, and AHEAD - 1 whole
+// steps stay in flight while one is multiplied. The shares of K (gridDim.y of them, so that the blocks fill
+// the chip also where N is small) leave their float32 partial sums in a workspace [shares][M][N] that a
+// second kernel adds up in a fixed order, with bias, activation and residual; one share alone writes the
+// result itself.
+template <int MT, int AHEAD>
+__global__ void __launch_bounds__(256)
+gemm_bf16_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w_tiles, const float* __restrict__ bias,
+                     const float* __restrict__ residual, void* __restrict__ out, int out_dtype, int act,
+                     float* __restrict__ partial, int M, int N, int K, int steps_per_share) {
+  extern __shared__ __attribute__((aligned(16))) char mid_smem[];
+  constexpr int NST = AHEAD + 1;                    // stages: the step that is multiplied and those in flight
+  constexpr int XSTAGE = 16 * MT * 256;             // bytes of a step's rows of x
+  constexpr int WSTAGE = 4 * 1024;                  // bytes of a step's weights of one wave
+  constexpr int LOADS = MT + 4;                     // loads of a wave a step
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane & 15, g = lane >> 4;
+  const int share = blockIdx.y;
+  const int steps_all = K / 128;
+  const int step0 = share * steps_per_share;
+  const int steps = min(steps_per_share, steps_all - step0);      // at least one: the host cuts no empty share
+  const int last = step0 + steps - 1;
+  const int tile = blockIdx.x * 4 + wave;           // this wave's tile of 16 weight rows
+  const char* wtile = (const char*)(w_tiles + (size_t)min(tile, N / 16 - 1) * 16 * K);
+  // the loads of x: wave-load u of this wave brings rows 4 q .. 4 q + 3 (q = wave + 4 u), 16 lanes a row; the
+  // lane at place p of row m brings chunk p ^ (m % 16), so that fragment reads meet no bank twice
+  unsigned xoff[MT];
+#pragma unroll
+  for (int u = 0; u < MT; ++u) {
+    const int row = 4 * (wave + 4 * u) + (lane >> 4);
+    xoff[u] = (unsigned)(((size_t)min(row, M - 1) * K + (((lane & 15) ^ (row & 15)) * 8)) * 2);
+  }
+  const unsigned x_lds = lds_offset(mid_smem);
+  const unsigned w_lds = x_lds + NST * XSTAGE + wave * NST * WSTAGE;
+  const char* w_mine = mid_smem + NST * XSTAGE + wave * NST * WSTAGE;
+  auto issue = [&](int stage, int step) {
+    const int st = min(step, last);                 // beyond the share: the last step again, into a stage nobody reads
+    const char* xbase = (const char*)(x + (size_t)st * 128);
+#pragma unroll
+    for (int u = 0; u < MT; ++u) load_to_lds(xbase, xoff[u], x_lds + stage * XSTAGE + (wave + 4 * u) * 1024);
+    const char* wbase = wtile + (size_t)st * (128 * 16 * 2);
+#pragma unroll
+    for (int s = 0; s < 4; ++s) load_to_lds(wbase + 1024 * s, (unsigned)((r * 4 + g) * 16), w_lds + stage * WSTAGE + 1024 * s);
+  };
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  auto products = [&](int stage) {
+    const char* xs = mid_smem + stage * XSTAGE;
+    const char* ws = w_mine + stage * WSTAGE + lane * 16;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const bf16x8 wf = *(const bf16x8*)(ws + 1024 * s);
+      bf16x8 xf[MT];
+#pragma unroll
+      for (int t = 0; t < MT; ++t) xf[t] = *(const bf16x8*)(xs + (16 * t + r) * 256 + (((4 * s + g) ^ r) * 16));
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[t], acc[t], 0, 0, 0);
+    }
+  };
+#pragma unroll
+  for (int a = 0; a < AHEAD; ++a) issue(a, step0 + a);
+  for (int i0 = 0; i0 < steps; i0 += NST) {
+#pragma unroll
+    for (int u = 0; u < NST; ++u) {
+      if (i0 + u < steps) {
+        // step i has landed when only the loads of the AHEAD - 1 steps after it are in flight
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((AHEAD - 1) * LOADS) : "memory");
+        __syncthreads();        // its rows of x are there for all; and all have done with the stage of step i - 1,
+        issue((u + AHEAD) % NST, step0 + i0 + u + AHEAD);      // where step i + AHEAD goes
+        products(u);
+      }
+    }
+  }
+  wait_for_loads();             // the loads beyond the last step write to LDS: they end before the block does
+  // acc[t][e] of a lane is row m = 16 t + r of the output at column 16 tile + 4 g + e
+  const int shares = gridDim.y;
+  const int n = 16 * tile + 4 * g;
+  if (n < N) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const int m = 16 * t + r;
+      if (m >= M) continue;
+      if (shares == 1) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) epilogue_store(acc[t][e], m, n + e, N, bias, residual, out, out_dtype, act);
+      } else {
+        *(f32x4*)(partial + ((size_t)share * M + m) * N + n) = acc[t];
+      }
+    }
+  }
+}
+
+// out = act(sum over the shares + bias) + residual, four columns a thread, the shares in their order
+__global__ void __launch_bounds__(256)
+gemm_mid_sum_kernel(const float* __restrict__ partial, const float* __restrict__ bias,
+                    const float* __restrict__ residual, void* __restrict__ out, int out_dtype, int act, int M, int N,
+                    int shares) {
+  const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i >= (size_t)M * N) return;
+  f32x4 v = *(const f32x4*)(partial + i);
+  for (int s = 1; s < shares; ++s) v += *(const f32x4*)(partial + (size_t)s * M * N + i);
+  const int m = (int)(i / N), n = (int)(i % N);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) epilogue_store(v[e], m, n + e, N, bias, residual, out, out_dtype, act);
+}
+
+template <int MT, int AHEAD>
+static int launch_mid(const bf16_t* x, const bf16_t* w_tiles, const float* bias, const float* residual, void* out,
+                      int out_dtype, int act, float* partial, int M, int N, int K, int shares, hipStream_t stream) {
+  constexpr int bytes = (AHEAD + 1) * (16 * MT * 256 + 4 * 4 * 1024);
+  static_assert(bytes <= 160 * 1024, "the stages do not fit the LDS of a compute unit");
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<MT, AHEAD>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) {
+      tnx_set_error("gemm_bf16_mid: cannot reserve %d bytes of LDS: %s", bytes, hipGetErrorString(e));
+      return 2;
+    }
+    configured = true;
+  }
+  const int steps_all = K / 128, per = (steps_all + shares - 1) / shares;
+  const dim3 grid((N / 16 + 3) / 4, (steps_all + per - 1) / per);
+  gemm_bf16_mid_kernel<MT, AHEAD><<<grid, 256, bytes, stream>>>(x, w_tiles, bias, residual, out, out_dtype, act,
+                                                                 partial, M, N, K, per);
+  TNX_CHECK_LAUNCH("gemm_bf16_mid");
+  if (grid.y > 1) {
+    gemm_mid_sum_kernel<<<(unsigned)(((size_t)M * N / 4 + 255) / 256), 256, 0, stream>>>(partial, bias, residual, out,
+                                                                                        out_dtype, act, M, N, grid.y);
+    TNX_CHECK_LAUNCH("gemm_mid_sum");
+  }
+  return 0;
+}
+
+// `shares` 0: chosen here (as many as give every compute unit a block at most, each with four steps of K or more,
+// within the workspace); `ahead` 0: three steps in flight up to 64 rows, two beyond (what LDS holds).
+extern "C" int tnx_gemm_bf16_mid(const void* x, const void* w_tiles, const float* bias, const float* residual,
+                                 void* out, int out_dtype, int act, int M, int N, int K, float* workspace,
+                                 size_t workspace_floats, int shares, int ahead, hipStream_t stream) {
+  TNX_REQUIRE(M > 0 && M <= 128 && N > 0 && K > 0, "gemm_bf16_mid: takes 1 to 128 rows, got M=%d N=%d K=%d", M, N, K);
+  TNX_REQUIRE(N % 16 == 0 && K % 128 == 0, "gemm_bf16_mid: the tile-ordered weight needs N a multiple of 16 and K "
+              "of 128, got N=%d K=%d", N, K);
+  TNX_REQUIRE(x && w_tiles && out && ((uintptr_t)x | (uintptr_t)w_tiles | (uintptr_t)workspace) % 16 == 0,
+              "gemm_bf16_mid: operands must be there and 16-byte aligned");
+  TNX_REQUIRE(out_dtype == TNX_F32 || out_dtype == TNX_BF16, "gemm_bf16_mid: the result is float32 or bfloat16");
+  TNX_REQUIRE(shares >= 0 && ahead >= 0 && ahead <= 4, "gemm_bf16_mid: bad shares or steps ahead");
+  const int blocks_n = (N / 16 + 3) / 4, steps_all = K / 128;
+  if (shares == 0) {
+    // a block a compute unit at most: blocks of one length in a ragged second round cost more than idle units
+    shares = tnx_compute_units() / blocks_n;
+    shares = max(1, min(shares, steps_all / 4));
+  }
+  shares = max(1, min(shares, steps_all));
+  if (shares > 1) {
+    const size_t room = workspace ? workspace_floats / ((size_t)M * N) : 0;
+    if ((size_t)shares > room) shares = (int)max((size_t)1, room);
+  }
+  const bf16_t* xp = (const bf16_t*)x;
+  const bf16_t* wp = (const bf16_t*)w_tiles;
+  const int mt = (M + 15) / 16;
+  if (ahead == 0) ahead = mt <= 4 ? 3 : 2;
+  if (mt > 4 && ahead > 2) ahead = 2;               // what LDS holds
+#define MID(MT, A) launch_mid<MT, A>(xp, wp, bias, residual, out, out_dtype, act, workspace, M, N, K, shares, stream)
+#define MID_LOW(MT) return ahead == 1 ? MID(MT, 1) : ahead == 2 ? MID(MT, 2) : ahead == 3 ? MID(MT, 3) : MID(MT, 4)
+#define MID_HIGH(MT) return ahead == 1 ? MID(MT, 1) : MID(MT, 2)
+  switch (mt) {
+    case 1: MID_LOW(1);
+    case 2: MID_LOW(2);
+    case 3: MID_LOW(3);
+    case 4: MID_LOW(4);
+    case 5: MID_HIGH(5);
+    case 6: MID_HIGH(6);
+    case 7: MID_HIGH(7);
+    default: MID_HIGH(8);
+  }
+#undef MID_HIGH
+#undef MID_LOW
+#undef MID
+}
+
 // ------------------------------------------------------------------------------------- the vendor library
 //
 // out = act(x w^T + bias) + residual for many rows, as one call of hipBLASLt: bfloat16 operands, float32 sums,
