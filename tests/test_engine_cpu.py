@@ -294,6 +294,13 @@ def test_entry_point_in_the_reference_manner(tiny_folders, tmp_path):
     padded = torch.tensor([[1, 1, 5, 9], [7, 7, 100, 3]])
     logits = model(padded, None, torch.tensor([2, 0]))
     torch.testing.assert_close(logits[0], plain_opt.forward_logits(weights, cfg, [5, 9])[-1], atol=1e-5, rtol=1e-5)
+    # every position's logits (`output_all_logits`, config.py:91): `[batch, tokens, vocab]`, zeros under the padding
+    model.neuron_config.output_all_logits = True
+    logits = model(padded, None, torch.tensor([2, 0]))
+    assert logits.shape == (2, 4, cfg["vocab_size"]) and not logits[0, :2].any()
+    torch.testing.assert_close(logits[0, 2:], plain_opt.forward_logits(weights, cfg, [5, 9]), atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(logits[1], plain_opt.forward_logits(weights, cfg, [7, 7, 100, 3]), atol=1e-5, rtol=1e-5)
+    model.neuron_config.output_all_logits = False
     model.reset()
     assert not model.engine.runner.cache.requests
     # a streamer gets one token of every row at a time and is told the end (sampling.py:159-160, :172-173),

@@ -149,7 +149,7 @@ class CausalLMForSampling:
     @torch.no_grad()
     def forward(self, input_ids, cache_ids=None, start_ids=None) -> torch.Tensor:
         """Logits `[batch, vocab]` of each row's last token (`[batch, tokens, vocab]` with
-        `output_all_logits`). `cache_ids=None` starts the rows afresh with `input_ids`
+        `output_all_logits`, zeros where a row is padded). `cache_ids=None` starts the rows afresh with `input_ids`
         as their prompts; otherwise the tokens go on from where the rows are, and
         `cache_ids` must say so (reference: opt/model.py:158-184; rows left-padded up
         to `start_ids` lose their padding here instead of masking it)."""
@@ -173,7 +173,14 @@ class CausalLMForSampling:
                    for b, toks in enumerate(rows)]
         logits = runner.step(entries)
         if every:
-            return logits.view(len(rows), -1, logits.shape[-1])
+            # `[batch, tokens, vocab]` over the width given; the places of a row's padding hold zeros
+            width = max(len(toks) for toks in rows) if start_ids is None else torch.as_tensor(input_ids).shape[-1]
+            out = logits.new_zeros(len(rows), width, logits.shape[-1])
+            at = 0
+            for b, toks in enumerate(rows):
+                out[b, width - len(toks):] = logits[at:at + len(toks)]
+                at += len(toks)
+            return out
         return logits
 
     def _forward_sequences(self, input_ids, cache_ids, seq_ids) -> torch.Tensor:
