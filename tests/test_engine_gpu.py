@@ -352,6 +352,15 @@ def test_full_layer_sizes_against_plain(size):
     plan = [[("a", 0, 300, [299])], [("a", 300, 110, [0, 109])], [("a", 410, 1, [0]), ("b", 0, 30, [29])]]
     plan += [[("a", 411 + i, 1, [0]), ("b", 30 + i, 1, [0])] for i in range(9)]
     toks = {"a": long, "b": short}
+    # decode batches of every class of row counts: 40 requests (the products of 33 to 128 rows), 20 (the norm's
+    # own kernel in front of the folded copies), 9 and 8 (the norm inside the product)
+    crowd = [f"c{i}" for i in range(40)]
+    for i, rid in enumerate(crowd):
+        toks[rid] = torch.randint(3, cfg.vocab_size, (4 + i % 3 + 4,), generator=g).tolist()
+    plan.append([(rid, 0, len(toks[rid]) - 4, [len(toks[rid]) - 5]) for rid in crowd])
+    for k, live in enumerate((40, 20, 9, 8)):
+        plan.append([(rid, len(toks[rid]) - 4 + k, 1, [0]) for rid in crowd[:live]])
+    recorded = sum(all(n == 1 and w == [0] for _, _, n, w in step) for step in plan)
     # the plain implementation: each request whole, then the head on the wanted positions only
     weights = {k: v.float().cpu() for k, v in tensors.items()}
     hidden = {}
@@ -366,13 +375,13 @@ def test_full_layer_sizes_against_plain(size):
     top2 = want.topk(2, dim=-1).values
 
     def run(dtype):
-        ecfg = EngineConfig(dtype=dtype, page_size=64, max_tokens=1024, max_num_seqs=4)
+        ecfg = EngineConfig(dtype=dtype, page_size=64, max_tokens=1024 + 64 * len(crowd), max_num_seqs=2 + len(crowd))
         runner = build_runner(cfg, TensorDict(tensors), ecfg)
         rows = []
         for step in plan:
             rows.append(runner.step([StepEntry(rid, toks[rid][first:first + n], w) for rid, first, n, w in step])
                         .float().cpu())
-        assert runner.graph_replays == 9
+        assert runner.graph_replays == recorded == 13
         return torch.cat(rows)
 
     for dtype in ("float32", "bfloat16"):
