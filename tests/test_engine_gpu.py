@@ -534,3 +534,35 @@ def test_drawn_configurations_and_schedules(tmp_path, seed):
     expected = _expected(weights, raw, requests)
     out, _ = _run(folder, dtype, steps, max_tokens, page, tmp_path, "drawn")
     _compare(out, place, expected, raw["vocab_size"], dtype)
+
+
+def test_command_line_options_of_the_reference(tiny_folders, capsys):
+    """`opt_demo run` with the options of the reference's demos that mean something on one GPU: rows of
+    different lengths (`--various`), an end-of-sequence token of the caller's, the accepted no-ops; and
+    `--quantize`, which is refused."""
+    import re
+    from transformers_neuronx_amd.opt import demo
+    folder, cfg, weights = tiny_folders["A"]
+    base = ["--amp", "f32", "run", folder, "--batch_size", "3", "--n_positions", "20", "--prompt_len", "6",
+            "--top_k", "1", "--unroll", "4", "--context_length_estimate", "16", "--continuous_batching"]
+
+    def generated(extra):
+        demo.main(base + extra)
+        text = capsys.readouterr().out
+        rows = re.findall(r"\[([\d,\s]+)\]", text[text.index("generated_sequence="):])
+        return [[int(t) for t in r.replace(",", " ").split()] for r in rows]
+    rows = generated(["--various", "--simple_sample_eos_token_override", "-1"])
+    assert len(rows) == 3 and all(len(r) == 20 for r in rows)
+    pad = cfg.get("pad_token_id", 1)
+    for b, row in enumerate(rows):
+        start = (b * 2) % 6
+        assert row[:start] == [pad] * start
+        want = plain_opt.greedy(weights, cfg, row[start:6], 14)      # nothing banned, nothing stops it
+        assert row[start:] == want, (b, row, want)
+    # a token the first row is known to generate ends that row: what follows is that token again
+    stop = rows[0][9]
+    again = generated(["--various", "--simple_sample_eos_token_override", str(stop)])
+    first = rows[0].index(stop, 6)
+    assert again[0][:first + 1] == rows[0][:first + 1] and set(again[0][first:]) == {stop}
+    with pytest.raises(SystemExit, match="quantize"):
+        demo.main(base + ["--quantize"])

@@ -44,6 +44,16 @@ def _parser():
     run.add_argument("--n_positions", type=int, default=128, help="Input sequence length")
     run.add_argument("--tp_degree", type=int, default=1, help="must be 1: one GPU")
     run.add_argument("--print_latency", action="store_true", help="Print latency of each step")
+    # gpt_demo.py:53, :55, :66 and generation_demo.py:245-262: taken where they mean something on one GPU
+    run.add_argument("--unroll", type=int, default=None, help="accepted; nothing is unrolled here")
+    run.add_argument("--context_length_estimate", type=int, default=None, help="accepted; prompts are not bucketed here")
+    run.add_argument("--quantize", action="store_true", help="refused: weights stay in the dtype of --amp")
+    run.add_argument("--continuous_batching", action="store_true",
+                     help="accepted: requests are batched continuously whether it is given or not")
+    run.add_argument("--various", action="store_true",
+                     help="Generated batched sequence with different length if set; otherwise using same length")
+    run.add_argument("--simple_sample_eos_token_override", type=int, default=None,
+                     help="override eos token, set to -1 to always generate exactly as many tokens as asked for")
     run.add_argument("--prompt_len", type=int, default=None, help="random token ids of this length as the prompt")
     run.add_argument("--prompt_ids", type=str, default=None, help="comma-separated token ids of the prompt")
     run.add_argument("--do_sample", action="store_true")
@@ -79,10 +89,13 @@ def save(args):
 def run(args):
     from ..config.engine_config import GenerationConfig
     from .model import OPTForSampling
+    if args.quantize:
+        raise SystemExit("run: --quantize is not to be had here: weights stay in the dtype of --amp")
     torch.manual_seed(args.seed)
     print("running OPTForSampling.from_pretrained")
     model = OPTForSampling.from_pretrained(args.load, batch_size=args.batch_size, amp=args.amp,
                                            tp_degree=args.tp_degree, n_positions=args.n_positions,
+                                           unroll=args.unroll, context_length_estimate=args.context_length_estimate,
                                            page_size=args.page_size)
     print("running model.load")
     model.load()
@@ -93,6 +106,14 @@ def run(args):
     else:
         n = args.prompt_len or 8
         input_ids = torch.randint(3, vocab, (args.batch_size, n))
+    start_ids = None
+    if args.various and args.batch_size > 1:
+        # rows of different lengths, padded on the left up to `start_ids` (generation_demo.py:262; the padding
+        # is the pad token and is dropped before the rows reach the engine)
+        width = input_ids.shape[1]
+        start_ids = torch.tensor([(b * max(1, width // args.batch_size)) % width for b in range(args.batch_size)])
+        for b in range(args.batch_size):
+            input_ids[b, :int(start_ids[b])] = getattr(model.config, "pad_token_id", 1)
     total = args.n_positions
     if args.max_new_tokens is not None:
         total = min(total, input_ids.shape[1] + args.max_new_tokens)
@@ -101,6 +122,11 @@ def run(args):
     gen = None
     if args.do_sample:
         gen = GenerationConfig(do_sample=True, top_k=args.top_k, top_p=args.top_p, temperature=args.temperature)
+    if args.simple_sample_eos_token_override is not None:
+        # the generation stops at this token (generation_demo.py:245); -1 is no token's id: it never stops early
+        eos = args.simple_sample_eos_token_override
+        gen = gen or GenerationConfig(do_sample=False, top_k=1)
+        gen.eos_token_id = eos if eos >= 0 else None
     dumped = []
     if args.dump_logits:
         # generation_demo.py:694-702 writes the scores of the first `dump_logits_limit` generated tokens
@@ -116,8 +142,8 @@ def run(args):
     print("running model.sample")
 
     def generate():
-        return model.sample(input_ids, sequence_length=total, top_k=args.top_k, temperature=args.temperature,
-                            top_p=args.top_p, seed=args.seed, generation_config=gen)
+        return model.sample(input_ids, sequence_length=total, start_ids=start_ids, top_k=args.top_k,
+                            temperature=args.temperature, top_p=args.top_p, seed=args.seed, generation_config=gen)
     out = generate()
     print("generated_sequence=", out)
     for i, logits in enumerate(dumped):
