@@ -13,6 +13,9 @@ def __getattr__(name):
     if name == "NeuronAutoModelForCausalLM":
         from .modeling_auto import NeuronAutoModelForCausalLM
         return NeuronAutoModelForCausalLM
+    if name == "testing":
+        import importlib
+        return importlib.import_module(".testing", __name__)
     if name == "LLMEngine":
         from .engine.engine import LLMEngine
         return LLMEngine
