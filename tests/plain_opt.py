@@ -229,6 +229,20 @@ def sample_row(scores, u, top_k=None, top_p=None, temperature=1.0, min_tokens_to
     return int(indices[min(pick, len(indices) - 1)])
 
 
+def banned_by_ngrams(tokens, n):
+    """sampling.py:267-300 for one row: every run of `n` tokens in `tokens` is filed under its first n - 1
+    (:275-277); with fewer than n - 1 tokens nothing is banned (:292-294); otherwise the tokens filed under
+    the last n - 1 (:284-286) may not come next."""
+    tokens = list(tokens)
+    if len(tokens) + 1 < n:
+        return []
+    filed = {}
+    for start in range(len(tokens) - n + 1):
+        run = tokens[start:start + n]
+        filed.setdefault(tuple(run[:-1]), []).append(run[-1])
+    return filed.get(tuple(tokens[len(tokens) + 1 - n:]), [])
+
+
 def philox_uniform(seed, counter):
     """Philox-4x32-10 (Salmon et al., 2011, public algorithm) keyed by the
     request's seed, counter = the request's step; first output word mapped to

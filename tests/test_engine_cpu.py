@@ -549,3 +549,54 @@ def test_a_step_planner_of_the_tests_rides_in_the_steps_integers(tiny_folders):
     runner, _ = _runner(folder, 128)
     runner.step([StepEntry("a", toks["r0"], [0])])
     assert "toy_even_runs" not in runner._last_ctx.plan
+
+
+def _plain_without_repeats(weights, cfg, prompt, n_new, size, banned_token=None):
+    toks = list(prompt)
+    for _ in range(n_new):
+        row = plain_opt.forward_logits(weights, cfg, toks)[-1].clone()
+        if banned_token is not None:
+            row[banned_token] = float("-inf")
+        row[plain_opt.banned_by_ngrams(toks, size)] = float("-inf")
+        toks.append(int(row.argmax()))
+    return toks[len(prompt):]
+
+
+@pytest.mark.parametrize("run_ahead", [False, True])
+def test_no_run_of_tokens_twice(tiny_folders, run_ahead):
+    """`no_repeat_ngram_size` (sampling.py:267-309): the greedy path of the narrow-weights model repeats one
+    token; with the ban no run of n tokens comes twice, the tokens are the plain implementation's under the same
+    ban, requests with and without it share steps, and a request put back and computed again keeps its path."""
+    folder, cfg, weights = tiny_folders["A"]
+    runner, ecfg = _runner(folder, max_tokens=64, run_ahead=run_ahead)
+    engine = LLMEngine(runner, ecfg)
+    prompts = [[5, 9, 200, 31, 9, 200], [7, 7, 100, 3], [11, 12]]
+    sizes = [2, 3, 0]
+    params = [SamplingParams(max_new_tokens=20, do_sample=False, ignore_eos=True, no_repeat_ngram_size=n) for n in sizes]
+    outs = engine.generate(prompts, params)
+    assert engine.scheduler.num_preemptions > 0            # four pages of 16 for three requests of up to 26 tokens
+    for prompt, out, n in zip(prompts, outs, sizes):
+        want = _plain_without_repeats(weights, cfg, prompt, 20, n) if n else plain_opt.greedy(weights, cfg, prompt, 20)[len(prompt):]
+        assert out == want, (n, out, want)
+        if n:
+            whole = prompt + out
+            runs = [tuple(whole[i:i + n]) for i in range(len(prompt) - n + 1, len(whole) - n + 1)]
+            seen = {tuple(whole[i:i + n]) for i in range(len(prompt) - n + 1)}
+            for r in runs:
+                assert r not in seen, r
+                seen.add(r)
+    assert len(set(outs[2])) < 4                           # the row without the ban does repeat itself
+    with pytest.raises(ValueError, match="strictly positive integer"):
+        SamplingParams(no_repeat_ngram_size=-2)
+
+
+def test_sample_takes_the_ngram_ban(tiny_folders):
+    from transformers_neuronx_amd import OPTForSampling
+    folder, cfg, weights = tiny_folders["A"]
+    model = OPTForSampling.from_pretrained(folder, batch_size=2, amp="f32", n_positions=32, kernels="reference",
+                                           device="cpu", page_size=16).to_neuron()
+    ids = torch.tensor([[5, 9, 200, 31], [7, 7, 100, 3]])
+    out = model.sample(ids, sequence_length=16, top_k=1, no_repeat_ngram_size=2)
+    eos = cfg.get("eos_token_id", 2)
+    for b in range(2):
+        assert out[b, 4:].tolist() == _plain_without_repeats(weights, cfg, ids[b].tolist(), 12, 2, banned_token=eos)

@@ -163,3 +163,33 @@ def test_generation_with_few_pages_bfloat16(tiny_folders_bf16, name):
             for pos in range(len(prompt) - 1, len(toks) - 1):
                 row = logits[pos]
                 assert float(row.max() - row[toks[pos + 1]]) <= 3e-2 * float(row.abs().max()), (pos, toks[pos + 1])
+
+
+def test_no_run_of_tokens_twice_on_the_gpu(tiny_folders):
+    """`no_repeat_ngram_size` through the HIP sampler's ban of (row, token) pairs, beside requests without it,
+    with few pages and recorded decode steps: the plain implementation's tokens under the same ban."""
+    from transformers_neuronx_amd.sampling import SamplingParams
+    folder, cfg, weights = tiny_folders["A"]
+    prompts = _prompts(cfg["vocab_size"], [6, 17, 3], 8)
+    sizes = [2, 0, 3]
+    params = [SamplingParams(max_new_tokens=24, do_sample=False, ignore_eos=True, no_repeat_ngram_size=n) for n in sizes]
+    engine, runner = _engine(folder, "float32", page_size=16, max_tokens=80, max_num_seqs=4, use_graphs=True)
+    outs = engine.generate(prompts, params)
+    runner.cache.check()
+    assert engine.scheduler.num_preemptions > 0
+    for prompt, out, n in zip(prompts, outs, sizes):
+        toks = list(prompt)
+        for _ in range(24):
+            row = plain_opt.forward_logits(weights, cfg, toks)[-1].clone()
+            if n:
+                row[plain_opt.banned_by_ngrams(toks, n)] = float("-inf")
+            toks.append(int(row.argmax()))
+        assert out == toks[len(prompt):], (n, out, toks[len(prompt):])
+    # the kernel alone: pairs out of range touch nothing
+    from transformers_neuronx_amd.kernels.hip import HipOps
+    ops = HipOps(torch.float32, DEV)
+    logits = torch.zeros(3, 10, device=DEV)
+    rows = torch.tensor([0, 2, 2, 5, 1], dtype=torch.int32, device=DEV)
+    toks = torch.tensor([4, 0, 9, 1, 10], dtype=torch.int32, device=DEV)
+    ops.ban_pairs(logits, rows, toks)
+    assert torch.isinf(logits).nonzero().tolist() == [[0, 4], [2, 0], [2, 9]]

@@ -279,3 +279,20 @@ def test_pre_norm_head_norms_the_stream_once():
                                               w["model.decoder.final_layer_norm.bias"], 1e-5),
                w["model.decoder.embed_tokens.weight"])
     torch.testing.assert_close(plain_opt.forward_logits(wz, cfg, toks.tolist()), want, rtol=1e-5, atol=1e-5)
+
+
+def test_ngram_ban_by_hand():
+    """What pins it beside the reference's text: cases small enough to read. After `1 2 3 1 2` a 3 would
+    repeat `1 2 3`; with n = 2 every token that ever followed a 2; with n = 1 every token seen; a sequence
+    shorter than n - 1 bans nothing; and the product's own function says the same on random rows."""
+    from transformers_neuronx_amd.sampling.sampler import banned_ngram_tokens
+    assert plain_opt.banned_by_ngrams([1, 2, 3, 1, 2], 3) == [3]
+    assert plain_opt.banned_by_ngrams([1, 2, 3, 1, 2, 4, 2], 2) == [3, 4]
+    assert sorted(set(plain_opt.banned_by_ngrams([5, 6, 5], 1))) == [5, 6]
+    assert plain_opt.banned_by_ngrams([7], 3) == [] and plain_opt.banned_by_ngrams([7, 8], 3) == []
+    assert plain_opt.banned_by_ngrams([7, 8, 9], 4) == []           # the one run of four would need a fourth token
+    g = torch.Generator().manual_seed(0)
+    for n in (1, 2, 3, 4):
+        for _ in range(50):
+            row = torch.randint(0, 4, (int(torch.randint(0, 30, (1,), generator=g)),), generator=g).tolist()
+            assert sorted(banned_ngram_tokens(row, n)) == sorted(plain_opt.banned_by_ngrams(row, n)), (row, n)

@@ -219,12 +219,15 @@ class CausalLMForSampling:
     @torch.no_grad()
     def sample(self, input_ids, sequence_length: int, start_ids=None, top_k: int = 50, streamer=None,
                temperature: float = 1.0, top_p: float = 1.0, seed: int = 0,
-               generation_config: Optional[GenerationConfig] = None) -> torch.Tensor:
+               generation_config: Optional[GenerationConfig] = None,
+               no_repeat_ngram_size: Optional[int] = None) -> torch.Tensor:
         """`[batch, sequence_length]`: the prompts and what follows them, up to a total
         length of `sequence_length`. As the reference's loop (sampling.py:131-180) it
         never picks the end-of-sequence token and keeps the `top_k` largest logits;
         `top_k=1` is greedy. With `on_device_generation` in the NeuronConfig, or a
-        `generation_config`, those options decide instead (sampling.py:33-105)."""
+        `generation_config`, those options decide instead (sampling.py:33-105).
+        `no_repeat_ngram_size`: no run of that many tokens appears twice in a row's prompt and what
+        follows it (the option of the reference's other loop, sampling.py:382-394)."""
         engine = self._need_engine()
         rows = self._rows(input_ids, start_ids)
         gen = generation_config or self.neuron_config.on_device_generation
@@ -249,11 +252,12 @@ class CausalLMForSampling:
                 p = SamplingParams(max_new_tokens=new, do_sample=gen.do_sample, temperature=float(line(gen.temperature)),
                                    top_k=k, top_p=float(line(gen.top_p)), seed=seed + b,
                                    min_tokens_to_keep=int(line(gen.top_p_min_tokens)), deterministic=gen.deterministic,
-                                   eos_token_id=gen.eos_token_id, ignore_eos=gen.eos_token_id is None)
+                                   eos_token_id=gen.eos_token_id, ignore_eos=gen.eos_token_id is None,
+                                   no_repeat_ngram_size=int(no_repeat_ngram_size or 0))
             else:
                 p = SamplingParams(max_new_tokens=new, do_sample=True, temperature=temperature, top_k=top_k,
                                    top_p=top_p, seed=seed + b, eos_token_id=getattr(self.config, 'eos_token_id', None),
-                                   ban_eos=True, ignore_eos=True)
+                                   ban_eos=True, ignore_eos=True, no_repeat_ngram_size=int(no_repeat_ngram_size or 0))
             params.append(p)
         engine.reset()
         ids = [engine.add_request(toks, p) for toks, p in zip(rows, params)]

@@ -108,6 +108,25 @@ __global__ void ban_tokens_kernel(float* __restrict__ logits, const int* __restr
   if (r < rows && token[r] >= 0 && token[r] < vocab) logits[(size_t)r * vocab + token[r]] = -INFINITY;
 }
 
+// logits[rows[i], tokens[i]] = -inf for a list of (row, token) pairs: tokens that must not follow what a
+// request has generated (the n-grams it may not repeat).
+__global__ void ban_pairs_kernel(float* __restrict__ logits, const int* __restrict__ rows,
+                                 const int* __restrict__ tokens, int n, int num_rows, int vocab) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int r = rows[i], t = tokens[i];
+  if (r >= 0 && r < num_rows && t >= 0 && t < vocab) logits[(size_t)r * vocab + t] = -INFINITY;
+}
+
+extern "C" int tnx_ban_pairs(float* logits, const int* rows, const int* tokens, int n, int num_rows, int vocab,
+                             hipStream_t stream) {
+  TNX_REQUIRE(n >= 0 && num_rows >= 0 && vocab > 0, "ban_pairs: bad sizes n=%d rows=%d vocab=%d", n, num_rows, vocab);
+  if (n == 0) return 0;
+  ban_pairs_kernel<<<(n + 255) / 256, 256, 0, stream>>>(logits, rows, tokens, n, num_rows, vocab);
+  TNX_CHECK_LAUNCH("ban_pairs");
+  return 0;
+}
+
 extern "C" int tnx_ban_tokens(float* logits, const int* token, int rows, int vocab, hipStream_t stream) {
   TNX_REQUIRE(rows >= 0 && vocab > 0, "ban_tokens: bad sizes rows=%d vocab=%d", rows, vocab);
   if (rows == 0) return 0;

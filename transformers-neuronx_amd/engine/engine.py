@@ -107,7 +107,13 @@ class LLMEngine:
             requests = [r.request for r in sampling]
             if self.logits_hook is not None:
                 self.logits_hook(requests, logits)
-            drawn = self.sampler.draw(logits, [q.params for q in requests], [len(q.output) for q in requests])
+            histories = None
+            if any(q.params.no_repeat_ngram_size for q in requests):
+                # (such requests never run ahead, see `step`: every token they hold is known here)
+                histories = [list(q.prompt) + list(q.output) if q.params.no_repeat_ngram_size else None
+                             for q in requests]
+            drawn = self.sampler.draw(logits, [q.params for q in requests], [len(q.output) for q in requests],
+                                      histories)
             sent = self.runner.keep_tokens(drawn)
         self.scheduler.record(runs)
         return _StartedStep(runs, sampling, sent, t0)
@@ -138,7 +144,9 @@ class LLMEngine:
     def step(self) -> List[StepOutput]:
         """Schedule, run, sample, record: one batch of portions and decoded tokens. Returns the tokens of
         the step it ran, or with `run_ahead` those of the step started by the call before."""
-        if not self.run_ahead or self.record_timings:
+        # a request that may not repeat its n-grams needs its last token on the host before the next is chosen
+        in_step = any(q.params.no_repeat_ngram_size and not q.finished for q in self.requests.values())
+        if not self.run_ahead or self.record_timings or in_step:
             out = self._finish(self._started) if self._started is not None else []
             self._started = None
             started = self._start()

@@ -68,6 +68,7 @@ _SIGNATURES = {
     },
     "sampling": {
         "tnx_ban_tokens": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+        "tnx_ban_pairs": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
         "tnx_store_tokens": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p,
                              _c_void_p],
@@ -795,6 +796,15 @@ class HipOps:
         _want(tokens, "tokens", torch.int32, (logits.shape[0],))
         self._call("sampling", "tnx_ban_tokens", _ptr(logits), _ptr(tokens), logits.shape[0], logits.shape[1],
                    _stream())
+        return logits
+
+    def ban_pairs(self, logits, rows, tokens):
+        """In place: `logits[rows[i], tokens[i]] = -inf` for every pair."""
+        _want(logits, "logits", torch.float32)
+        _want(rows, "rows", torch.int32)
+        _want(tokens, "tokens", torch.int32, (rows.numel(),))
+        self._call("sampling", "tnx_ban_pairs", _ptr(logits), _ptr(rows), _ptr(tokens), rows.numel(), logits.shape[0],
+                   logits.shape[1], _stream())
         return logits
 
     def argmax(self, logits):

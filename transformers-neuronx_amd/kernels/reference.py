@@ -189,6 +189,10 @@ class ReferenceOps:
         logits[rows, tokens[rows].long()] = float("-inf")
         return logits
 
+    def ban_pairs(self, logits, rows, tokens):
+        logits[rows.long(), tokens.long()] = float("-inf")
+        return logits
+
     def argmax(self, logits):
         return logits.argmax(dim=-1).to(torch.int32)
 

@@ -60,6 +60,7 @@ def _parser():
     run.add_argument("--top_k", type=int, default=50)
     run.add_argument("--top_p", type=float, default=1.0)
     run.add_argument("--temperature", type=float, default=1.0)
+    run.add_argument("--no_repeat_ngram_size", type=int, default=0)
     run.add_argument("--max_new_tokens", type=int, default=None)
     run.add_argument("--max_length", type=int, default=None)
     run.add_argument("--seed", type=int, default=15213)
@@ -143,7 +144,8 @@ def run(args):
 
     def generate():
         return model.sample(input_ids, sequence_length=total, start_ids=start_ids, top_k=args.top_k,
-                            temperature=args.temperature, top_p=args.top_p, seed=args.seed, generation_config=gen)
+                            temperature=args.temperature, top_p=args.top_p, seed=args.seed, generation_config=gen,
+                            no_repeat_ngram_size=args.no_repeat_ngram_size)
     out = generate()
     print("generated_sequence=", out)
     for i, logits in enumerate(dumped):

@@ -23,6 +23,9 @@ class SamplingParams:
     ban_eos      the end-of-sequence token is never chosen (`scores[:, eos] = -inf`,
                  sampling.py:143-144, the OPT loop's behaviour)
     ignore_eos   generation does not stop at the end-of-sequence token
+    no_repeat_ngram_size  n: no run of n tokens appears twice in the prompt and what follows it; a token
+                 that would complete a run seen before gets the logit -inf before anything else is done
+                 (sampling.py:267-309, :334-335); 0 switches it off
     max_new_tokens  the most tokens to generate
     """
     max_new_tokens: int = 16
@@ -36,6 +39,7 @@ class SamplingParams:
     eos_token_id: Optional[int] = None
     ban_eos: bool = False
     ignore_eos: bool = False
+    no_repeat_ngram_size: int = 0
 
     def __post_init__(self):
         if self.max_new_tokens < 0:
@@ -46,6 +50,8 @@ class SamplingParams:
             raise ValueError("top_p has to be a strictly positive float that less than or equal to 1.0.")
         if not isinstance(self.min_tokens_to_keep, int) or self.min_tokens_to_keep < 1:
             raise ValueError("min_tokens_to_keep has to be a positive int.")
+        if self.no_repeat_ngram_size and (not isinstance(self.no_repeat_ngram_size, int) or self.no_repeat_ngram_size <= 0):
+            raise ValueError(f"`ngram_size` has to be a strictly positive integer, but is {self.no_repeat_ngram_size}")
         if float(self.temperature) < 0:
             raise ValueError("temperature has to be a non-negative float (0 is greedy).")
 

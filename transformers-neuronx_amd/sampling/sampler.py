@@ -1,10 +1,19 @@
 """From logits rows to tokens, one kernel launch for the batch."""
-from typing import List
+from typing import List, Optional, Sequence
 
 import numpy as np
 import torch
 
 from .params import SamplingParams
+
+
+def banned_ngram_tokens(history: Sequence[int], n: int) -> List[int]:
+    """The tokens that would, after `history`, complete a run of `n` tokens that `history` already holds
+    (reference: sampling.py:267-300; with n = 1 every token seen so far)."""
+    if n <= 0 or len(history) + 1 < n:
+        return []
+    tail = list(history[len(history) - (n - 1):]) if n > 1 else []
+    return [history[i + n - 1] for i in range(len(history) - n + 1) if list(history[i:i + n - 1]) == tail]
 
 
 class Sampler:
@@ -15,15 +24,32 @@ class Sampler:
     def __init__(self, ops, device):
         self.ops, self.device = ops, device
 
-    def __call__(self, logits: torch.Tensor, params: List[SamplingParams], draws: List[int]) -> List[int]:
-        return self.draw(logits, params, draws).tolist()
+    def __call__(self, logits: torch.Tensor, params: List[SamplingParams], draws: List[int],
+                 histories: Optional[List[Sequence[int]]] = None) -> List[int]:
+        return self.draw(logits, params, draws, histories).tolist()
 
-    def draw(self, logits: torch.Tensor, params: List[SamplingParams], draws: List[int]) -> torch.Tensor:
+    def draw(self, logits: torch.Tensor, params: List[SamplingParams], draws: List[int],
+             histories: Optional[List[Sequence[int]]] = None) -> torch.Tensor:
         """The chosen tokens, int32 on the logits' device; nothing waits for the device here.
-        `draws[i]` is how many tokens request i has drawn before: the counter of its stream."""
+        `draws[i]` is how many tokens request i has drawn before: the counter of its stream.
+        `histories[i]`: the tokens request i holds so far, prompt and all (asked for where a request
+        has `no_repeat_ngram_size`)."""
         m = logits.shape[0]
         if m != len(params):
             raise ValueError(f"{m} logits rows for {len(params)} requests")
+        pairs = []
+        for i, p in enumerate(params):
+            if p.no_repeat_ngram_size:
+                if histories is None or histories[i] is None:
+                    raise ValueError("no_repeat_ngram_size needs the tokens a request holds so far")
+                pairs += [(i, t) for t in banned_ngram_tokens(histories[i], p.no_repeat_ngram_size)]
+        if pairs:
+            flat = np.array(pairs, dtype=np.int32).T.copy()            # rows, then tokens
+            if hasattr(self.ops, "send_ints"):
+                dev = self.ops.send_ints(flat.reshape(-1))
+            else:
+                dev = torch.from_numpy(flat.reshape(-1)).to(self.device)
+            self.ops.ban_pairs(logits, dev[:len(pairs)], dev[len(pairs):])
         banned = [p.eos_token_id if (p.ban_eos and p.eos_token_id is not None) else -1 for p in params]
         if any(b >= 0 for b in banned):
             if hasattr(self.ops, "send_ints"):
