@@ -549,7 +549,9 @@ class HipOps:
     @classmethod
     def _library_workspace(cls, device) -> torch.Tensor:
         """Memory the library's algorithms may ask for (those that split the inner dimension over blocks keep
-        partial sums there), one block per device, made at the first product and kept."""
+        partial sums there, as does our kernel for some rows), one block per device, made at the first product
+        and kept. Products on different streams of one device would share it: the engine runs its steps on
+        one stream."""
         key = str(device)
         if key not in cls._workspaces:
             cls._workspaces[key] = torch.empty(32 << 20, dtype=torch.uint8, device=device)
