@@ -122,7 +122,9 @@ def main():
     runner = runner_from_random(cfg, seed=0, cfg=ecfg)
     torch.cuda.synchronize()
     print(f"[bench] model ready in {time.time() - t0:.1f} s "
-          f"({runner.model.weight_bytes / 1e9:.2f} GB of weights)", file=sys.stderr, flush=True)
+          f"({runner.model.weight_bytes / 1e9:.2f} GB of weights"
+          + (f", {runner.ops.copy_bytes / 1e9:.1f} GB of them a second time in tile order" if getattr(runner.ops, "copy_bytes", None) is not None else "")
+          + ")", file=sys.stderr, flush=True)
     engine = LLMEngine(runner, ecfg)
     gen = torch.Generator().manual_seed(1)
 

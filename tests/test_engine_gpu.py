@@ -566,3 +566,39 @@ def test_command_line_options_of_the_reference(tiny_folders, capsys):
     assert again[0][:first + 1] == rows[0][:first + 1] and set(again[0][first:]) == {stop}
     with pytest.raises(SystemExit, match="quantize"):
         demo.main(base + ["--quantize"])
+
+
+def test_weight_copies_within_a_number_of_bytes(tiny_folders_bf16, tmp_path):
+    """A model whose tile-ordered copies do not all fit gets those a number of bytes allows, the matrices with
+    the fewest rows first, and the LayerNorm is folded into those that got one: the logits are the same
+    with none, with some and with all."""
+    from transformers_neuronx_amd.config import EngineConfig
+    from transformers_neuronx_amd.engine.factory import runner_from_folder
+    from transformers_neuronx_amd.kernels.hip import PreparedWeight
+    folder, cfg, weights = tiny_folders_bf16["C"]        # width 128, inner width 256: every matrix can have a copy
+    requests = _requests(cfg, [40, 9], seed=2)
+    expected = _expected(weights, cfg, requests)
+    steps, place = schedules.head_then_singles(requests, tail=6)
+    seen = {}
+    for name, kw in (("none", dict(weight_copies=False)), ("all", dict(weight_copies=True)),
+                     ("some", dict(weight_copy_bytes=224 << 10))):
+        runner = runner_from_folder(folder, EngineConfig(dtype="bfloat16", page_size=16, max_tokens=128, max_num_seqs=4,
+                                                         device=DEV, **kw))
+        held = [w for layer in runner.model.layers for w in (layer.mixer.w_qkv, layer.mixer.w_out, layer.feed_forward.w1,
+                                                             layer.feed_forward.w2)]
+        assert all(isinstance(w, PreparedWeight) for w in held)
+        seen[name] = [(tuple(w.tensor.shape), w.tiles is not None or w.folded is not None) for w in held]
+        rows = {}
+        for rec in steps:
+            from transformers_neuronx_amd.engine import StepEntry
+            logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in rec["entries"]]).float().cpu()
+            for row in range(logits.shape[0]):
+                rid, pos = place[(rec["step"], row)]
+                err = float((logits[row] - expected[rid][pos]).abs().max() / expected[rid].abs().max())
+                assert err <= TOL["bfloat16"], (name, rec["step"], rid, pos, err)
+            for rid in rec["end"]:
+                runner.finish(rid)
+    assert not any(c for _, c in seen["none"]) and all(c for _, c in seen["all"])
+    # 224 KB: by rising rows, the output products (128 x 128, 32 KB each) and fc2 (128 x 256, 64 KB each) of both
+    # layers; then no fc1 (256 x 128), QKV (384 x 128) or head fits what is left
+    assert sorted(shape for shape, c in seen["some"] if c) == [(128, 128), (128, 128), (128, 256), (128, 256)]

@@ -156,7 +156,9 @@ class EngineConfig:
                      is sized from memory
     weight_copies    keep a second copy of every matrix in the order the few-rows product streams it
                      (faster decoding at small batches, twice the memory for matrices); None decides by
-                     what fits beside the cache
+                     what fits beside the cache: all, or, where they do not all fit, those that do
+    weight_copy_bytes  the most bytes such copies may take (those of the matrices with the fewest rows
+                     are made first); None: what is free beside the weights and the cache
     run_ahead        a step is started before the host has read the tokens of the step before it (they
                      stay on the device for it); generation is the same, tokens are reported one call later
     cast_float32_weights   bfloat16 engine: matrices stored in 32-bit are rounded to bfloat16 at load, as the
@@ -180,6 +182,7 @@ class EngineConfig:
     prompts_first: bool = False
     run_ahead: bool = True
     weight_copies: Optional[bool] = None
+    weight_copy_bytes: Optional[int] = None
     cast_float32_weights: bool = False
     seed: int = 0
 
@@ -191,5 +194,7 @@ class EngineConfig:
             raise ValueError(f"kernels must be 'hip' or 'reference', got {self.kernels!r}")
         if self.max_num_seqs <= 0 or self.max_num_batched_tokens <= 0:
             raise ValueError("max_num_seqs and max_num_batched_tokens must be positive")
+        if self.weight_copy_bytes is not None and self.weight_copy_bytes < 0:
+            raise ValueError(f"weight_copy_bytes must not be negative, got {self.weight_copy_bytes}")
         if self.chunk_size is not None and self.chunk_size <= 0:
             raise ValueError(f"chunk_size must be positive, got {self.chunk_size}")

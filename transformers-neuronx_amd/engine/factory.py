@@ -34,23 +34,29 @@ def size_page_pool(cfg: EngineConfig, bytes_per_page: int, device: torch.device)
     return 256
 
 
-def _room_for_weight_copies(cfg: EngineConfig, model: DecoderModel, bytes_per_page: int, device) -> bool:
-    """Whether the matrices get a second, tile-ordered copy for the few-rows product (`weight_copies`;
-    left open, they do when matrices twice over and the cache asked for fit 90 % of the device's memory,
-    a quarter of it standing in for a cache sized from what is left)."""
-    if cfg.weight_copies is not None:
+def _cache_bytes(cfg: EngineConfig, bytes_per_page: int, total: int) -> int:
+    """The cache's size as far as it is known before it is made (a quarter of the device's memory stands in
+    for one sized from what is left)."""
+    if cfg.num_pages is not None:
+        return cfg.num_pages * bytes_per_page
+    if cfg.max_tokens is not None:
+        return -(-cfg.max_tokens // cfg.page_size) * bytes_per_page
+    return total // 4
+
+
+def _room_for_weight_copies(cfg: EngineConfig, model: DecoderModel, bytes_per_page: int, device):
+    """Whether the matrices get a second, tile-ordered copy for the few-rows product (`weight_copies`): True
+    when matrices twice over and the cache asked for fit 90 % of the device's memory, "later" when they do
+    not (then as many as fit are made once the weights are loaded), or what the configuration says."""
+    if cfg.weight_copies is not None and (not cfg.weight_copies or cfg.weight_copy_bytes is None):
         return bool(cfg.weight_copies)
     if device.type != "cuda" or cfg.dtype != torch.bfloat16:
         return False
+    if cfg.weight_copy_bytes is not None:
+        return "later"
     matrices = sum(2 * int(torch.Size(d.shape).numel()) for d in model.param_decls() if d.role in ("matrix", "table"))
     _, total = torch.cuda.mem_get_info(device)
-    if cfg.num_pages is not None:
-        cache = cfg.num_pages * bytes_per_page
-    elif cfg.max_tokens is not None:
-        cache = -(-cfg.max_tokens // cfg.page_size) * bytes_per_page
-    else:
-        cache = total // 4
-    return 2.2 * matrices + cache <= 0.9 * total
+    return True if 2.2 * matrices + _cache_bytes(cfg, bytes_per_page, total) <= 0.9 * total else "later"
 
 
 def build_runner(model_config, source, cfg: EngineConfig) -> ModelRunner:
@@ -63,11 +69,21 @@ def build_runner(model_config, source, cfg: EngineConfig) -> ModelRunner:
     bytes_per_page = CacheManager.bytes_per_page(needs, cfg.page_size, cfg.dtype)
     if hasattr(ops, "decode_copies"):
         ops.decode_copies = _room_for_weight_copies(cfg, model, bytes_per_page, device)
-    model.load(source, ops, cfg.dtype, device, cast_float32=cfg.cast_float32_weights)
+    later = getattr(ops, "decode_copies", None) == "later"
+    model.load(source, ops, cfg.dtype, device, cast_float32=cfg.cast_float32_weights, finish=not later)
     if hasattr(source, "release"):
         source.release()        # before the cache is sized and made: what the source held is free again,
         if device.type == "cuda":  # and goes back to the device, so that the cache's large blocks find room
             torch.cuda.empty_cache()
+    if later:
+        # the copies that fit beside the weights and the cache, with a twentieth of the device and 4 GB to spare
+        free, total = torch.cuda.mem_get_info(device)
+        room = free - _cache_bytes(cfg, bytes_per_page, total) - total // 20 - (4 << 30)
+        if cfg.weight_copy_bytes is not None:
+            room = min(room, cfg.weight_copy_bytes)
+        ops.copy_bytes = ops.finish_weights(max(0, room))
+        model.finish_load()
+        torch.cuda.empty_cache()
     num_pages = size_page_pool(cfg, bytes_per_page, device)
     cache = CacheManager(needs, cfg.page_size, num_pages, cfg.max_num_seqs, cfg.dtype, device)
     return ModelRunner(model, cache, ops, use_graphs=cfg.use_graphs)

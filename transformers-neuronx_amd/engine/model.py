@@ -34,10 +34,11 @@ class _Layer:
     def param_decls(self) -> List[ParamDecl]:
         return [d for part, prefix in self._named() for d in part.param_decls(prefix)]
 
-    def load(self, tensors, ops, dtype):
+    def load(self, tensors, ops, dtype, finish=True):
         for part, prefix in self._named():
             part.load(tensors, prefix, ops, dtype)
-        self.block.after_load()
+        if finish:
+            self.block.after_load()
 
 
 def _spec_of(kind):
@@ -81,16 +82,23 @@ class DecoderModel:
 
     # ---------------------------------------------------------------- weights
 
-    def load(self, source, ops, dtype: torch.dtype, device, cast_float32: bool = False) -> "DecoderModel":
+    def load(self, source, ops, dtype: torch.dtype, device, cast_float32: bool = False,
+             finish: bool = True) -> "DecoderModel":
+        """`finish=False` leaves out what the blocks do once their parts have their tensors (`finish_load`
+        does it later: the caller has something to do to the weights in between)."""
         tensors = load_tensors(self.param_decls(), source, dtype, device, self.spec.base_model_prefix, cast_float32)
         self.embedding.load(tensors, "", ops, dtype)
         for layer in self.layers:
-            layer.load(tensors, ops, dtype)
+            layer.load(tensors, ops, dtype, finish)
         self.head.load(tensors, "", ops, dtype)
         self.ops, self.dtype, self.device = ops, dtype, device
         self.weight_bytes = sum(t.numel() * t.element_size() for t in {id(t): t for t in tensors.values()}.values())
         self.loaded = True
         return self
+
+    def finish_load(self) -> None:
+        for layer in self.layers:
+            layer.block.after_load()
 
     # ---------------------------------------------------------------- one step
 
