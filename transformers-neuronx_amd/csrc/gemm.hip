@@ -1220,13 +1220,15 @@ __global__ void __launch_bounds__(256) library_flush_kernel(const float4* __rest
   if (a == 12345.678f) *sink = a;      // never true for memory that holds no such sum; keeps the loads alive
 }
 
-// Time in ms of one run of an algorithm with cold caches, or a negative number if it cannot be run.
+// Time in ms of a run of an algorithm with cold caches, the quickest of five (one run's time moves by more
+// than the candidates differ when something else touches the device meanwhile), or a negative number if it
+// cannot be run.
 float library_time(hipblasLtHandle_t handle, const LibraryPlan& p, const hipblasLtMatmulAlgo_t& algo,
                    const LibraryCall& call, void* flush, size_t flush_bytes, hipEvent_t begin, hipEvent_t end) {
   for (int warm = 0; warm < 2; ++warm)
     if (library_run(handle, p, algo, call) != HIPBLAS_STATUS_SUCCESS) return -1.f;
-  float total = 0.f;
-  for (int run = 0; run < 3; ++run) {
+  float best = -1.f;
+  for (int run = 0; run < 5; ++run) {
     library_flush_kernel<<<2048, 256, 0, call.stream>>>((const float4*)flush, flush_bytes / 16, (float*)flush);
     if (hipGetLastError() != hipSuccess || hipEventRecord(begin, call.stream) != hipSuccess) return -1.f;
     if (library_run(handle, p, algo, call) != HIPBLAS_STATUS_SUCCESS) return -1.f;
@@ -1234,9 +1236,9 @@ float library_time(hipblasLtHandle_t handle, const LibraryPlan& p, const hipblas
     if (hipEventRecord(end, call.stream) != hipSuccess || hipEventSynchronize(end) != hipSuccess ||
         hipEventElapsedTime(&ms, begin, end) != hipSuccess)
       return -1.f;
-    total += ms;
+    if (best < 0.f || ms < best) best = ms;
   }
-  return total;
+  return best;
 }
 
 // The plan of one product: descriptors and an algorithm. Row-major out[M][N] = x[M][K] w[N][K]^T is, in the
