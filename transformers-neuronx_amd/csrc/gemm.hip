@@ -1085,7 +1085,8 @@ extern "C" int tnx_gemm_bf16_mid(const void* x, const void* w_tiles, const float
   TNX_REQUIRE(x && w_tiles && out && ((uintptr_t)x | (uintptr_t)w_tiles | (uintptr_t)workspace) % 16 == 0,
               "gemm_bf16_mid: operands must be there and 16-byte aligned");
   TNX_REQUIRE(out_dtype == TNX_F32 || out_dtype == TNX_BF16, "gemm_bf16_mid: the result is float32 or bfloat16");
-  TNX_REQUIRE(shares >= 0 && ahead >= 0 && ahead <= 4, "gemm_bf16_mid: bad shares or steps ahead");
+  TNX_REQUIRE(shares >= 0 && (ahead == 0 || ahead == 2 || ahead == 3), "gemm_bf16_mid: bad shares, or steps ahead "
+              "other than 2 and 3");
   const int blocks_n = (N / 16 + 3) / 4, steps_all = K / 128;
   if (shares == 0) {
     // a block a compute unit at most: blocks of one length in a ragged second round cost more than idle units
@@ -1103,8 +1104,8 @@ extern "C" int tnx_gemm_bf16_mid(const void* x, const void* w_tiles, const float
   if (ahead == 0) ahead = mt <= 4 ? 3 : 2;
   if (mt > 4 && ahead > 2) ahead = 2;               // what LDS holds
 #define MID(MT, A) launch_mid<MT, A>(xp, wp, bias, residual, out, out_dtype, act, workspace, M, N, K, shares, stream)
-#define MID_LOW(MT) return ahead == 1 ? MID(MT, 1) : ahead == 2 ? MID(MT, 2) : ahead == 3 ? MID(MT, 3) : MID(MT, 4)
-#define MID_HIGH(MT) return ahead == 1 ? MID(MT, 1) : MID(MT, 2)
+#define MID_LOW(MT) return ahead == 2 ? MID(MT, 2) : MID(MT, 3)
+#define MID_HIGH(MT) return MID(MT, 2)
   switch (mt) {
     case 1: MID_LOW(1);
     case 2: MID_LOW(2);
