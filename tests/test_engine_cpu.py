@@ -600,3 +600,38 @@ def test_sample_takes_the_ngram_ban(tiny_folders):
     eos = cfg.get("eos_token_id", 2)
     for b in range(2):
         assert out[b, 4:].tolist() == _plain_without_repeats(weights, cfg, ids[b].tolist(), 12, 2, banned_token=eos)
+
+
+@pytest.mark.parametrize("run_ahead", [False, True])
+def test_a_request_taken_out_midway(tiny_folders, run_ahead):
+    """`abort_request` between two steps: the request reports nothing more (a step under way may still hold
+    a token for it), what it held is free at once, and the others go on as if it had never been there."""
+    folder, cfg, weights = tiny_folders["B"]
+    runner, ecfg = _runner(folder, max_tokens=256, run_ahead=run_ahead)
+    engine = LLMEngine(runner, ecfg)
+    prompts = [[5, 9, 200, 31], [7, 7, 100, 3, 8, 15], [11, 12, 13]]
+    params = SamplingParams(max_new_tokens=12, do_sample=False, ignore_eos=True)
+    ids = [engine.add_request(p, params) for p in prompts]
+    late = engine.add_request([4, 4, 4], params)           # one that is still waiting when it is taken out
+    engine.scheduler.max_num_seqs = 3
+    got = {i: [] for i in ids + [late]}
+    gone = None
+    for step in range(200):
+        if not engine.has_work:
+            break
+        for out in engine.step():
+            assert out.req_id != ids[1] or gone is None, "a token after the request was taken out"
+            got[out.req_id].append(out.token)
+        if step == 4:
+            assert runner.cache.has(ids[1])
+            gone = engine.abort_request(ids[1])
+            engine.abort_request(late)
+            assert gone.finished and gone.finish_reason == "aborted" and not runner.cache.has(ids[1])
+            assert gone.output == got[ids[1]] and 0 < len(gone.output) < 12
+            runner.cache.check()
+    assert not engine.has_work and not runner.cache.requests
+    for i in (0, 2):
+        assert got[ids[i]] == plain_opt.greedy(weights, cfg, prompts[i], 12)[len(prompts[i]):]
+    assert got[late] == [] and ids[1] not in engine.requests
+    with pytest.raises(KeyError):
+        engine.abort_request("nobody")

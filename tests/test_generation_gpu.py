@@ -193,3 +193,30 @@ def test_no_run_of_tokens_twice_on_the_gpu(tiny_folders):
     toks = torch.tensor([4, 0, 9, 1, 10], dtype=torch.int32, device=DEV)
     ops.ban_pairs(logits, rows, toks)
     assert torch.isinf(logits).nonzero().tolist() == [[0, 4], [2, 0], [2, 9]]
+
+
+@pytest.mark.parametrize("run_ahead", [False, True])
+def test_a_request_taken_out_midway_on_the_gpu(tiny_folders, run_ahead):
+    """`abort_request` while steps run ahead on the device: the slot and the pages it gives back go to a request
+    that arrives afterwards, and every other request keeps the plain implementation's tokens."""
+    from transformers_neuronx_amd.sampling import SamplingParams
+    folder, cfg, weights = tiny_folders["A"]
+    engine, runner = _engine(folder, "float32", page_size=16, max_tokens=96, max_num_seqs=3, run_ahead=run_ahead,
+                             use_graphs=True)
+    prompts = _prompts(cfg["vocab_size"], [9, 20, 5, 12], 3)
+    params = SamplingParams(max_new_tokens=14, do_sample=False, ignore_eos=True)
+    ids = [engine.add_request(p, params) for p in prompts[:3]]
+    got = {}
+    for step in range(300):
+        if not engine.has_work:
+            break
+        for out in engine.step():
+            got.setdefault(out.req_id, []).append(out.token)
+        if step == 5:
+            engine.abort_request(ids[1])
+            ids.append(engine.add_request(prompts[3], params))     # takes the slot and pages just given back
+    runner.cache.check()
+    assert not engine.has_work and not runner.cache.requests
+    for i in (0, 2, 3):
+        assert got[ids[i]] == plain_opt.greedy(weights, cfg, prompts[i], 14)[len(prompts[i]):], i
+    assert 0 < len(got[ids[1]]) < 14

@@ -192,6 +192,15 @@ class LLMEngine:
         self.run()
         return [list(self.pop_request(i).output) for i in ids]
 
+    def abort_request(self, req_id: Hashable) -> Request:
+        """Stop a request whose caller has gone, between two calls of `step()`: its pages and its slot are
+        free for the next step, no further token of it is reported (one that a step already started would
+        still deliver is dropped), and the request is handed over with what it has generated so far."""
+        req = self.requests[req_id]
+        self.scheduler.abort(req)
+        self.scheduler.finished.clear()
+        return self.requests.pop(req_id)
+
     def pop_request(self, req_id: Hashable) -> Request:
         """Hand over a request that has ended and forget it. A request stays in `requests`, with its prompt
         and output, until this is called (or `reset`): a caller that drives `step()` itself calls it when it

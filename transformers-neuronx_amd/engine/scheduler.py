@@ -257,6 +257,16 @@ class Scheduler:
         self.finished.append(req)
         ended.append(req)
 
+    def abort(self, req: Request) -> None:
+        """Take a request out, wherever it stands: it ends with the reason "aborted" and gives back what it
+        holds. A token that a step under way is still to deliver for it is dropped when it comes (`resolve`
+        finds the request shorter than the place the token was meant for)."""
+        if req.finished:
+            return
+        if PENDING in req.output:
+            del req.output[req.output.index(PENDING):]
+        self._end(req, "aborted", [])
+
     def record(self, runs: List[ScheduledRun]) -> List[Request]:
         """What the step computes, before its tokens are known: every run that samples gets `PENDING` as
         its request's newest token. Requests that reach `max_new_tokens` or the length limit with it end
