@@ -635,3 +635,24 @@ def test_a_request_taken_out_midway(tiny_folders, run_ahead):
     assert got[late] == [] and ids[1] not in engine.requests
     with pytest.raises(KeyError):
         engine.abort_request("nobody")
+
+
+def test_several_tokens_end_a_request(tiny_folders):
+    """`eos_token_id` as a list (sampling.py:319-322): the request ends at the first of them it generates, and
+    with `ban_eos` none of them is ever chosen."""
+    folder, cfg, weights = tiny_folders["B"]
+    runner, ecfg = _runner(folder, max_tokens=128)
+    engine = LLMEngine(runner, ecfg)
+    prompt = [5, 9, 200, 31]
+    free = plain_opt.greedy(weights, cfg, prompt, 12)[len(prompt):]
+    stops = [free[6], free[3], 999]
+    out = engine.generate([prompt], SamplingParams(max_new_tokens=12, do_sample=False, eos_token_id=stops))[0]
+    assert out == free[:free.index(free[3]) + 1]
+    out = engine.generate([prompt], SamplingParams(max_new_tokens=12, do_sample=False, eos_token_id=stops, ban_eos=True,
+                                                   ignore_eos=True))[0]
+    toks = list(prompt)
+    for _ in range(12):
+        row = plain_opt.forward_logits(weights, cfg, toks)[-1].clone()
+        row[stops] = float("-inf")
+        toks.append(int(row.argmax()))
+    assert out == toks[len(prompt):] and not set(out) & set(stops)

@@ -273,7 +273,7 @@ class CausalLMForSampling:
                     (len(q.output) > column and q.output[column] >= 0) or (q.finished and len(q.output) <= column)
                     for q in reqs):
                 streamer.put(torch.tensor([[q.output[column] if len(q.output) > column else
-                                            (p.eos_token_id if p.eos_token_id is not None else 0)]
+                                            (p.eos_ids[0] if p.eos_ids else 0)]
                                            for q, p in zip(reqs, params)], dtype=prompts.dtype))
                 column += 1
         if streamer is not None:
@@ -282,7 +282,7 @@ class CausalLMForSampling:
         result[:, :width] = prompts
         for b, i in enumerate(ids):
             out = engine.requests[i].output
-            eos = params[b].eos_token_id if params[b].eos_token_id is not None else 0
+            eos = params[b].eos_ids[0] if params[b].eos_ids else 0
             out = out + [eos] * (sequence_length - width - len(out))   # rows that stopped early repeat eos
             result[b, width:] = torch.tensor(out, dtype=prompts.dtype)
         return result

@@ -6,7 +6,7 @@ options (config.py:73-139, :206-363) for the ones that have a counterpart on one
 GPU, so that code written against the reference's API keeps working.
 """
 from dataclasses import dataclass, field
-from typing import Optional
+from typing import List, Optional, Union
 
 import torch
 
@@ -68,7 +68,7 @@ class GenerationConfig:
     top_p: float = 1.0
     top_p_min_tokens: int = 1
     global_top_k: Optional[int] = None
-    eos_token_id: Optional[int] = None
+    eos_token_id: Optional[Union[int, List[int]]] = None
     temperature: float = 1.0
     dynamic: bool = False
     deterministic: bool = False

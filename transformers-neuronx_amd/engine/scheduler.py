@@ -303,7 +303,7 @@ class Scheduler:
             req.output[run.out_index] = int(token)
             kept.append(int(token))
             p = req.params
-            if p.eos_token_id is not None and int(token) == p.eos_token_id and not p.ignore_eos:
+            if not p.ignore_eos and int(token) in p.eos_ids:
                 del req.output[run.out_index + 1:]      # what was drawn after it is dropped
                 self._end(req, "eos", [])
         return kept

@@ -1,6 +1,6 @@
 """What a request asks of the sampler."""
 from dataclasses import dataclass
-from typing import Optional
+from typing import Optional, Sequence, Tuple, Union
 
 
 @dataclass
@@ -20,6 +20,7 @@ class SamplingParams:
                  counter n, whatever else is in the batch; None lets the engine give one
                  (its own seed plus the request's number of arrival)
     deterministic  every draw uses 0.5 in place of a random number (hlo.py:2455-2456)
+    eos_token_id the token that ends the request, or a list of such tokens (sampling.py:319-322)
     ban_eos      the end-of-sequence token is never chosen (`scores[:, eos] = -inf`,
                  sampling.py:143-144, the OPT loop's behaviour)
     ignore_eos   generation does not stop at the end-of-sequence token
@@ -36,7 +37,7 @@ class SamplingParams:
     seed: Optional[int] = 0
     min_tokens_to_keep: int = 1
     deterministic: bool = False
-    eos_token_id: Optional[int] = None
+    eos_token_id: Optional[Union[int, Sequence[int]]] = None      # one token or several (sampling.py:319-322)
     ban_eos: bool = False
     ignore_eos: bool = False
     no_repeat_ngram_size: int = 0
@@ -54,6 +55,15 @@ class SamplingParams:
             raise ValueError(f"`ngram_size` has to be a strictly positive integer, but is {self.no_repeat_ngram_size}")
         if float(self.temperature) < 0:
             raise ValueError("temperature has to be a non-negative float (0 is greedy).")
+
+    @property
+    def eos_ids(self) -> Tuple[int, ...]:
+        """The tokens that end the request, as a tuple (empty: none does)."""
+        if self.eos_token_id is None:
+            return ()
+        if isinstance(self.eos_token_id, int):
+            return (self.eos_token_id,)
+        return tuple(int(t) for t in self.eos_token_id)
 
     @property
     def greedy(self) -> bool:

@@ -37,7 +37,9 @@ class Sampler:
         m = logits.shape[0]
         if m != len(params):
             raise ValueError(f"{m} logits rows for {len(params)} requests")
-        pairs = []
+        # (row, token) pairs that get -inf: every end-of-sequence token of a request that has several and must not
+        # choose one, and the tokens that would repeat a run of n
+        pairs = [(i, t) for i, p in enumerate(params) if p.ban_eos and len(p.eos_ids) > 1 for t in p.eos_ids]
         for i, p in enumerate(params):
             if p.no_repeat_ngram_size:
                 if histories is None or histories[i] is None:
@@ -50,7 +52,7 @@ class Sampler:
             else:
                 dev = torch.from_numpy(flat.reshape(-1)).to(self.device)
             self.ops.ban_pairs(logits, dev[:len(pairs)], dev[len(pairs):])
-        banned = [p.eos_token_id if (p.ban_eos and p.eos_token_id is not None) else -1 for p in params]
+        banned = [p.eos_ids[0] if (p.ban_eos and len(p.eos_ids) == 1) else -1 for p in params]
         if any(b >= 0 for b in banned):
             if hasattr(self.ops, "send_ints"):
                 self.ops.ban_tokens(logits, self.ops.send_ints(np.array(banned, dtype=np.int32)))
