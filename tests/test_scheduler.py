@@ -197,3 +197,27 @@ def test_a_step_recorded_before_its_tokens_are_known():
     assert a.output == [4, 5, 9] and a.finish_reason == "eos" and b.output == [9]
     assert [r.req_id for r in s.finished] == ["b", "a"]
     cache.check()
+
+
+def test_a_request_ends_when_its_time_is_up():
+    """`max_time` (stopping_criteria.py:15-35): the first token that comes later than that ends the request,
+    with the reason "time"; a request with time to spare is not touched."""
+    import time
+    from transformers_neuronx_amd.engine.scheduler import Request, Scheduler
+    from transformers_neuronx_amd.sampling import SamplingParams
+    cache = CacheManager({0: CacheNeed("paged")}, 16, 8, 4, torch.float32, "cpu")
+    sched = Scheduler(cache, 4, 64, 128)
+    slow = Request("slow", [1, 2, 3], SamplingParams(max_new_tokens=10, max_time=0.0, ignore_eos=True))
+    fast = Request("fast", [4, 5], SamplingParams(max_new_tokens=3, max_time=3600.0, ignore_eos=True))
+    sched.add(slow)
+    sched.add(fast)
+    time.sleep(0.002)
+    steps = 0
+    while sched.has_work:
+        runs = sched.schedule()
+        sched.update(runs, [7 if r.samples else None for r in runs])
+        steps += 1
+    assert slow.output == [7] and slow.finish_reason == "time"
+    assert fast.output == [7, 7, 7] and fast.finish_reason == "length" and steps == 3
+    cache.check()
+    assert not cache.requests

@@ -16,7 +16,9 @@ Every decision is a function of arrival order, lengths and capacities only:
     from its first token later, generated tokens included (they are kept). A
     lone request that does not fit raises `OutOfPages`;
   * a request ends at its end-of-sequence token (unless told to ignore it), at
-    `max_new_tokens`, or at the length limit, and frees its pages in that step.
+    `max_new_tokens`, or at the length limit, and frees its pages in that step
+    (a `max_time`, the one decision that looks at a clock, ends it at the first
+    token that comes too late).
 
 A step's outcome may be recorded in two halves, so that the next step can be planned and started
 while the device still works on this one: `record` notes what was computed and puts `PENDING` in
@@ -26,6 +28,7 @@ token. A request that is found to have ended this way may already be part of the
 started meanwhile: that run's work is wasted and its token is dropped when it is resolved.
 `update` does both at once.
 """
+import time
 from collections import deque
 from dataclasses import dataclass, field
 from typing import Deque, Hashable, List, Optional
@@ -49,6 +52,7 @@ class Request:
     finish_reason: Optional[str] = None
     preemptions: int = 0
     arrival: int = 0
+    taken_in: float = 0.0           # when the scheduler took it in (time.monotonic), for `max_time`
 
     @property
     def tokens(self) -> List[int]:
@@ -118,6 +122,7 @@ class Scheduler:
                              f"({len(request.prompt)} prompt + {request.params.max_new_tokens} new); "
                              f"the limit is {self.max_model_len}")
         request.arrival = self._arrivals
+        request.taken_in = time.monotonic()
         self._arrivals += 1
         self.waiting.append(request)
 
@@ -306,6 +311,9 @@ class Scheduler:
             if not p.ignore_eos and int(token) in p.eos_ids:
                 del req.output[run.out_index + 1:]      # what was drawn after it is dropped
                 self._end(req, "eos", [])
+            elif p.max_time is not None and time.monotonic() - req.taken_in > p.max_time:
+                del req.output[run.out_index + 1:]
+                self._end(req, "time", [])
         return kept
 
     def update(self, runs: List[ScheduledRun], sampled: List[Optional[int]]) -> List[Request]:

@@ -27,6 +27,8 @@ class SamplingParams:
     no_repeat_ngram_size  n: no run of n tokens appears twice in the prompt and what follows it; a token
                  that would complete a run seen before gets the logit -inf before anything else is done
                  (sampling.py:267-309, :334-335); 0 switches it off
+    max_time     seconds: the request ends after the first token that arrives later than this after it was
+                 taken in (stopping_criteria.py:15-35, `MaxTimeCriteria`)
     max_new_tokens  the most tokens to generate
     """
     max_new_tokens: int = 16
@@ -41,6 +43,7 @@ class SamplingParams:
     ban_eos: bool = False
     ignore_eos: bool = False
     no_repeat_ngram_size: int = 0
+    max_time: Optional[float] = None
 
     def __post_init__(self):
         if self.max_new_tokens < 0:
