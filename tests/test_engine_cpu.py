@@ -656,3 +656,25 @@ def test_several_tokens_end_a_request(tiny_folders):
         row[stops] = float("-inf")
         toks.append(int(row.argmax()))
     assert out == toks[len(prompt):] and not set(out) & set(stops)
+
+
+def test_host_loops_by_their_names(tiny_folders):
+    """`sampling.simple_sample` and `sampling.sample_greedy` (sampling.py:26-30, :108-128) as functions of a
+    model: greedy with top_k 1, the scores of every step on request, another end-of-sequence token than the
+    configuration's."""
+    from transformers_neuronx_amd import OPTForSampling
+    from transformers_neuronx_amd.sampling import sample_greedy, simple_sample
+    folder, cfg, weights = tiny_folders["B"]
+    model = OPTForSampling.from_pretrained(folder, batch_size=2, amp="f32", n_positions=32, kernels="reference",
+                                           device="cpu", page_size=16).to_neuron()
+    ids = torch.tensor([[5, 9, 200, 31], [7, 7, 100, 3]])
+    free = [plain_opt.greedy(weights, cfg, ids[b].tolist(), 8) for b in range(2)]
+    assert sample_greedy(model, ids, sequence_length=12).tolist() == free
+    banned = free[0][6]                                        # a token the free path takes
+    tokens, scores = simple_sample(model, ids, None, 12, eos_token_id=banned, top_k=1, output_scores=True)
+    assert len(scores) == 8 and scores[0].shape == (2, cfg["vocab_size"]) and bool(torch.isinf(scores[3][:, banned]).all())
+    assert banned not in tokens[0, 4:].tolist() and tokens[0, :6].tolist() == free[0][:6]
+    row = plain_opt.forward_logits(weights, cfg, ids[0].tolist())[-1]
+    keep = [i for i in range(cfg["vocab_size"]) if i != banned]
+    torch.testing.assert_close(scores[0][0][keep], row[keep], rtol=1e-4, atol=1e-5)
+    assert model.config.eos_token_id == cfg.get("eos_token_id", 2) and model.engine.logits_hook is None

@@ -220,12 +220,13 @@ class CausalLMForSampling:
     def sample(self, input_ids, sequence_length: int, start_ids=None, top_k: int = 50, streamer=None,
                temperature: float = 1.0, top_p: float = 1.0, seed: int = 0,
                generation_config: Optional[GenerationConfig] = None,
-               no_repeat_ngram_size: Optional[int] = None) -> torch.Tensor:
+               no_repeat_ngram_size: Optional[int] = None, eos_token_id: Optional[int] = None) -> torch.Tensor:
         """`[batch, sequence_length]`: the prompts and what follows them, up to a total
         length of `sequence_length`. As the reference's loop (sampling.py:131-180) it
         never picks the end-of-sequence token and keeps the `top_k` largest logits;
         `top_k=1` is greedy. With `on_device_generation` in the NeuronConfig, or a
         `generation_config`, those options decide instead (sampling.py:33-105).
+        `eos_token_id`: the token the loop never picks, where it is not the configuration's.
         `no_repeat_ngram_size`: no run of that many tokens appears twice in a row's prompt and what
         follows it (the option of the reference's other loop, sampling.py:382-394)."""
         engine = self._need_engine()
@@ -256,7 +257,9 @@ class CausalLMForSampling:
                                    no_repeat_ngram_size=int(no_repeat_ngram_size or 0))
             else:
                 p = SamplingParams(max_new_tokens=new, do_sample=True, temperature=temperature, top_k=top_k,
-                                   top_p=top_p, seed=seed + b, eos_token_id=getattr(self.config, 'eos_token_id', None),
+                                   top_p=top_p, seed=seed + b,
+                                   eos_token_id=(eos_token_id if eos_token_id is not None
+                                                 else getattr(self.config, 'eos_token_id', None)),
                                    ban_eos=True, ignore_eos=True, no_repeat_ngram_size=int(no_repeat_ngram_size or 0))
             params.append(p)
         engine.reset()
