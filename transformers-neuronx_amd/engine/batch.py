@@ -48,7 +48,14 @@ def attention_plan(run_lens: np.ndarray, cached: np.ndarray, page_size: int):
     arrays = {"decode_runs": decode_runs, "tile_run": np.array([t[1] for t in tiles], dtype=np.int32),
               "tile_start": np.array([t[2] for t in tiles], dtype=np.int32),
               "longest_decode": np.array([longest], dtype=np.int32)}
-    return arrays, {"longest_decode": longest}
+    # What a recorded decode step is sized by beside its requests (a key that begins with "record:" is part
+    # of what two steps must share to share a recording): how many blocks of 256 keys the longest request
+    # fills, up to 8, and whether the requests are about as long as it (their mean at least 0.8 of it), which
+    # is when cutting every request into that many blocks pays.
+    mean = float((cached[single] + 1).mean()) if single.any() else 0.0
+    alike = bool(mean >= 0.8 * longest)
+    shape = (min(8, -(-longest // 256)) if alike else 0, alike)     # (requests that differ: one recording serves)
+    return arrays, {"longest_decode": longest, "record:decode": shape}
 
 
 register_step_planner("attention", attention_plan)
@@ -150,7 +157,8 @@ class PackedStep:
     def layout(self):
         """What two steps must share for one to reuse the other's device buffer and views."""
         return (tuple(self.offsets), tuple(self.sizes), self.num_tokens, self.num_requests,
-                tuple(self.group_names), tuple(sorted(self.widths.items())), self.page_size)
+                tuple(self.group_names), tuple(sorted(self.widths.items())), self.page_size,
+                tuple(sorted((k, v) for k, v in self.plan_host.items() if k.startswith("record:"))))
 
 
 _FIXED_PIECES = 7    # the step's own pieces, before the planners' and the per-group ones, see pack_step

@@ -799,28 +799,34 @@ class HipOps:
 
     def _decode_splits(self, ctx, pairs: int, window: int, head_size: int = 128):
         """(splits, waves): how many blocks share the keys of one decoding (request, head), and how many
-        waves a block has. Enough blocks to give every compute unit one, no block with less than 256 keys
-        (a 64-key tile a wave). Blocks of four waves: with the products on the matrix unit a wave keeps the
+        waves a block has. Blocks of four waves: with the products on the matrix unit a wave keeps the
         next tile's keys and values in flight by itself, and more waves bought nothing (measured at head
         size 128 and a context of 2,048: one request 8 x 4 waves 15.6 us against 16.9 for 4 x 8; eight
-        requests 49.7 against 50.9; 64 requests 369 against 376). A step that is recorded for replay is
-        sized for the longest request the engine allows."""
+        requests 49.7 against 50.9; 64 requests 369 against 376).
+        No block gets less than 256 keys of the longest request (a 64-key tile a wave). Requests about as
+        long as one another are cut into as many blocks as that allows, up to 8: small blocks spread evenly
+        over the compute units whatever the number of pairs (32 heads at 2,048 tokens, tokens a second: 9
+        requests 1,582 -> 1,801, 20: 2,388 -> 2,545, 33: 3,067 -> 3,150, 128: 4,398 -> 4,487), except
+        where the pairs alone give 0.7 to 1 block a compute unit (7 and 8 requests: whole requests, 1,548
+        against 1,520 and 1,675 against 1,654). Requests of very different lengths are not cut beyond what
+        gives every compute unit a block: most blocks of a short request would be empty (64 requests of 16
+        to 1,280 tokens: 6,430 tokens a second whole, 4,760 in eight blocks each). A recorded step is sized
+        by the same two facts, which are part of what it is recorded under."""
         longest = ctx.length_bound if ctx.length_bound is not None else ctx.longest_decode_host
+        fills, alike = ctx.plan_host.get("record:decode", (0, False))
+        if not alike:
+            fills = min(8, -(-longest // 256))
         if window:
             longest = min(longest, window + 64)
-        wanted = self.decode_blocks_wanted or self.compute_units
+            fills = min(fills, -(-longest // 256))
         waves = 8 if self.decode_waves == 8 and head_size <= 128 else 4
-        splits = max(1, min(-(-wanted // pairs), -(-longest // 256)))
-        if splits == 1 and not self.decode_blocks_wanted:
-            # The chip holds two blocks of four waves a compute unit at a time (one at head sizes beyond 128). A
-            # few pairs more than it holds at once make a last round of whole-length blocks on a nearly empty
-            # chip: then four splits, so that the last round is a quarter as long (17 requests of 32 heads at
-            # 2,048 tokens: 8.13 -> 7.51 ms a step, 33 requests: 11.46 -> 10.70; at half a round over nothing)
-            held = self.compute_units * (1 if head_size > 128 else 2)
-            over = pairs % held
-            if pairs > held and 0 < over <= 0.35 * held:
-                splits = max(1, min(4, -(-longest // 256)))
-        return splits, waves
+        units = self.decode_blocks_wanted or self.compute_units
+        if self.decode_blocks_wanted:                  # told how many blocks to make (measurements and tests)
+            return max(1, min(-(-units // pairs), -(-longest // 256))), waves
+        if 0.7 * units <= pairs <= units:
+            return 1, waves
+        fill_the_chip = max(1, min(-(-units // pairs), fills))
+        return (max(fill_the_chip, fills) if alike else fill_the_chip), waves
 
     # ---------------------------------------------------------------- output end
 
