@@ -808,7 +808,9 @@ class HipOps:
         over the compute units whatever the number of pairs (32 heads at 2,048 tokens, tokens a second: 9
         requests 1,582 -> 1,801, 20: 2,388 -> 2,545, 33: 3,067 -> 3,150, 128: 4,398 -> 4,487), except
         where the pairs alone give 0.7 to 1 block a compute unit (7 and 8 requests: whole requests, 1,548
-        against 1,520 and 1,675 against 1,654). Requests of very different lengths are not cut beyond what
+        against 1,520 and 1,675 against 1,654) or a whole number of blocks each, within a twentieth (16, 24,
+        32, 48, 64 requests: the many small blocks and the kernel that merges them cost 2 to 3 % there and
+        have nothing to even out). Requests of very different lengths are not cut beyond what
         gives every compute unit a block: most blocks of a short request would be empty (64 requests of 16
         to 1,280 tokens: 6,430 tokens a second whole, 4,760 in eight blocks each). A recorded step is sized
         by the same two facts, which are part of what it is recorded under."""
@@ -826,6 +828,8 @@ class HipOps:
         if 0.7 * units <= pairs <= units:
             return 1, waves
         fill_the_chip = max(1, min(-(-units // pairs), fills))
+        if pairs > units and -(-pairs // units) * units <= 1.05 * pairs:
+            alike = False         # whole requests already come out even over the compute units
         return (max(fill_the_chip, fills) if alike else fill_the_chip), waves
 
     # ---------------------------------------------------------------- output end
