@@ -135,6 +135,29 @@ extern "C" int tnx_ban_tokens(float* logits, const int* token, int rows, int voc
   return 0;
 }
 
+// Inclusive sums from the top: out[d] = x[d] + x[d + 1] + ... + x[255], by the first 256 threads of the block
+// (four waves); `carry` holds four values. Every thread of the block calls it.
+template <typename T>
+__device__ __forceinline__ void sums_from_the_top(const T* x, T* out, T* carry) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  T v = 0;
+  if (tid < 256) {
+    v = x[255 - tid];                    // thread t takes digit 255 - t: a scan upwards over t runs down the digits
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const T w = __shfl_up(v, o, 64);
+      if (lane >= o) v += w;
+    }
+    if (lane == 63) carry[wave] = v;
+  }
+  __syncthreads();
+  if (tid < 256) {
+    for (int w = 0; w < wave; ++w) v += carry[w];
+    out[255 - tid] = v;
+  }
+  __syncthreads();
+}
+
 // One block per row.
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature, const int* __restrict__ top_k,
@@ -149,7 +172,9 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
   __shared__ int sh_digit;
   __shared__ unsigned int sh_remaining, sh_bin;
   __shared__ float sh_above, sh_total;
-  __shared__ int sh_result, sh_last;
+  __shared__ int sh_result, sh_last, sh_n;
+  __shared__ unsigned int cnt_above[256], carry_u[4];
+  __shared__ float mass_above[256], carry_f[4];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rowi = blockIdx.x;
@@ -192,16 +217,15 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
         if ((key & mask) == prefix) atomicAdd(&cnt[(unsigned int)(key >> shift) & 255u], 1u);
       }
       __syncthreads();
-      if (tid == 0) {
-        unsigned int rem = remaining;
-        int d = 255;
-        for (; d > 0; --d) {
-          if (cnt[d] >= rem) break;
-          rem -= cnt[d];
+      // the digit of the `remaining`-th largest: the highest one with that many keys at or above it
+      sums_from_the_top(cnt, cnt_above, carry_u);
+      if (tid < 256) {
+        const unsigned int here = cnt_above[tid], over = tid < 255 ? cnt_above[tid + 1] : 0u;
+        if ((here >= remaining && over < remaining) || (tid == 0 && here < remaining)) {
+          sh_digit = tid;
+          sh_remaining = remaining - min(over, remaining);
+          sh_bin = cnt[tid];
         }
-        sh_digit = d;
-        sh_remaining = rem;
-        sh_bin = cnt[d];
       }
       __syncthreads();
       prefix |= (uint64_t)sh_digit << shift;
@@ -221,8 +245,92 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
   if (k > 0) k = max(k, keep);
   if (k > 0 && k < vocab) floor_key = kth_largest((unsigned int)k);
 
-  // top-p: the smallest kept key is the last one whose predecessors hold less than p of the mass
   const float p = top_p[rowi];
+  // a counter below zero asks for the constant 0.5 the reference calls deterministic (hlo.py:2455-2456)
+  const float u = counters[rowi] < 0 ? 0.5f : philox_uniform((uint64_t)seeds[rowi], (uint64_t)counters[rowi]);
+  if (k > 0 && k < vocab && k <= SAMPLE_THREADS) {
+    // Few tokens are left, the k largest exactly (keys differ in their token ids): they are gathered, one a
+    // thread, put in the order of their token ids, and top-p and the draw are made over these alone.
+    __shared__ unsigned long long tkey[SAMPLE_THREADS], ckey[SAMPLE_THREADS];
+    __shared__ float tval[SAMPLE_THREADS];
+    if (tid == 0) {
+      sh_n = 0;
+      sh_result = -1;
+      sh_last = -1;
+    }
+    __syncthreads();
+    for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
+      const uint64_t key = order_key(row[i], i);
+      if (key >= floor_key) {
+        const int at = atomicAdd(&sh_n, 1);
+        if (at < SAMPLE_THREADS) {
+          tkey[at] = key;
+          tval[at] = __expf(row[i] * inv_temp - xmax);
+        }
+      }
+    }
+    __syncthreads();
+    const int n = min(sh_n, SAMPLE_THREADS);
+    // of each of them: its place in the order of token ids, and the mass and the number of those with a larger key
+    const bool have = tid < n;
+    const uint64_t my_key = have ? tkey[tid] : 0;
+    const float my_val = have ? tval[tid] : 0.f;
+    const uint32_t my_low = (uint32_t)my_key;          // the complement of the token id: larger is earlier
+    float above = 0.f, z = 0.f;
+    int rank = 0, place = 0;
+    for (int j = 0; j < n; ++j) {
+      const uint64_t kj = tkey[j];
+      const float e = tval[j];
+      z += e;
+      if (kj > my_key) {
+        above += e;
+        ++rank;
+      }
+      place += (uint32_t)kj > my_low ? 1 : 0;
+    }
+    // top-p keeps a token while those above it hold less than p of the mass, the largest always, and never
+    // fewer than `keep` (sampling.py:213-249, :232)
+    const bool kept = have && (p >= 1.f || above < p * z || rank == 0 || rank < keep);
+    part[tid] = 0.f;
+    __syncthreads();
+    if (have) {
+      ckey[place] = my_key;
+      part[place] = kept ? my_val : 0.f;
+    }
+    __syncthreads();
+    const float mine = part[tid];
+    if (mine > 0.f) atomicMax(&sh_last, tid);
+    __syncthreads();
+    if (wave == 0) {          // exclusive scan of the kept masses, in the order of the token ids
+      float local[16], run = 0.f;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        local[j] = run;
+        run += part[lane * 16 + j];
+      }
+      float incl = run;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const float w = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += w;
+      }
+#pragma unroll
+      for (int j = 0; j < 16; ++j) part[lane * 16 + j] = incl - run + local[j];
+      if (lane == 63) sh_total = incl;
+    }
+    __syncthreads();
+    const float goal = u * sh_total;
+    const float base = part[tid];
+    if (mine > 0.f && base <= goal && goal < base + mine) atomicMax(&sh_result, tid);
+    __syncthreads();
+    if (tid == 0) {
+      const int pick = sh_result >= 0 ? sh_result : max(sh_last, 0);
+      out[rowi] = (int)(~(uint32_t)ckey[pick]);
+    }
+    return;
+  }
+
+  // top-p: the smallest kept key is the last one whose predecessors hold less than p of the mass
   if (p < 1.f) {
     float z = 0.f;
     for (int i = tid; i < vocab; i += SAMPLE_THREADS)
@@ -251,22 +359,20 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
         }
       }
       __syncthreads();
-      if (tid == 0) {
-        float running = above, chosen_above = above;
-        int chosen = -1;
-        for (int d = 255; d >= 0; --d) {
-          if (cnt[d] == 0) continue;
-          if (running < target || chosen < 0) {
-            chosen = d;
-            chosen_above = running;
-          } else {
-            break;
-          }
-          running += mass[d];
-        }
-        sh_digit = chosen;
-        sh_above = chosen_above;
-        sh_bin = cnt[chosen];
+      // the lowest digit in use with less than the target above it (the highest in use, if none has)
+      sums_from_the_top(mass, mass_above, carry_f);
+      sums_from_the_top(cnt, cnt_above, carry_u);
+      if (tid == 0) sh_digit = 256;
+      __syncthreads();
+      if (tid < 256 && cnt[tid] > 0) {
+        const float over = above + (tid < 255 ? mass_above[tid + 1] : 0.f);     // the mass above this digit
+        const bool top = tid == 255 || cnt_above[tid + 1] == 0;                  // no digit in use above it
+        if (over < target || top) atomicMin(&sh_digit, tid);
+      }
+      __syncthreads();
+      if (tid == sh_digit) {
+        sh_above = above + (tid < 255 ? mass_above[tid + 1] : 0.f);
+        sh_bin = cnt[tid];
       }
       __syncthreads();
       prefix |= (uint64_t)sh_digit << shift;
@@ -325,8 +431,6 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     if (lane == 63) sh_total = incl;
   }
   __syncthreads();
-  // a counter below zero asks for the constant 0.5 the reference calls deterministic (hlo.py:2455-2456)
-  const float u = counters[rowi] < 0 ? 0.5f : philox_uniform((uint64_t)seeds[rowi], (uint64_t)counters[rowi]);
   const float goal = u * sh_total;
   // thread t owns [base_t, base_{t+1}): the scanned values tile the line without gaps
   const float base = part[tid];
