@@ -400,6 +400,35 @@ def test_argmax_and_sampling(vocab):
         same_or_on_a_boundary(t_h, t_r, tight_p, counters, least)
 
 
+@pytest.mark.parametrize("vocab", [1500, 50272])
+def test_sampling_after_a_top_k_with_ties(vocab):
+    """Logits in steps of a half, so that the k-th largest value is shared by many tokens (the lower ids stay),
+    at numbers of kept tokens around what the kernel gathers (256) and around a wave."""
+    import plain_opt
+    hip, ref = _ops(torch.float32)
+    g = torch.Generator(device=DEV).manual_seed(vocab + 1)
+    ks = [2, 63, 64, 65, 255, 256, 257, 1024, vocab - 1, 7]
+    rows = 3 * len(ks)
+    logits = torch.round(torch.randn(rows, vocab, device=DEV, generator=g) * 4) / 2
+    temp = torch.tensor([1.0, 0.6, 1.7] * len(ks), device=DEV)
+    top_k = torch.tensor([k for k in ks for _ in range(3)], device=DEV, dtype=torch.int32)
+    top_p = torch.tensor([1.0, 0.8, 0.3, 0.97, 0.5] * (rows // 5), device=DEV)
+    least = torch.tensor([1, 1, 5, 1, 70, 1] * (rows // 6), device=DEV, dtype=torch.int32)
+    seeds = torch.arange(rows, device=DEV, dtype=torch.int64) * 104729 + 5
+    for step in (-1, 0, 1, 2, 3):
+        counters = torch.full((rows,), step, device=DEV, dtype=torch.int64)
+        t_h = hip.sample(logits, temp, top_k, top_p, seeds, counters, least)
+        t_r = ref.sample(logits, temp, top_k, top_p, seeds, counters, least)
+        for i in range(rows):
+            values, indices = plain_opt.filter_top_k_top_p(logits[i].cpu() / float(temp[i]), int(top_k[i]),
+                                                           float(top_p[i]), int(least[i]))
+            assert int(t_h[i]) in set(indices.tolist()), f"row {i}: token {int(t_h[i])} is outside what the filters keep"
+            if int(t_h[i]) != int(t_r[i]):      # only where the random number lies on the boundary between two tokens
+                u = 0.5 if step < 0 else plain_opt.philox_uniform(int(seeds[i]), step)
+                cum = torch.cumsum(torch.softmax(values[torch.argsort(indices)].double(), -1), -1)
+                assert float((cum - u).abs().min()) < 1e-5, (i, int(t_h[i]), int(t_r[i]), u)
+
+
 def test_sampling_distribution():
     """Frequencies over many draws follow the softmax over the kept tokens."""
     hip, _ = _ops(torch.float32)

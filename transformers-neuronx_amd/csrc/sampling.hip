@@ -12,6 +12,9 @@
 TNX_DEFINE_ERROR_API
 
 #define SAMPLE_THREADS 1024
+// The most keys that are gathered in LDS and ranked against one another there (each against all: what a wave
+// reads from LDS is the limit, 256 keys take a few microseconds, 1,024 would take a hundred).
+#define SAMPLE_GATHER 256
 
 __device__ __forceinline__ uint64_t order_key(float x, int idx) {
   if (x != x) x = -INFINITY;  // NaN orders last
@@ -166,13 +169,21 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
               int vocab) {
   __shared__ unsigned int cnt[256];
   __shared__ float mass[256];
+  // Eight copies of both, a lane adding to copy lane % 8: in the first pass nearly all keys of a row fall into
+  // two or three bins, and 64 lanes adding to one word take their turns one after the other.
+  __shared__ unsigned int cnt8[256 * 8];
+  __shared__ unsigned long long mass8[256 * 8];     // in units of 2^-40: whole numbers add up in any order alike
+  const int copy = threadIdx.x & 7;
   __shared__ float part[SAMPLE_THREADS];
   __shared__ float wsum[16];
   __shared__ unsigned long long best[16];
   __shared__ int sh_digit;
   __shared__ unsigned int sh_remaining, sh_bin;
   __shared__ float sh_above, sh_total;
-  __shared__ int sh_result, sh_last, sh_n;
+  __shared__ int sh_result, sh_last, sh_n, sh_owner, sh_owner_last;
+  __shared__ unsigned long long sh_key;
+  __shared__ unsigned long long tkey[SAMPLE_GATHER], ckey[SAMPLE_GATHER];
+  __shared__ float tval[SAMPLE_GATHER];
   __shared__ unsigned int cnt_above[256], carry_u[4];
   __shared__ float mass_above[256], carry_f[4];
 
@@ -180,29 +191,39 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
   const int rowi = blockIdx.x;
   const float* row = logits + (size_t)rowi * vocab;
   const float temp = temperature[rowi];
+  const bool greedy = !(temp > 0.f);
+  const int keep = min_keep ? max(min_keep[rowi], 1) : 1;
+  int k = top_k[rowi];
+  if (k > 0) k = max(k, keep);
+  // after a top-k of no more than that, the kept tokens are gathered and the rest is done over these
+  const bool few = !greedy && k > 0 && k < vocab && k <= SAMPLE_GATHER;
+  const float inv_temp = greedy ? 0.f : 1.f / temp;
 
-  // the largest key: argmax, and the maximum for the softmax
-  uint64_t b = 0;
-  for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
-    const uint64_t k = order_key(row[i], i);
-    b = k > b ? k : b;
-  }
+  // the largest key: argmax, and the maximum for the softmax (the gathered tokens bring their own)
+  float xmax = 0.f;
+  int arg = 0;
+  if (!few) {
+    uint64_t b = 0;
+    for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
+      const uint64_t key = order_key(row[i], i);
+      b = key > b ? key : b;
+    }
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    const uint64_t other = __shfl_xor((unsigned long long)b, o, 64);
-    b = other > b ? other : b;
+    for (int o = 32; o > 0; o >>= 1) {
+      const uint64_t other = __shfl_xor((unsigned long long)b, o, 64);
+      b = other > b ? other : b;
+    }
+    if (lane == 0) best[wave] = b;
+    __syncthreads();
+    b = best[0];
+    for (int w = 1; w < 16; ++w) b = best[w] > b ? best[w] : b;
+    arg = (int)(~(uint32_t)b);
+    if (greedy) {
+      if (tid == 0) out[rowi] = arg;
+      return;
+    }
+    xmax = row[arg] * inv_temp;
   }
-  if (lane == 0) best[wave] = b;
-  __syncthreads();
-  b = best[0];
-  for (int w = 1; w < 16; ++w) b = best[w] > b ? best[w] : b;
-  const int arg = (int)(~(uint32_t)b);
-  if (!(temp > 0.f)) {
-    if (tid == 0) out[rowi] = arg;
-    return;
-  }
-  const float inv_temp = 1.f / temp;
-  const float xmax = row[arg] * inv_temp;
 
   // the k-th largest key of the row, by radix selection; every thread of the block calls it together
   auto kth_largest = [&](unsigned int k) -> uint64_t {
@@ -210,11 +231,18 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     unsigned int remaining = k;
     for (int pass = 0; pass < 8; ++pass) {
       const int shift = 56 - 8 * pass;
-      if (tid < 256) cnt[tid] = 0;
+      for (int j = tid; j < 256 * 8; j += SAMPLE_THREADS) cnt8[j] = 0;
       __syncthreads();
       for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
         const uint64_t key = order_key(row[i], i);
-        if ((key & mask) == prefix) atomicAdd(&cnt[(unsigned int)(key >> shift) & 255u], 1u);
+        if ((key & mask) == prefix) atomicAdd(&cnt8[((unsigned int)(key >> shift) & 255u) * 8 + copy], 1u);
+      }
+      __syncthreads();
+      if (tid < 256) {
+        unsigned int c = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) c += cnt8[tid * 8 + j];
+        cnt[tid] = c;
       }
       __syncthreads();
       // the digit of the `remaining`-th largest: the highest one with that many keys at or above it
@@ -231,28 +259,44 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
       prefix |= (uint64_t)sh_digit << shift;
       mask |= 0xFFull << shift;
       remaining = sh_remaining;
-      const bool whole_bin = sh_bin == remaining;
+      const unsigned int bin = sh_bin;
       __syncthreads();
-      if (whole_bin) break;  // everything under this prefix is kept: the threshold is the prefix itself
+      if (bin == remaining) break;  // everything under this prefix is kept: the threshold is the prefix itself
+      if (pass < 7 && bin <= SAMPLE_GATHER) {
+        // few keys are left under the prefix: they are gathered, and the one with remaining - 1 larger
+        // ones beside it is the threshold (keys differ, so there is exactly one)
+        if (tid == 0) sh_n = 0;
+        __syncthreads();
+        for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
+          const uint64_t key = order_key(row[i], i);
+          if ((key & mask) == prefix) tkey[atomicAdd(&sh_n, 1)] = key;
+        }
+        __syncthreads();
+        if (tid < (int)bin) {
+          const uint64_t mine = tkey[tid];
+          unsigned int larger = 0;
+          for (unsigned int j = 0; j < bin; ++j) larger += tkey[j] > mine ? 1u : 0u;
+          if (larger == remaining - 1) sh_key = mine;
+        }
+        __syncthreads();
+        prefix = sh_key;
+        __syncthreads();
+        break;
+      }
     }
     return prefix;
   };
 
   // top-k: tokens with key >= floor_key are kept; never fewer than `min_keep` (sampling.py:204-205)
   uint64_t floor_key = 0;
-  const int keep = min_keep ? max(min_keep[rowi], 1) : 1;
-  int k = top_k[rowi];
-  if (k > 0) k = max(k, keep);
   if (k > 0 && k < vocab) floor_key = kth_largest((unsigned int)k);
 
   const float p = top_p[rowi];
   // a counter below zero asks for the constant 0.5 the reference calls deterministic (hlo.py:2455-2456)
   const float u = counters[rowi] < 0 ? 0.5f : philox_uniform((uint64_t)seeds[rowi], (uint64_t)counters[rowi]);
-  if (k > 0 && k < vocab && k <= SAMPLE_THREADS) {
+  if (few) {
     // Few tokens are left, the k largest exactly (keys differ in their token ids): they are gathered, one a
     // thread, put in the order of their token ids, and top-p and the draw are made over these alone.
-    __shared__ unsigned long long tkey[SAMPLE_THREADS], ckey[SAMPLE_THREADS];
-    __shared__ float tval[SAMPLE_THREADS];
     if (tid == 0) {
       sh_n = 0;
       sh_result = -1;
@@ -263,14 +307,20 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
       const uint64_t key = order_key(row[i], i);
       if (key >= floor_key) {
         const int at = atomicAdd(&sh_n, 1);
-        if (at < SAMPLE_THREADS) {
+        if (at < SAMPLE_GATHER) {
           tkey[at] = key;
-          tval[at] = __expf(row[i] * inv_temp - xmax);
+          tval[at] = row[i] * inv_temp;
         }
       }
     }
     __syncthreads();
-    const int n = min(sh_n, SAMPLE_THREADS);
+    const int n = min(sh_n, SAMPLE_GATHER);
+    const bool mine_too = wave * 64 < n;         // a wave with none of them has nothing to find out
+    float largest = -INFINITY;
+    for (int j = 0; mine_too && j < n; ++j) largest = fmaxf(largest, tval[j]);
+    __syncthreads();
+    if (tid < n) tval[tid] = __expf(tval[tid] - largest);
+    __syncthreads();
     // of each of them: its place in the order of token ids, and the mass and the number of those with a larger key
     const bool have = tid < n;
     const uint64_t my_key = have ? tkey[tid] : 0;
@@ -278,7 +328,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     const uint32_t my_low = (uint32_t)my_key;          // the complement of the token id: larger is earlier
     float above = 0.f, z = 0.f;
     int rank = 0, place = 0;
-    for (int j = 0; j < n; ++j) {
+    for (int j = 0; mine_too && j < n; ++j) {
       const uint64_t kj = tkey[j];
       const float e = tval[j];
       z += e;
@@ -330,38 +380,65 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     return;
   }
 
-  // top-p: the smallest kept key is the last one whose predecessors hold less than p of the mass
+  // top-p: the smallest kept key is the last one whose predecessors hold less than p of the mass. The search
+  // narrows level by level, at each with a count and a mass for each of 256 bins: first bins an eighth wide
+  // of the distance below the row's maximum, then each of these in 256 (over such bins the keys of a row
+  // spread, where the first bytes of the key, sign, exponent and first fraction bits, are the same for most of
+  // them), then the bytes of the key among the tokens of the chosen bin; the first level's sums give the
+  // whole mass.
   if (p < 1.f) {
-    float z = 0.f;
-    for (int i = tid; i < vocab; i += SAMPLE_THREADS)
-      if (order_key(row[i], i) >= floor_key) z += __expf(row[i] * inv_temp - xmax);
-    z = wave_sum(z);
-    if (lane == 0) wsum[wave] = z;
-    __syncthreads();
-    z = 0.f;
-    for (int w = 0; w < 16; ++w) z += wsum[w];
-    const float target = p * z;
+    // both larger for larger values; 255, 255 for the maximum
+    auto below_max = [&](float x, int& coarse, int& fine) {
+      const float t = fmaxf((xmax - x * inv_temp) * 8.f, 0.f);
+      const float c = fminf(floorf(t), 255.f);
+      coarse = 255 - (int)c;
+      fine = 255 - (int)fminf((t - c) * 256.f, 255.f);
+    };
+    float target = 0.f;
+    int level = -1, sublevel = -1;
     uint64_t prefix = 0, mask = 0;
     float above = 0.f;
-    for (int pass = 0; pass < 8; ++pass) {
-      const int shift = 56 - 8 * pass;
-      if (tid < 256) {
-        cnt[tid] = 0;
-        mass[tid] = 0.f;
+    for (int pass = -2; pass < 8; ++pass) {
+      const int shift = 56 - 8 * max(pass, 0);
+      for (int j = tid; j < 256 * 8; j += SAMPLE_THREADS) {
+        cnt8[j] = 0;
+        mass8[j] = 0;
       }
       __syncthreads();
       for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
-        const uint64_t key = order_key(row[i], i);
-        if (key >= floor_key && (key & mask) == prefix) {
-          const unsigned int d = (unsigned int)(key >> shift) & 255u;
-          atomicAdd(&cnt[d], 1u);
-          atomicAdd(&mass[d], __expf(row[i] * inv_temp - xmax));
+        const float x = row[i];
+        const uint64_t key = order_key(x, i);
+        int coarse, fine;
+        below_max(x, coarse, fine);
+        const bool in = pass == -2 || (coarse == level && (pass == -1 || (fine == sublevel && (key & mask) == prefix)));
+        if (key >= floor_key && in) {
+          const unsigned int digit = pass == -2 ? coarse : pass == -1 ? fine : (unsigned int)(key >> shift) & 255u;
+          const unsigned int d = digit * 8 + copy;
+          atomicAdd(&cnt8[d], 1u);
+          // at most 1, as 24 bits before and 16 bits behind the point of e * 2^24
+          const float e24 = __expf(x * inv_temp - xmax) * 16777216.f;
+          const uint32_t whole = (uint32_t)e24;
+          const uint32_t rest = (uint32_t)((e24 - (float)whole) * 65536.f);
+          atomicAdd(&mass8[d], ((unsigned long long)whole << 16) + rest);
         }
+      }
+      __syncthreads();
+      if (tid < 256) {
+        unsigned int c = 0;
+        unsigned long long m = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          c += cnt8[tid * 8 + j];
+          m += mass8[tid * 8 + j];
+        }
+        cnt[tid] = c;
+        mass[tid] = (float)m * 9.094947017729282e-13f;        // 2^-40
       }
       __syncthreads();
       // the lowest digit in use with less than the target above it (the highest in use, if none has)
       sums_from_the_top(mass, mass_above, carry_f);
       sums_from_the_top(cnt, cnt_above, carry_u);
+      if (pass == -2) target = p * mass_above[0];
       if (tid == 0) sh_digit = 256;
       __syncthreads();
       if (tid < 256 && cnt[tid] > 0) {
@@ -375,12 +452,54 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
         sh_bin = cnt[tid];
       }
       __syncthreads();
-      prefix |= (uint64_t)sh_digit << shift;
-      mask |= 0xFFull << shift;
+      if (pass == -2) {
+        level = sh_digit;
+      } else if (pass == -1) {
+        sublevel = sh_digit;
+      } else {
+        prefix |= (uint64_t)sh_digit << shift;
+        mask |= 0xFFull << shift;
+      }
       above = sh_above;
-      const bool single = sh_bin == 1;
+      const unsigned int bin = sh_bin;
       __syncthreads();
-      if (single) break;
+      if (pass >= 0 && bin == 1) break;
+      if (pass < 7 && bin <= SAMPLE_GATHER) {
+        // few keys are left in the bin: they are gathered with their masses, and the threshold is the lowest
+        // of them with less than the target above it (the largest of them has: its bin was chosen so)
+        if (tid == 0) {
+          sh_n = 0;
+          sh_key = ~0ull;
+        }
+        __syncthreads();
+        for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
+          const float x = row[i];
+          const uint64_t key = order_key(x, i);
+          int coarse, fine;
+          below_max(x, coarse, fine);
+          if (key >= floor_key && coarse == level && (sublevel < 0 || fine == sublevel) && (key & mask) == prefix) {
+            const int at = atomicAdd(&sh_n, 1);
+            tkey[at] = key;
+            tval[at] = __expf(x * inv_temp - xmax);
+          }
+        }
+        __syncthreads();
+        if (tid < (int)bin) {
+          const uint64_t mine = tkey[tid];
+          float over = above;
+          bool top = true;
+          for (unsigned int j = 0; j < bin; ++j)
+            if (tkey[j] > mine) {
+              over += tval[j];
+              top = false;
+            }
+          if (over < target || top) atomicMin(&sh_key, (unsigned long long)mine);
+        }
+        __syncthreads();
+        prefix = sh_key;
+        __syncthreads();
+        break;
+      }
     }
     uint64_t by_mass = prefix > floor_key ? prefix : floor_key;
     if (keep > 1) {
@@ -393,19 +512,40 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     floor_key = by_mass;
   }
 
-  // the draw, over the kept tokens in ascending order of token id; thread t owns a contiguous segment
-  const int seg = (vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
-  const int i0 = tid * seg, i1 = min(vocab, i0 + seg);
+  // the draw, over the kept tokens in ascending order of token id; thread t owns a contiguous segment, which
+  // it reads four floats a load: segments are counted from the 16-byte boundary at or before the row's start
+  // (`lead` floats before it), and a group of four that reaches outside the row is read one by one
+  const int lead = (int)(((uintptr_t)row >> 2) & 3);
+  const int seg = (((vocab + lead + SAMPLE_THREADS - 1) / SAMPLE_THREADS) + 3) & ~3;
+  const int i0 = tid * seg - lead;           // may lie before the row or beyond it
+  auto four = [&](int i, float (&x)[4]) {
+    if (i >= 0 && i + 3 < vocab) {
+      const float4 v = *(const float4*)(row + i);
+      x[0] = v.x, x[1] = v.y, x[2] = v.z, x[3] = v.w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[e] = i + e >= 0 && i + e < vocab ? row[i + e] : 0.f;
+    }
+  };
   float s = 0.f;
   int last = -1;
-  for (int i = i0; i < i1; ++i)
-    if (order_key(row[i], i) >= floor_key) {
-      s += __expf(row[i] * inv_temp - xmax);
-      last = i;
+#pragma unroll 4
+  for (int q = 0; q < seg; q += 4) {
+    float x[4];
+    four(i0 + q, x);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int i = i0 + q + e;
+      if (i >= 0 && i < vocab && order_key(x[e], i) >= floor_key) {
+        s += __expf(x[e] * inv_temp - xmax);
+        last = i;
+      }
     }
+  }
   if (tid == 0) {
     sh_result = -1;
     sh_last = -1;
+    sh_owner = -1;
   }
   part[tid] = s;
   __syncthreads();
@@ -435,21 +575,36 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
   // thread t owns [base_t, base_{t+1}): the scanned values tile the line without gaps
   const float base = part[tid];
   const float next = tid + 1 < SAMPLE_THREADS ? part[tid + 1] : INFINITY;
+  // its owner's segment is walked by the first wave, 64 tokens a turn: one trip to memory where the owner alone
+  // would make one for every four tokens, each waiting for the one before
   if (last >= 0 && base <= goal && goal < next) {
-    float run = base;
-    int pick = last;
-    for (int i = i0; i < i1; ++i)
-      if (order_key(row[i], i) >= floor_key) {
-        run += __expf(row[i] * inv_temp - xmax);
-        if (run > goal) {
-          pick = i;
-          break;
-        }
-      }
-    atomicMax(&sh_result, pick);
+    sh_owner = tid;
+    sh_owner_last = last;
   }
   __syncthreads();
-  if (tid == 0) out[rowi] = sh_result >= 0 ? sh_result : sh_last;
+  if (wave == 0 && sh_owner >= 0) {
+    const int o0 = sh_owner * seg - lead;
+    float run = part[sh_owner];
+    int pick = -1;
+    for (int q = 0; q < seg && pick < 0; q += 64) {
+      const int i = o0 + q + lane;
+      const bool ok = q + lane < seg && i >= 0 && i < vocab;
+      const float x = ok ? row[i] : 0.f;
+      const bool kept = ok && order_key(x, i) >= floor_key;
+      float incl = kept ? __expf(x * inv_temp - xmax) : 0.f;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const float v = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += v;
+      }
+      const unsigned long long hit = __ballot(kept && run + incl > goal);
+      if (hit) pick = o0 + q + __ffsll(hit) - 1;
+      run += __shfl(incl, 63, 64);
+    }
+    if (lane == 0) sh_result = pick >= 0 ? pick : sh_owner_last;
+  }
+  __syncthreads();
+  if (tid == 0) out[rowi] = sh_result >= 0 ? sh_result : sh_last >= 0 ? sh_last : arg;
 }
 
 extern "C" int tnx_sample(const float* logits, const float* temperature, const int* top_k, const float* top_p,
