@@ -96,6 +96,30 @@ def test_generation_with_few_pages_float32(tiny_folders, name, run_ahead):
     _check_exact(results["tight"], prompts, params, weights, cfg)
 
 
+def test_every_way_of_choosing_a_token_in_one_batch_float32(tiny_folders):
+    """Requests that differ in how their tokens are chosen, side by side in every step: greedy, top-p alone, a
+    top-k beyond what the sampler gathers with top-p, a small top-k alone, a top-p so tight that the least
+    number of tokens to keep decides, and the plain softmax. Each takes its own way through the sampling
+    kernel; all are the plain implementation's tokens."""
+    from transformers_neuronx_amd.sampling import SamplingParams
+    folder, cfg, weights = tiny_folders["B"]
+    prompts = _prompts(cfg["vocab_size"], [7, 30, 2, 55, 18, 41], 77)
+    params = [SamplingParams(max_new_tokens=20, do_sample=False, ignore_eos=True),
+              SamplingParams(max_new_tokens=20, temperature=1.1, top_p=0.7, seed=11, ignore_eos=True),
+              SamplingParams(max_new_tokens=20, temperature=0.9, top_k=300, top_p=0.95, seed=12, ignore_eos=True),
+              SamplingParams(max_new_tokens=20, temperature=1.4, top_k=5, seed=13, ignore_eos=True),
+              SamplingParams(max_new_tokens=20, temperature=1.3, top_p=0.05, min_tokens_to_keep=4, seed=14,
+                             ignore_eos=True),
+              SamplingParams(max_new_tokens=20, temperature=0.7, seed=15, ignore_eos=True)]
+    engine, runner = _engine(folder, "float32", page_size=16, max_tokens=640, max_num_seqs=6,
+                             max_num_batched_tokens=64, use_graphs=True)
+    outs = engine.generate(prompts, params)
+    runner.cache.check()
+    assert not runner.cache.requests and not engine.requests
+    assert all(len(o) == 20 for o in outs)
+    _check_exact(outs, prompts, params, weights, cfg)
+
+
 @pytest.mark.parametrize("prompts_first", [False, True])
 def test_late_end_of_sequence_and_arrivals_float32(tiny_folders, prompts_first):
     """Requests that stop at a token they generate (found out a step late when steps run ahead), others
