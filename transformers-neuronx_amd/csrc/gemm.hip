@@ -774,6 +774,35 @@ static void launch_skinny(const bf16_t* xp, const bf16_t* wp, const bf16_t* ws, 
                                                                                   out_dtype, act, M, N, K, none, plain);
 }
 
+// How many tiles of 16 weight rows a block of the few-rows kernel takes (1, 2 or 3). Every block reads all of
+// `x`, so fewer and larger blocks read less of it (normalised rows, which are float32, most of all); what
+// decides is how evenly the blocks fall on the compute units, which take them in turns: the most tiles that a
+// unit gets, ceil(blocks / units) * tiles, is what the launch takes, and among equals the larger blocks win
+// (12,288 columns on 256 units: 768, 384 or 256 blocks, 3, 4 or 3 tiles a unit: 21.2 us with one tile a block,
+// 20.5 with three; 9,216 columns and K = 36,864: 576, 288 or 192 blocks, again 3, 4 or 3: 139, 159 and 114 us).
+// With blocks for four rounds or more the units even out by themselves. Three tiles up to 16 rows of `x`.
+static int skinny_tiles_per_block(int M, int N) {
+  if (M > 32) return 1;
+  const int units = tnx_compute_units();
+  const int tiles = (N + 15) / 16;
+  int best = 1, best_load = (tiles + units - 1) / units;
+  for (int rt = 2; rt <= (M <= 16 ? 3 : 2); ++rt) {
+    const int blocks = (tiles + rt - 1) / rt;
+    if (blocks >= 4 * units) {
+      best = rt;
+      continue;
+    }
+    const int load = (blocks + units - 1) / units * rt;
+    if (2 * blocks >= units && load <= best_load) {
+      best = rt;
+      best_load = load;
+    }
+  }
+  return best;
+}
+
+extern "C" int tnx_gemm_skinny_tiles_per_block(int M, int N) { return skinny_tiles_per_block(M, N); }
+
 static int gemm_bf16_dispatch(const void* x, const void* w, const void* w_tiles, const float* bias,
                               const float* residual, void* out, int out_dtype, int act, int M, int N, int K,
                               int force_tiled, const QkvScatter* sc, hipStream_t stream,
@@ -801,17 +830,7 @@ static int gemm_bf16_dispatch(const void* x, const void* w, const void* w_tiles,
     // enough to share (more bytes in flight for each of the few blocks). Two weight tiles a block for wide
     // matrices. force_tiled 4 or 8 picks the wave count and 2 the two tiles, for measurements and tests.
     const int waves = force_tiled == 4 || force_tiled == 8 ? force_tiled : (N < 4096 && K >= 2048 ? 8 : 4);
-    // Two or three tiles of weight rows a block where the blocks still fill the chip in whole rounds: every
-    // block reads all of `x`, so fewer blocks read less (up to 16 rows, 12,288 columns on 256 compute
-    // units: 21.2 -> 20.5 us with three tiles, and 27.8 -> 22.7 for normalised rows, which are float32)
-    int tiles_per_block = 1;
-    if (force_tiled == 0 && waves == 4 && M <= 32) {
-      const int units = tnx_compute_units();
-      for (int rt = (M <= 16 ? 3 : 2); rt >= 2 && tiles_per_block == 1; --rt) {
-        const int blocks = (N + 16 * rt - 1) / (16 * rt), rounds = (blocks + units - 1) / units;
-        if (blocks >= 4 * units || (blocks >= units && blocks * 20 >= rounds * units * 19)) tiles_per_block = rt;
-      }
-    }
+    const int tiles_per_block = force_tiled == 0 && waves == 4 ? skinny_tiles_per_block(M, N) : 1;
     const bool two_tiles = force_tiled == 2 || tiles_per_block == 2;
     const bool three_tiles = tiles_per_block == 3;
 #define SKINNY(MT, WV, RT) \

@@ -40,6 +40,7 @@ _SIGNATURES = {
         "tnx_gemm_bf16_qkv": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
                               _c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int,
                               _c_int, _c_void_p],
+        "tnx_gemm_skinny_tiles_per_block": [_c_int, _c_int],
         "tnx_gemm_bf16_mid": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                               _c_int, _c_void_p, ctypes.c_size_t, _c_int, _c_int, _c_void_p],
         "tnx_gemm_library": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
@@ -222,6 +223,7 @@ class HipOps:
         self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         self._bias_copies = {}
         self._later = []
+        self._tiles_per_block = {}
         self._landing, self._landing_turn = [None, None], 0
         self._ints, self._ints_done, self._ints_turn = [None, None], [None, None], 0
 
@@ -375,8 +377,19 @@ class HipOps:
     # (measured at 4,096 -> 12,288: 23.0 us against 24.4 for norm and product at 8 rows, but 25.8 against 25.2 at
     # 16 and twice the time at 32: every block reads all rows, and these are float32); beyond that, as far as
     # the few-rows kernel goes, the norm's kernel normalises and the folded copy does the rest.
+    # Where the blocks take one tile of weight rows each (what `tnx_gemm_skinny_tiles_per_block` says), every
+    # 32 bytes of weight come with 64 of float32 rows and the norm's own kernel is the cheaper way again
+    # (9,216 -> 27,648 at 8 rows: 120 us against 10 + 91).
     fuse_norm = True
     fuse_norm_rows = 8
+
+    def _norm_in_the_product(self, m, n) -> bool:
+        if m > self.fuse_norm_rows:
+            return False
+        key = (m, n)
+        if key not in self._tiles_per_block:
+            self._tiles_per_block[key] = library("gemm").tnx_gemm_skinny_tiles_per_block(m, n)
+        return self._tiles_per_block[key] >= 2
     few_rows = 32           # the few-rows kernel takes up to this many rows
 
     def fold_norm(self, w, weight, bias) -> bool:
@@ -433,9 +446,9 @@ class HipOps:
 
     def finish_weights(self, budget_bytes: int) -> int:
         """The tile-ordered copies that `budget_bytes` allow, of the matrices that waited for them: those
-        with the fewest rows first (measured at OPT-66B sizes, 8 rows: the copy saves 8 us of 45 for
-        9,216 x 9,216, 27 of 165 for 9,216 x 36,864, 16 of 105 for 27,648 x 9,216 and 5 of 121 for
-        36,864 x 9,216, that is 47, 39, 31 and 8 us a GB). Returns the bytes taken."""
+        with the fewest rows first (measured at OPT-66B sizes, 8 rows: the copy saves 5 us of 37 for
+        9,216 x 9,216, 20 of 134 for 9,216 x 36,864, 14 of 105 for 27,648 x 9,216 and 6 of 121 for
+        36,864 x 9,216, that is 29, 29, 28 and 8 us a GB). Returns the bytes taken."""
         taken = 0
         waiting, self._later = self._later, []
         for pw in sorted(waiting, key=lambda pw: pw.tensor.shape[0]):      # (stable: layer order within a size)
@@ -453,7 +466,7 @@ class HipOps:
                 folded = None
             if folded is None:
                 x = x.materialize()
-            elif x.shape[0] > self.fuse_norm_rows:
+            elif not self._norm_in_the_product(x.shape[0], w.tensor.shape[0]):
                 # the norm's kernel without weight and bias, then the plain product of the folded copy
                 m, k = x.shape
                 n = w.tensor.shape[0]
@@ -641,7 +654,7 @@ class HipOps:
                 folded = None
             if folded is None:
                 h = h.materialize()
-            elif h.shape[0] > self.fuse_norm_rows:
+            elif not self._norm_in_the_product(h.shape[0], w.tensor.shape[0]):
                 # the norm's kernel without weight and bias, then the fused projection of the folded copy
                 h, w, bias = h.normalised(), PreparedWeight(w.tensor, folded.tiles), folded.d_with(bias)
             else:
