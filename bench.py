@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine at OPT-6.7B size with random weights.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--model 6.7b|350m|66b] [--mix]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--model 6.7b|350m|1.3b|2.7b|13b|30b|66b] [--mix]
 
 One JSON line: `value` is decoded tokens per second at batch 8 and a 2,048-token context
 (a "step" is one decode step of the whole engine: schedule, model, sampling);
@@ -28,10 +28,14 @@ MODEL = dict(architectures=["OPTForCausalLM"], model_type="opt", vocab_size=5027
              num_hidden_layers=32, num_attention_heads=32, ffn_dim=16384, max_position_embeddings=2048,
              word_embed_proj_dim=4096, do_layer_norm_before=True, activation_function="relu", enable_bias=True,
              layer_norm_elementwise_affine=True, init_std=0.02, torch_dtype="bfloat16")
-# Two more members of the family, for `--model` (the default run and its JSON line stay OPT-6.7B)
+# More members of the family, for `--model` (the default run and its JSON line stay OPT-6.7B)
 OTHER_MODELS = {
     "350m": dict(hidden_size=1024, num_hidden_layers=24, num_attention_heads=16, ffn_dim=4096, word_embed_proj_dim=512,
                  do_layer_norm_before=False),
+    "1.3b": dict(hidden_size=2048, num_hidden_layers=24, num_attention_heads=32, ffn_dim=8192, word_embed_proj_dim=2048),
+    "2.7b": dict(hidden_size=2560, num_hidden_layers=32, num_attention_heads=32, ffn_dim=10240, word_embed_proj_dim=2560),
+    "13b": dict(hidden_size=5120, num_hidden_layers=40, num_attention_heads=40, ffn_dim=20480, word_embed_proj_dim=5120),
+    "30b": dict(hidden_size=7168, num_hidden_layers=48, num_attention_heads=56, ffn_dim=28672, word_embed_proj_dim=7168),
     "66b": dict(hidden_size=9216, num_hidden_layers=64, num_attention_heads=72, ffn_dim=36864, word_embed_proj_dim=9216),
 }
 CONTEXT = 2048
@@ -61,7 +65,7 @@ def main():
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--prefill-only", action="store_true", help="measure the prompt step alone (for profiles)")
     ap.add_argument("--model", default="6.7b", choices=["6.7b"] + sorted(OTHER_MODELS),
-                    help="layer sizes: OPT-6.7B (the measurement of record), OPT-350m or OPT-66B")
+                    help="layer sizes: OPT-6.7B (the measurement of record) or another member of the family")
     ap.add_argument("--do-sample", action="store_true",
                     help="decode with temperature 0.8, top-k 50 and top-p 0.95 instead of greedily")
     ap.add_argument("--mix", action="store_true",

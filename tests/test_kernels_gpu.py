@@ -757,3 +757,22 @@ def test_product_of_some_rows(m, n, k):
     with pytest.raises(RuntimeError, match="1 to 128 rows"):
         hip.call("gemm", "tnx_gemm_bf16_mid", _ptr(x), _ptr(pw.tiles), None, None, _ptr(out), _code(out.dtype), 0, 129,
                  n, k, None, 0, 0, 0, _stream())
+
+
+def test_which_products_of_some_rows_go_to_our_kernel():
+    """The rule of `linear` at the sizes it was measured at (256 compute units): blocks of 64 columns, K shared
+    out until every unit has a block at most, taken where three units in four get one."""
+    from transformers_neuronx_amd.kernels.hip import HipOps
+    hip = HipOps(torch.bfloat16, DEV)
+    if hip.compute_units != 256:
+        pytest.skip("the cases are those of 256 compute units")
+    w = torch.empty(0, dtype=torch.bfloat16)
+    res = object()
+    rule = lambda m, n, k, r: hip._some_rows_product(m, n, k, w, w, r, True, 0)
+    assert rule(24, 4096, 4096, res) and rule(128, 4096, 16384, res)          # 64 column blocks, 4 shares
+    assert rule(32, 5120, 20480, res) and rule(128, 7168, 28672, res)         # 80 x 3 and 112 x 2 blocks
+    assert not rule(40, 9216, 36864, res) and not rule(64, 9216, 9216, res)   # 144 blocks, and 288 would be ragged
+    assert not rule(20, 1024, 1024, res) and rule(40, 1024, 1024, res)        # small: one launch up to 32 rows
+    assert rule(17, 50272, 4096, None) and rule(64, 50272, 4096, None) and not rule(65, 50272, 4096, None)
+    assert not rule(16, 4096, 4096, res) and not rule(129, 4096, 4096, res)
+    assert not hip._some_rows_product(64, 4096, 4096, w, None, res, True, 0)  # no tile-ordered copy

@@ -605,19 +605,29 @@ class HipOps:
             self._bias_copies[bias.data_ptr()] = kept
         return kept[1]
 
-    # Products of 33 to 128 rows with a float32 result (those that end in the residual sum, and the head): the
-    # vendor library's kernels for such sizes leave much of the memory's rate unused where the output is small
-    # (4,096 columns, K of 16,384, 64 rows: 41 us against 31 here; at 9,216 columns the library is as good or
-    # better), and the head never goes to the library (50,272 columns, 64 rows: 156 us on the tiled kernel
-    # against 117 here; at 128 rows every block's reading of all rows costs more than it saves).
+    # Products of 17 to 128 rows with a float32 result (those that end in the residual sum, and the head): the
+    # vendor library's kernels for such sizes leave much of the memory's rate unused (4,096 columns, K of
+    # 16,384, 64 rows: 41 us against 31 here; 5,120 columns, K of 20,480, 32 rows: 68 against 41). Our kernel
+    # gives a block 64 columns and shares K out until every compute unit has a block at most, so it is taken
+    # where that leaves three units in four with one (9,216 columns make 144 blocks on 256 units, and there
+    # the library is as good or better: 147 us against 195 at K of 36,864 and 64 rows), for matrices small
+    # enough that the launches count and not the bytes, and for the head up to 64 rows (50,272 columns, more
+    # column blocks than units; at 128 rows every block's reading of all rows costs more than it saves). Up to
+    # 32 rows a small matrix stays with the few-rows kernel, one launch.
     some_rows = True
-    some_rows_outputs = 1 << 19
 
     def _some_rows_product(self, m, n, k, w, tiles, residual, out_f32, force_tiled) -> bool:
-        if not (self.some_rows and tiles is not None and self.few_rows < m <= 128 and out_f32 and not force_tiled
+        if not (self.some_rows and tiles is not None and 16 < m <= 128 and out_f32 and not force_tiled
                 and self.dtype == torch.bfloat16 and w.dtype == torch.bfloat16):
             return False
-        return n * (-(-m // 16) * 16) <= self.some_rows_outputs or (residual is None and m <= 64)
+        small = n * k <= self.small_matrix
+        if m <= self.few_rows and small:
+            return False
+        column_blocks = -(-n // 64)
+        if column_blocks > self.compute_units:
+            return residual is None and m <= 64
+        shares = max(1, min(self.compute_units // column_blocks, k // 512))     # as the kernel shares K out
+        return small or 4 * column_blocks * shares >= 3 * self.compute_units
 
     def _library_product(self, m, n, k, w, force_tiled) -> bool:
         if not (self.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and self.library_rows > 0
