@@ -775,27 +775,32 @@ static void launch_skinny(const bf16_t* xp, const bf16_t* wp, const bf16_t* ws, 
 }
 
 // How many tiles of 16 weight rows a block of the few-rows kernel takes (1, 2 or 3). Every block reads all of
-// `x`, so fewer and larger blocks read less of it (normalised rows, which are float32, most of all); what
-// decides is how evenly the blocks fall on the compute units, which take them in turns: the most tiles that a
-// unit gets, ceil(blocks / units) * tiles, is what the launch takes, and among equals the larger blocks win
-// (12,288 columns on 256 units: 768, 384 or 256 blocks, 3, 4 or 3 tiles a unit: 21.2 us with one tile a block,
-// 20.5 with three; 9,216 columns and K = 36,864: 576, 288 or 192 blocks, again 3, 4 or 3: 139, 159 and 114 us).
-// With blocks for four rounds or more the units even out by themselves. Three tiles up to 16 rows of `x`.
+// `x`, so fewer and larger blocks read less of it; what decides is how evenly the blocks fall on the compute
+// units, which take them in turns: the launch takes what the fullest unit gets, ceil(blocks / units) blocks of
+// `tiles` tiles and one reading of `x` each, which costs about a fortieth of a tile for every row of `x`
+// (lanes beyond the last row read it again, from the cache), and among equals the larger blocks win.
+// 12,288 columns on 256 units: 768, 384 or 256 blocks, 3, 4 or 3 tiles a unit: 21.2 us with one tile a block,
+// 20.5 with three; 9,216 columns and K = 36,864: 576, 288 or 192 blocks, again 3, 4 or 3: 139, 159 and 114 us;
+// 20,480 columns, K = 5,120: 5, 6 and 6 tiles a unit, and one tile a block is quickest at 8 rows (39.6 us
+// against 41.3 with three), three tiles at 16 rows (45.7 against 48.9 with one). With blocks for four rounds or
+// more the units even out by themselves. Three tiles up to 16 rows of `x`, two up to 32.
 static int skinny_tiles_per_block(int M, int N) {
   if (M > 32) return 1;
   const int units = tnx_compute_units();
   const int tiles = (N + 15) / 16;
-  int best = 1, best_load = (tiles + units - 1) / units;
+  const float x_cost = 0.025f * (float)min(M, 16);
+  int best = 1;
+  float best_cost = (float)((tiles + units - 1) / units) * (1.f + x_cost);
   for (int rt = 2; rt <= (M <= 16 ? 3 : 2); ++rt) {
     const int blocks = (tiles + rt - 1) / rt;
     if (blocks >= 4 * units) {
       best = rt;
       continue;
     }
-    const int load = (blocks + units - 1) / units * rt;
-    if (2 * blocks >= units && load <= best_load) {
+    const float cost = (float)((blocks + units - 1) / units) * ((float)rt + x_cost);
+    if (2 * blocks >= units && cost <= best_cost + 1e-3f) {
       best = rt;
-      best_load = load;
+      best_cost = cost;
     }
   }
   return best;
