@@ -429,6 +429,31 @@ def test_sampling_after_a_top_k_with_ties(vocab):
                 assert float((cum - u).abs().min()) < 1e-5, (i, int(t_h[i]), int(t_r[i]), u)
 
 
+def test_sampling_with_logits_that_are_no_numbers():
+    """A NaN orders last and has no weight: the draw is the one over the same row with -inf in its place, on
+    every way through the kernel, and never lands on it."""
+    hip, _ = _ops(torch.float32)
+    vocab, rows = 3000, 12
+    g = torch.Generator(device=DEV).manual_seed(5)
+    clean = torch.randn(rows, vocab, device=DEV, generator=g) * 2
+    holes = torch.rand(rows, vocab, device=DEV, generator=g) < 0.05
+    holes[:, 0] = True
+    clean[holes] = -float("inf")
+    dirty = clean.clone()
+    dirty[holes] = float("nan")
+    temp = torch.tensor([0.0, 1.0, 0.7, 1.3] * 3, device=DEV)
+    top_k = torch.tensor([0, 0, 40, 500, 0, 5], device=DEV, dtype=torch.int32).repeat(2)
+    top_p = torch.tensor([1.0, 0.9, 0.5, 0.95], device=DEV).repeat(3)
+    seeds = torch.arange(rows, device=DEV, dtype=torch.int64) + 77
+    for step in range(5):
+        counters = torch.full((rows,), step, device=DEV, dtype=torch.int64)
+        a = hip.sample(dirty, temp, top_k, top_p, seeds, counters)
+        b = hip.sample(clean, temp, top_k, top_p, seeds, counters)
+        assert torch.equal(a, b)
+        assert not holes[torch.arange(rows, device=DEV), a.long()].any()
+    assert torch.equal(hip.argmax(dirty), hip.argmax(clean))
+
+
 def test_sampling_distribution():
     """Frequencies over many draws follow the softmax over the kept tokens."""
     hip, _ = _ops(torch.float32)

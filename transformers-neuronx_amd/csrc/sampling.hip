@@ -5,8 +5,9 @@
 // Order among tokens is total: by logit, ties to the lower token id (a 64-bit key: ordered logit bits above
 // the inverted token id). Top-k keeps the k largest keys. Top-p keeps, of those, every token whose
 // predecessors in descending order hold less than top_p of the softmax mass (the first token always).
-// Both thresholds are found by radix selection, eight bits at a time, without sorting. The draw runs over
-// the kept tokens in ascending order of token id.
+// Both thresholds are found without sorting, by narrowing level by level with 256 bins a level (the bytes of
+// the key; for top-p first the distance below the row's maximum), until few enough keys are left to rank in
+// LDS. The draw runs over the kept tokens in ascending order of token id.
 #include "common.h"
 
 TNX_DEFINE_ERROR_API
@@ -161,7 +162,7 @@ __device__ __forceinline__ void sums_from_the_top(const T* x, T* out, T* carry) 
   __syncthreads();
 }
 
-// One block per row.
+// One block per row; a row with temperature 0 takes its argmax.
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature, const int* __restrict__ top_k,
               const float* __restrict__ top_p, const long long* __restrict__ seeds,
@@ -175,7 +176,6 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
   __shared__ unsigned long long mass8[256 * 8];     // in units of 2^-40: whole numbers add up in any order alike
   const int copy = threadIdx.x & 7;
   __shared__ float part[SAMPLE_THREADS];
-  __shared__ float wsum[16];
   __shared__ unsigned long long best[16];
   __shared__ int sh_digit;
   __shared__ unsigned int sh_remaining, sh_bin;
@@ -195,7 +195,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
   const int keep = min_keep ? max(min_keep[rowi], 1) : 1;
   int k = top_k[rowi];
   if (k > 0) k = max(k, keep);
-  // after a top-k of no more than that, the kept tokens are gathered and the rest is done over these
+  // after a top-k of no more than SAMPLE_GATHER the kept tokens are gathered and the rest is done over these
   const bool few = !greedy && k > 0 && k < vocab && k <= SAMPLE_GATHER;
   const float inv_temp = greedy ? 0.f : 1.f / temp;
 
@@ -224,6 +224,9 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     }
     xmax = row[arg] * inv_temp;
   }
+
+  // a token's share of the softmax before it is divided by the sum; a NaN has none, as it orders last
+  auto weight = [&](float x) -> float { return x != x ? 0.f : __expf(x * inv_temp - xmax); };
 
   // the k-th largest key of the row, by radix selection; every thread of the block calls it together
   auto kth_largest = [&](unsigned int k) -> uint64_t {
@@ -309,7 +312,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
         const int at = atomicAdd(&sh_n, 1);
         if (at < SAMPLE_GATHER) {
           tkey[at] = key;
-          tval[at] = row[i] * inv_temp;
+          tval[at] = row[i] != row[i] ? -INFINITY : row[i] * inv_temp;
         }
       }
     }
@@ -319,7 +322,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     float largest = -INFINITY;
     for (int j = 0; mine_too && j < n; ++j) largest = fmaxf(largest, tval[j]);
     __syncthreads();
-    if (tid < n) tval[tid] = __expf(tval[tid] - largest);
+    if (tid < n) tval[tid] = largest == -INFINITY ? 1.f : __expf(tval[tid] - largest);     // (all -inf: alike)
     __syncthreads();
     // of each of them: its place in the order of token ids, and the mass and the number of those with a larger key
     const bool have = tid < n;
@@ -389,6 +392,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
   if (p < 1.f) {
     // both larger for larger values; 255, 255 for the maximum
     auto below_max = [&](float x, int& coarse, int& fine) {
+      if (x != x) x = -INFINITY;      // as in the order of the keys
       const float t = fmaxf((xmax - x * inv_temp) * 8.f, 0.f);
       const float c = fminf(floorf(t), 255.f);
       coarse = 255 - (int)c;
@@ -416,7 +420,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
           const unsigned int d = digit * 8 + copy;
           atomicAdd(&cnt8[d], 1u);
           // at most 1, as 24 bits before and 16 bits behind the point of e * 2^24
-          const float e24 = __expf(x * inv_temp - xmax) * 16777216.f;
+          const float e24 = weight(x) * 16777216.f;
           const uint32_t whole = (uint32_t)e24;
           const uint32_t rest = (uint32_t)((e24 - (float)whole) * 65536.f);
           atomicAdd(&mass8[d], ((unsigned long long)whole << 16) + rest);
@@ -480,7 +484,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
           if (key >= floor_key && coarse == level && (sublevel < 0 || fine == sublevel) && (key & mask) == prefix) {
             const int at = atomicAdd(&sh_n, 1);
             tkey[at] = key;
-            tval[at] = __expf(x * inv_temp - xmax);
+            tval[at] = weight(x);
           }
         }
         __syncthreads();
@@ -537,7 +541,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     for (int e = 0; e < 4; ++e) {
       const int i = i0 + q + e;
       if (i >= 0 && i < vocab && order_key(x[e], i) >= floor_key) {
-        s += __expf(x[e] * inv_temp - xmax);
+        s += weight(x[e]);
         last = i;
       }
     }
@@ -591,7 +595,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
       const bool ok = q + lane < seg && i >= 0 && i < vocab;
       const float x = ok ? row[i] : 0.f;
       const bool kept = ok && order_key(x, i) >= floor_key;
-      float incl = kept ? __expf(x * inv_temp - xmax) : 0.f;
+      float incl = kept ? weight(x) : 0.f;
 #pragma unroll
       for (int o = 1; o < 64; o <<= 1) {
         const float v = __shfl_up(incl, o, 64);
