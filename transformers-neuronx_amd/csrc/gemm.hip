@@ -831,10 +831,10 @@ static int gemm_bf16_dispatch(const void* x, const void* w, const void* w_tiles,
   // The few-rows kernel up to 32 rows (beyond that every block reading all of `x` again costs more than the
   // tiles' detour through LDS: 245 against 151 us for the 50,272 x 4,096 head at 64 rows), or when asked for.
   if ((M <= 32 || ((force_tiled == 4 || force_tiled == 8) && M <= 64)) && force_tiled != 1) {
-    // Four waves a block; eight when the blocks are fewer than the compute units and the sum over K is long
-    // enough to share (more bytes in flight for each of the few blocks). Two weight tiles a block for wide
-    // matrices. force_tiled 4 or 8 picks the wave count and 2 the two tiles, for measurements and tests.
-    const int waves = force_tiled == 4 || force_tiled == 8 ? force_tiled : (N < 4096 && K >= 2048 ? 8 : 4);
+    // Four waves a block (eight, for the few blocks of a narrow matrix with a long K, are no quicker anywhere
+    // and 5 to 8 % slower at 2,048 x 8,192 to 3,072 x 12,288). force_tiled 4 or 8 picks the wave count and 2
+    // or 3 the tiles a block, for measurements and tests.
+    const int waves = force_tiled == 8 ? 8 : 4;
     const int tiles_per_block = force_tiled == 0 && waves == 4 ? skinny_tiles_per_block(M, N) : 1;
     const bool two_tiles = force_tiled == 2 || tiles_per_block == 2;
     const bool three_tiles = tiles_per_block == 3;
