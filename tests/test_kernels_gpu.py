@@ -784,6 +784,24 @@ def test_product_of_some_rows(m, n, k):
                  n, k, None, 0, 0, 0, _stream())
 
 
+def test_tiles_a_block_of_the_few_rows_product():
+    """The choice at the sizes it was measured at (256 compute units): what the fullest unit gets, with the
+    reading of `x` counted, and the larger blocks among equals."""
+    from transformers_neuronx_amd.kernels.hip import HipOps, library
+    hip = HipOps(torch.bfloat16, DEV)
+    if hip.compute_units != 256:
+        pytest.skip("the cases are those of 256 compute units")
+    rule = library("gemm").tnx_gemm_skinny_tiles_per_block
+    assert [rule(8, n) for n in (12288, 16384, 4096, 50272)] == [3, 2, 1, 3]          # OPT-6.7B and the head
+    assert [rule(8, n) for n in (27648, 9216, 36864)] == [1, 3, 3]                     # OPT-66B
+    assert [rule(8, n) for n in (15360, 5120, 20480)] == [2, 2, 1]                     # OPT-13B
+    assert rule(16, 20480) == 3 and rule(16, 28672) == 2 and rule(8, 28672) == 1       # 16 rows read twice the `x`
+    assert rule(24, 12288) <= 2 and rule(33, 12288) == 1 and rule(8, 288) == 1
+    # and the norm is done by the product only where a block takes two tiles or more
+    assert hip._norm_in_the_product(8, 12288) and not hip._norm_in_the_product(8, 27648)
+    assert not hip._norm_in_the_product(9, 12288)
+
+
 def test_which_products_of_some_rows_go_to_our_kernel():
     """The rule of `linear` at the sizes it was measured at (256 compute units): blocks of 64 columns, K shared
     out until every unit has a block at most, taken where three units in four get one."""
