@@ -315,12 +315,15 @@ def test_schedules_with_library_products(tiny_folders_bf16, tmp_path, monkeypatc
 
 
 FULL_SIZES = {
-    # the layer sizes of three members of the family (reference: the 175B key set, gen_random_pretrained.py:105-140)
+    # the layer sizes of four members of the family (reference: the 175B key set, gen_random_pretrained.py:105-140)
     "6.7b": dict(vocab_size=50272, hidden_size=4096, num_hidden_layers=2, num_attention_heads=32, ffn_dim=16384,
                  max_position_embeddings=2048, init_std=0.02),
     # heads of 80: no power of two
     "2.7b": dict(vocab_size=50272, hidden_size=2560, num_hidden_layers=2, num_attention_heads=32, ffn_dim=10240,
                  max_position_embeddings=2048, init_std=0.02),
+    # 40 heads; 80 and 320 blocks of 64 columns, which the products share out otherwise than 64 and 256
+    "13b": dict(vocab_size=50272, hidden_size=5120, num_hidden_layers=2, num_attention_heads=40, ffn_dim=20480,
+                max_position_embeddings=2048, init_std=0.02),
     # the norm after each half, an embedding narrower than the model
     "350m": dict(vocab_size=50272, hidden_size=1024, num_hidden_layers=3, num_attention_heads=16, ffn_dim=4096,
                  max_position_embeddings=2048, word_embed_proj_dim=512, do_layer_norm_before=False, init_std=0.02),
@@ -330,7 +333,7 @@ FULL_SIZES = {
 @pytest.mark.parametrize("size", list(FULL_SIZES))
 def test_full_layer_sizes_against_plain(size):
     """A few layers of the sizes of OPT-6.7B (width 4096, 32 heads of 128, inner width 16384, vocabulary
-    50272), OPT-2.7B and OPT-350m on bfloat16-stored random weights: the float32 engine and the bfloat16
+    50272), OPT-2.7B, OPT-13B and OPT-350m on bfloat16-stored random weights: the float32 engine and the bfloat16
     engine against the plain implementation, under a schedule that takes a long prompt in portions, decodes
     beside another prompt, and ends with recorded decode steps. The reference's own yardstick for a
     low-precision run against a float32 one is `allclose(atol=1.0, rtol=1e-3)` with equal argmax
