@@ -162,6 +162,16 @@ __device__ __forceinline__ void sums_from_the_top(const T* x, T* out, T* carry) 
   __syncthreads();
 }
 
+// A weight of at most 1 as a whole number of 2^-40: 24 bits before and 16 behind the point of w * 2^24. Sums of
+// such numbers do not depend on the order they are added in, and differ from the exact sum by less than
+// 2^-40 a term.
+__device__ __forceinline__ unsigned long long fixed40(float w) {
+  const float w24 = w * 16777216.f;
+  const uint32_t whole = (uint32_t)w24;
+  const uint32_t rest = (uint32_t)((w24 - (float)whole) * 65536.f);
+  return ((unsigned long long)whole << 16) + rest;
+}
+
 // One block per row; a row with temperature 0 takes its argmax.
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature, const int* __restrict__ top_k,
@@ -181,7 +191,8 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
   __shared__ unsigned int sh_remaining, sh_bin;
   __shared__ float sh_above, sh_total;
   __shared__ int sh_result, sh_last, sh_n, sh_owner, sh_owner_last;
-  __shared__ unsigned long long sh_key;
+  __shared__ unsigned long long sh_key, sh_itotal;
+  __shared__ unsigned long long ipart[SAMPLE_THREADS];
   __shared__ unsigned long long tkey[SAMPLE_GATHER], ckey[SAMPLE_GATHER];
   __shared__ float tval[SAMPLE_GATHER];
   __shared__ unsigned int cnt_above[256], carry_u[4];
@@ -419,11 +430,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
           const unsigned int digit = pass == -2 ? coarse : pass == -1 ? fine : (unsigned int)(key >> shift) & 255u;
           const unsigned int d = digit * 8 + copy;
           atomicAdd(&cnt8[d], 1u);
-          // at most 1, as 24 bits before and 16 bits behind the point of e * 2^24
-          const float e24 = weight(x) * 16777216.f;
-          const uint32_t whole = (uint32_t)e24;
-          const uint32_t rest = (uint32_t)((e24 - (float)whole) * 65536.f);
-          atomicAdd(&mass8[d], ((unsigned long long)whole << 16) + rest);
+          atomicAdd(&mass8[d], fixed40(weight(x)));
         }
       }
       __syncthreads();
@@ -531,7 +538,9 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
       for (int e = 0; e < 4; ++e) x[e] = i + e >= 0 && i + e < vocab ? row[i + e] : 0.f;
     }
   };
-  float s = 0.f;
+  // the masses are added as whole numbers of 2^-40: the sums are the same whatever the order, so the thread
+  // that owns the drawn point finds it in its segment, and the draw is that of exact arithmetic to 2^-40 a token
+  unsigned long long s = 0;
   int last = -1;
 #pragma unroll 4
   for (int q = 0; q < seg; q += 4) {
@@ -541,7 +550,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     for (int e = 0; e < 4; ++e) {
       const int i = i0 + q + e;
       if (i >= 0 && i < vocab && order_key(x[e], i) >= floor_key) {
-        s += weight(x[e]);
+        s += fixed40(weight(x[e]));
         last = i;
       }
     }
@@ -551,34 +560,36 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     sh_last = -1;
     sh_owner = -1;
   }
-  part[tid] = s;
+  ipart[tid] = s;
   __syncthreads();
   if (last >= 0) atomicMax(&sh_last, last);
-  // exclusive scan of part[] by one wave: 16 values per lane
+  // exclusive scan of ipart[] by one wave: 16 values per lane
   if (wave == 0) {
-    float local[16];
-    float run = 0.f;
+    unsigned long long local[16];
+    unsigned long long run = 0;
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
       local[j] = run;
-      run += part[lane * 16 + j];
+      run += ipart[lane * 16 + j];
     }
-    float incl = run;
+    unsigned long long incl = run;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
-      const float v = __shfl_up(incl, o, 64);
+      const unsigned long long v = __shfl_up(incl, o, 64);
       if (lane >= o) incl += v;
     }
-    const float base = incl - run;
+    const unsigned long long base = incl - run;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) part[lane * 16 + j] = base + local[j];
-    if (lane == 63) sh_total = incl;
+    for (int j = 0; j < 16; ++j) ipart[lane * 16 + j] = base + local[j];
+    if (lane == 63) sh_itotal = incl;
   }
   __syncthreads();
-  const float goal = u * sh_total;
+  const unsigned long long total = sh_itotal;
+  unsigned long long goal = (unsigned long long)((double)u * (double)total);
+  if (total > 0 && goal >= total) goal = total - 1;
   // thread t owns [base_t, base_{t+1}): the scanned values tile the line without gaps
-  const float base = part[tid];
-  const float next = tid + 1 < SAMPLE_THREADS ? part[tid + 1] : INFINITY;
+  const unsigned long long base = ipart[tid];
+  const unsigned long long next = tid + 1 < SAMPLE_THREADS ? ipart[tid + 1] : total;
   // its owner's segment is walked by the first wave, 64 tokens a turn: one trip to memory where the owner alone
   // would make one for every four tokens, each waiting for the one before
   if (last >= 0 && base <= goal && goal < next) {
@@ -588,17 +599,17 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
   __syncthreads();
   if (wave == 0 && sh_owner >= 0) {
     const int o0 = sh_owner * seg - lead;
-    float run = part[sh_owner];
+    unsigned long long run = ipart[sh_owner];
     int pick = -1;
     for (int q = 0; q < seg && pick < 0; q += 64) {
       const int i = o0 + q + lane;
       const bool ok = q + lane < seg && i >= 0 && i < vocab;
       const float x = ok ? row[i] : 0.f;
       const bool kept = ok && order_key(x, i) >= floor_key;
-      float incl = kept ? weight(x) : 0.f;
+      unsigned long long incl = kept ? fixed40(weight(x)) : 0;
 #pragma unroll
       for (int o = 1; o < 64; o <<= 1) {
-        const float v = __shfl_up(incl, o, 64);
+        const unsigned long long v = __shfl_up(incl, o, 64);
         if (lane >= o) incl += v;
       }
       const unsigned long long hit = __ballot(kept && run + incl > goal);
@@ -615,6 +626,8 @@ extern "C" int tnx_sample(const float* logits, const float* temperature, const i
                           const long long* seeds, const long long* counters, const int* min_keep, int* out,
                           int rows, int vocab, hipStream_t stream) {
   TNX_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
+  TNX_REQUIRE(vocab <= (1 << 22), "sample: a vocabulary of %d is more than the %d that the sums of masses (whole "
+              "numbers of 2^-40 in 64 bits) are sized for", vocab, 1 << 22);
   if (rows == 0) return 0;
   sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, temperature, top_k, top_p, seeds, counters, min_keep,
                                                      out, vocab);
