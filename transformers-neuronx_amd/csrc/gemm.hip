@@ -1354,8 +1354,12 @@ extern "C" int tnx_gemm_library(const void* x, const void* w, const float* bias,
   const auto key = std::make_tuple(device, M, N, K, what);
   auto it = library_plans.find(key);
   if (it == library_plans.end()) {
-    // `tune` 1: up to TUNED_ROWS rows, the first few of the ranking; 2: every product, more of the ranking
-    bool timed = tune >= 2 || (tune && M <= TUNED_ROWS);
+    // `tune` 1: up to TUNED_ROWS rows, and row counts that are multiples of 256 (the portions a token budget
+    // cuts prompts into come again and again, and the ranking's first choice can be far off there too:
+    // 2,048 x 9,216 over 36,864 with bias and ReLU, first choice 1.88 ms, the quickest of six about 1.1),
+    // the first few of the ranking (more of it for the many rows, where the quickest was the ranking's
+    // ninth or later); 2: every product, more of the ranking
+    bool timed = tune >= 2 || (tune && (M <= TUNED_ROWS || M % 256 == 0));
     if (timed) {
       // nothing is timed inside a recording: the first choice of the library's ranking stands in there
       hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
@@ -1364,7 +1368,7 @@ extern "C" int tnx_gemm_library(const void* x, const void* w, const float* bias,
     if (timed && (flush == nullptr || flush_bytes == 0)) return 3;
     it = library_plans.emplace(key, make_plan(library_handles[device], M, N, K, bias, act == TNX_ACT_RELU,
                                               out_dtype == TNX_F32, call, timed ? flush : nullptr, flush_bytes,
-                                              tune >= 2 ? CANDIDATES : FEW_CANDIDATES)).first;
+                                              tune >= 2 || M > TUNED_ROWS ? CANDIDATES : FEW_CANDIDATES)).first;
   }
   const LibraryPlan& p = it->second;
   if (!p.usable || p.workspace > workspace_bytes) return 2;
