@@ -229,6 +229,41 @@ def sample_row(scores, u, top_k=None, top_p=None, temperature=1.0, min_tokens_to
     return int(indices[min(pick, len(indices) - 1)])
 
 
+def draw_slack(scores, u, token, top_k=None, top_p=None, temperature=1.0, min_tokens_to_keep=1):
+    """How far outside `token`'s stretch of the line [0, 1) the drawn point `u` lies, and the bound that float32
+    rounding puts on that: `(slack, bound)`, slack 0 where `sample_row` computed without any rounding draws
+    `token`. The bound is derived, not chosen: a float32 weight exp(x/T - max/T) is within 2 units of 2^-23
+    of the exact one (the library's exponential one, the subtraction another), so a sum of weights divided by
+    the whole sum is within 4 * 2^-23 of the exact ratio, whatever the number of tokens; a sampler that adds
+    weights as whole numbers of 2^-40 adds 2^-40 a kept token. The same bound decides which numbers of kept
+    tokens top-p may arrive at: a token with a mass above it that close to `top_p` may stay or go, and every
+    such number is tried (sampling.py:213-249 compares float32 sums, which carry the same rounding)."""
+    values, indices = torch.sort(scores.float() / temperature, descending=True, stable=True)
+    if top_k is not None:
+        k = min(max(top_k, min_tokens_to_keep), values.numel())
+        values, indices = values[:k], indices[:k]
+    exact = torch.softmax(values.double(), -1)
+    n = values.numel()
+    bound = 4 * 2.0 ** -23 + n * 2.0 ** -40
+    counts = [n]
+    if top_p is not None and top_p < 1.0:
+        above = torch.cumsum(exact, -1) - exact                    # the mass of the tokens before each one
+        fewest = max(int((above < top_p - bound).sum()), min_tokens_to_keep, 1)
+        most = max(int((above < top_p + bound).sum()), min_tokens_to_keep, 1)
+        counts = list(range(fewest, min(most, n) + 1))
+    best = float("inf")
+    for count in counts:
+        ids, order = torch.sort(indices[:count])
+        at = int(torch.searchsorted(ids, token))
+        if at >= count or int(ids[at]) != token:
+            continue
+        mass = exact[:count][order]
+        cum = torch.cumsum(mass, -1)
+        low, high = float(cum[at] - mass[at]) / float(cum[-1]), float(cum[at]) / float(cum[-1])
+        best = min(best, max(low - u, u - high, 0.0))
+    return best, bound
+
+
 def banned_by_ngrams(tokens, n):
     """sampling.py:267-300 for one row: every run of `n` tokens in `tokens` is filed under its first n - 1
     (:275-277); with fewer than n - 1 tokens nothing is banned (:292-294); otherwise the tokens filed under

@@ -164,6 +164,32 @@ def test_draw():
     assert plain_opt.sample_row(s, 0.9, top_k=2) == 2                            # within the top k only
 
 
+def test_draw_slack():
+    """The yardstick for samplers that round differently: zero for the token `sample_row` draws, the distance
+    to the token's stretch for any other, and both numbers of kept tokens count where top-p's sum lies on a
+    threshold."""
+    s = torch.log(torch.tensor([0.125, 0.5, 0.25, 0.125]))
+    assert plain_opt.draw_slack(s, 0.3, 1)[0] == 0.0
+    assert abs(plain_opt.draw_slack(s, 0.3, 0)[0]- 0.175) < 1e-6             # token 0 ends at .125
+    assert abs(plain_opt.draw_slack(s, 0.3, 2)[0] - 0.325) < 1e-6             # token 2 begins at .625
+    assert plain_opt.draw_slack(s, 0.3, 3, top_k=2)[0] == float("inf")         # not kept at all
+    assert plain_opt.draw_slack(s, 0.3, 1)[1] == 4 * 2.0 ** -23 + 4 * 2.0 ** -40
+    # top-p .75 exactly: tokens 1 and 2 hold .75, so token 0 (first of two at .125, ties to the lower id) may
+    # stay or go; with it u = .1 draws token 0, without it token 1; token 3 stays out either way
+    assert plain_opt.draw_slack(s, 0.1, 0, top_p=0.75)[0] == 0.0
+    assert plain_opt.draw_slack(s, 0.1, 1, top_p=0.75)[0] == 0.0
+    assert plain_opt.draw_slack(s, 0.99, 3, top_p=0.75)[0] == float("inf")
+    assert plain_opt.draw_slack(s, 0.1, 1, top_p=0.76)[0] > 0.01
+    g = torch.Generator().manual_seed(0)
+    for t in range(60):
+        row = torch.randn(int(torch.randint(2, 2000, (1,), generator=g)), generator=g) * 3
+        u = float(torch.rand(1, generator=g))
+        k, p, temp, least = [None, 5, 50][t % 3], [None, 0.9, 0.5, 0.05][t % 4], [1.0, 0.3, 1.5][t % 3], [1, 3][t % 2]
+        tok = plain_opt.sample_row(row, u, k, p, temp, least)
+        slack, bound = plain_opt.draw_slack(row, u, tok, k, p, temp, least)
+        assert slack <= bound < 1e-6
+
+
 def test_philox_known_answers():
     """Known-answer vectors of Philox-4x32-10 (Random123's kat_vectors): counter and key all zero give
     6627e8d5 as the first word; all ones give 408f276d."""

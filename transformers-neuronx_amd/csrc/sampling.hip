@@ -172,6 +172,19 @@ __device__ __forceinline__ unsigned long long fixed40(float w) {
   return ((unsigned long long)whole << 16) + rest;
 }
 
+// exp(a - m) for a <= m, to the last place or two of a float: the rounding of a - m is found (two-sum) and put
+// back after the exponential, which is the library's full-precision one. What is below 2^-40 counts as nothing
+// (fixed40 would cut it off anyway); that takes in a = -inf, and m = +inf beside a finite a.
+__device__ __forceinline__ float exp_below(float a, float m) {
+  if (a == m) return 1.f;
+  const float d = a - m;
+  if (!(d > -30.f)) return 0.f;
+  const float b = -m, bb = d - a;
+  const float err = (a - (d - bb)) + (b - bb);
+  const float e = expf(d);
+  return fmaf(e, err, e);
+}
+
 // One block per row; a row with temperature 0 takes its argmax.
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature, const int* __restrict__ top_k,
@@ -179,24 +192,23 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
               const long long* __restrict__ counters, const int* __restrict__ min_keep, int* __restrict__ out,
               int vocab) {
   __shared__ unsigned int cnt[256];
-  __shared__ float mass[256];
+  __shared__ unsigned long long mass[256];           // in units of 2^-40, like every sum of weights here
   // Eight copies of both, a lane adding to copy lane % 8: in the first pass nearly all keys of a row fall into
   // two or three bins, and 64 lanes adding to one word take their turns one after the other.
   __shared__ unsigned int cnt8[256 * 8];
   __shared__ unsigned long long mass8[256 * 8];     // in units of 2^-40: whole numbers add up in any order alike
   const int copy = threadIdx.x & 7;
-  __shared__ float part[SAMPLE_THREADS];
   __shared__ unsigned long long best[16];
   __shared__ int sh_digit;
   __shared__ unsigned int sh_remaining, sh_bin;
-  __shared__ float sh_above, sh_total;
+  __shared__ unsigned long long sh_above;
   __shared__ int sh_result, sh_last, sh_n, sh_owner, sh_owner_last;
   __shared__ unsigned long long sh_key, sh_itotal;
   __shared__ unsigned long long ipart[SAMPLE_THREADS];
-  __shared__ unsigned long long tkey[SAMPLE_GATHER], ckey[SAMPLE_GATHER];
+  __shared__ unsigned long long tkey[SAMPLE_GATHER], ckey[SAMPLE_GATHER], tmass[SAMPLE_GATHER];
   __shared__ float tval[SAMPLE_GATHER];
   __shared__ unsigned int cnt_above[256], carry_u[4];
-  __shared__ float mass_above[256], carry_f[4];
+  __shared__ unsigned long long mass_above[256], carry_m[4];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rowi = blockIdx.x;
@@ -208,7 +220,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
   if (k > 0) k = max(k, keep);
   // after a top-k of no more than SAMPLE_GATHER the kept tokens are gathered and the rest is done over these
   const bool few = !greedy && k > 0 && k < vocab && k <= SAMPLE_GATHER;
-  const float inv_temp = greedy ? 0.f : 1.f / temp;
+  const float inv_temp = greedy ? 0.f : 1.f / temp;     // for the bins of the search only; weights divide by temp
 
   // the largest key: argmax, and the maximum for the softmax (the gathered tokens bring their own)
   float xmax = 0.f;
@@ -233,11 +245,17 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
       if (tid == 0) out[rowi] = arg;
       return;
     }
-    xmax = row[arg] * inv_temp;
+    xmax = row[arg] / temp;
   }
 
-  // a token's share of the softmax before it is divided by the sum; a NaN has none, as it orders last
-  auto weight = [&](float x) -> float { return x != x ? 0.f : __expf(x * inv_temp - xmax); };
+  // A token's share of the softmax before it is divided by the sum, as sampling.py:337-345 computes it: the
+  // logit divided by the temperature (a true division), less the largest such, exponentiated in full precision;
+  // as a whole number of 2^-40. A NaN has none, as it orders last.
+  auto weight = [&](float x) -> unsigned long long { return x != x ? 0ull : fixed40(exp_below(x / temp, xmax)); };
+  // p of a sum of weights, rounded down
+  auto share = [](float p, unsigned long long total) -> unsigned long long {
+    return (unsigned long long)((double)p * (double)total);
+  };
 
   // the k-th largest key of the row, by radix selection; every thread of the block calls it together
   auto kth_largest = [&](unsigned int k) -> uint64_t {
@@ -323,7 +341,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
         const int at = atomicAdd(&sh_n, 1);
         if (at < SAMPLE_GATHER) {
           tkey[at] = key;
-          tval[at] = row[i] != row[i] ? -INFINITY : row[i] * inv_temp;
+          tval[at] = row[i] != row[i] ? -INFINITY : row[i] / temp;
         }
       }
     }
@@ -333,18 +351,18 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     float largest = -INFINITY;
     for (int j = 0; mine_too && j < n; ++j) largest = fmaxf(largest, tval[j]);
     __syncthreads();
-    if (tid < n) tval[tid] = largest == -INFINITY ? 1.f : __expf(tval[tid] - largest);     // (all -inf: alike)
+    if (tid < n) tmass[tid] = fixed40(exp_below(tval[tid], largest));     // (all -inf: alike, 1 each)
     __syncthreads();
     // of each of them: its place in the order of token ids, and the mass and the number of those with a larger key
     const bool have = tid < n;
     const uint64_t my_key = have ? tkey[tid] : 0;
-    const float my_val = have ? tval[tid] : 0.f;
+    const unsigned long long my_val = have ? tmass[tid] : 0;
     const uint32_t my_low = (uint32_t)my_key;          // the complement of the token id: larger is earlier
-    float above = 0.f, z = 0.f;
+    unsigned long long above = 0, z = 0;
     int rank = 0, place = 0;
     for (int j = 0; mine_too && j < n; ++j) {
       const uint64_t kj = tkey[j];
-      const float e = tval[j];
+      const unsigned long long e = tmass[j];
       z += e;
       if (kj > my_key) {
         above += e;
@@ -354,38 +372,40 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     }
     // top-p keeps a token while those above it hold less than p of the mass, the largest always, and never
     // fewer than `keep` (sampling.py:213-249, :232)
-    const bool kept = have && (p >= 1.f || above < p * z || rank == 0 || rank < keep);
-    part[tid] = 0.f;
+    const bool kept = have && (p >= 1.f || above < share(p, z) || rank == 0 || rank < keep);
+    if (tid < SAMPLE_GATHER) ipart[tid] = 0;
     __syncthreads();
     if (have) {
       ckey[place] = my_key;
-      part[place] = kept ? my_val : 0.f;
+      ipart[place] = kept ? my_val : 0;
+      if (kept) atomicMax(&sh_last, place);
     }
     __syncthreads();
-    const float mine = part[tid];
-    if (mine > 0.f) atomicMax(&sh_last, tid);
+    const unsigned long long mine = tid < SAMPLE_GATHER ? ipart[tid] : 0;
     __syncthreads();
     if (wave == 0) {          // exclusive scan of the kept masses, in the order of the token ids
-      float local[16], run = 0.f;
+      unsigned long long local[SAMPLE_GATHER / 64], run = 0;
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
+      for (int j = 0; j < SAMPLE_GATHER / 64; ++j) {
         local[j] = run;
-        run += part[lane * 16 + j];
+        run += ipart[lane * (SAMPLE_GATHER / 64) + j];
       }
-      float incl = run;
+      unsigned long long incl = run;
 #pragma unroll
       for (int o = 1; o < 64; o <<= 1) {
-        const float w = __shfl_up(incl, o, 64);
+        const unsigned long long w = __shfl_up(incl, o, 64);
         if (lane >= o) incl += w;
       }
 #pragma unroll
-      for (int j = 0; j < 16; ++j) part[lane * 16 + j] = incl - run + local[j];
-      if (lane == 63) sh_total = incl;
+      for (int j = 0; j < SAMPLE_GATHER / 64; ++j) ipart[lane * (SAMPLE_GATHER / 64) + j] = incl - run + local[j];
+      if (lane == 63) sh_itotal = incl;
     }
     __syncthreads();
-    const float goal = u * sh_total;
-    const float base = part[tid];
-    if (mine > 0.f && base <= goal && goal < base + mine) atomicMax(&sh_result, tid);
+    const unsigned long long total = sh_itotal;
+    unsigned long long goal = share(u, total);
+    if (total > 0 && goal >= total) goal = total - 1;
+    const unsigned long long base = tid < SAMPLE_GATHER ? ipart[tid] : 0;
+    if (mine > 0 && base <= goal && goal < base + mine) sh_result = tid;       // one thread at most
     __syncthreads();
     if (tid == 0) {
       const int pick = sh_result >= 0 ? sh_result : max(sh_last, 0);
@@ -409,10 +429,10 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
       coarse = 255 - (int)c;
       fine = 255 - (int)fminf((t - c) * 256.f, 255.f);
     };
-    float target = 0.f;
+    unsigned long long target = 0;
     int level = -1, sublevel = -1;
     uint64_t prefix = 0, mask = 0;
-    float above = 0.f;
+    unsigned long long above = 0;
     for (int pass = -2; pass < 8; ++pass) {
       const int shift = 56 - 8 * max(pass, 0);
       for (int j = tid; j < 256 * 8; j += SAMPLE_THREADS) {
@@ -430,7 +450,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
           const unsigned int digit = pass == -2 ? coarse : pass == -1 ? fine : (unsigned int)(key >> shift) & 255u;
           const unsigned int d = digit * 8 + copy;
           atomicAdd(&cnt8[d], 1u);
-          atomicAdd(&mass8[d], fixed40(weight(x)));
+          atomicAdd(&mass8[d], weight(x));
         }
       }
       __syncthreads();
@@ -443,23 +463,23 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
           m += mass8[tid * 8 + j];
         }
         cnt[tid] = c;
-        mass[tid] = (float)m * 9.094947017729282e-13f;        // 2^-40
+        mass[tid] = m;
       }
       __syncthreads();
       // the lowest digit in use with less than the target above it (the highest in use, if none has)
-      sums_from_the_top(mass, mass_above, carry_f);
+      sums_from_the_top(mass, mass_above, carry_m);
       sums_from_the_top(cnt, cnt_above, carry_u);
-      if (pass == -2) target = p * mass_above[0];
+      if (pass == -2) target = share(p, mass_above[0]);
       if (tid == 0) sh_digit = 256;
       __syncthreads();
       if (tid < 256 && cnt[tid] > 0) {
-        const float over = above + (tid < 255 ? mass_above[tid + 1] : 0.f);     // the mass above this digit
+        const unsigned long long over = above + (tid < 255 ? mass_above[tid + 1] : 0);     // the mass above this digit
         const bool top = tid == 255 || cnt_above[tid + 1] == 0;                  // no digit in use above it
         if (over < target || top) atomicMin(&sh_digit, tid);
       }
       __syncthreads();
       if (tid == sh_digit) {
-        sh_above = above + (tid < 255 ? mass_above[tid + 1] : 0.f);
+        sh_above = above + (tid < 255 ? mass_above[tid + 1] : 0);
         sh_bin = cnt[tid];
       }
       __syncthreads();
@@ -491,17 +511,17 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
           if (key >= floor_key && coarse == level && (sublevel < 0 || fine == sublevel) && (key & mask) == prefix) {
             const int at = atomicAdd(&sh_n, 1);
             tkey[at] = key;
-            tval[at] = weight(x);
+            tmass[at] = weight(x);
           }
         }
         __syncthreads();
         if (tid < (int)bin) {
           const uint64_t mine = tkey[tid];
-          float over = above;
+          unsigned long long over = above;
           bool top = true;
           for (unsigned int j = 0; j < bin; ++j)
             if (tkey[j] > mine) {
-              over += tval[j];
+              over += tmass[j];
               top = false;
             }
           if (over < target || top) atomicMin(&sh_key, (unsigned long long)mine);
@@ -550,7 +570,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     for (int e = 0; e < 4; ++e) {
       const int i = i0 + q + e;
       if (i >= 0 && i < vocab && order_key(x[e], i) >= floor_key) {
-        s += fixed40(weight(x[e]));
+        s += weight(x[e]);
         last = i;
       }
     }
@@ -585,7 +605,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
   }
   __syncthreads();
   const unsigned long long total = sh_itotal;
-  unsigned long long goal = (unsigned long long)((double)u * (double)total);
+  unsigned long long goal = share(u, total);
   if (total > 0 && goal >= total) goal = total - 1;
   // thread t owns [base_t, base_{t+1}): the scanned values tile the line without gaps
   const unsigned long long base = ipart[tid];
@@ -606,7 +626,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
       const bool ok = q + lane < seg && i >= 0 && i < vocab;
       const float x = ok ? row[i] : 0.f;
       const bool kept = ok && order_key(x, i) >= floor_key;
-      unsigned long long incl = kept ? fixed40(weight(x)) : 0;
+      unsigned long long incl = kept ? weight(x) : 0;
 #pragma unroll
       for (int o = 1; o < 64; o <<= 1) {
         const unsigned long long v = __shfl_up(incl, o, 64);
