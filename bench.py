@@ -1,20 +1,30 @@
 #!/usr/bin/env python3
-"""Decode and prefill throughput of the engine at OPT-6.7B size with random weights.
+"""Decode and prefill throughput of the engine with random weights; by default at OPT-6.7B's sizes.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--model 6.7b|350m|1.3b|2.7b|13b|30b|66b] [--mix]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--model NAME | FOLDER | CONFIG.json] [--mix] ...
 
 One JSON line: `value` is decoded tokens per second at batch 8 and a 2,048-token context
 (a "step" is one decode step of the whole engine: schedule, model, sampling);
 `prefill` is one 2,048-token prompt in one step; `roofline` sets the bytes a decode step has
 to read (every weight once, and the cache of the live requests) against its time; `points`
-holds decoding at batch 1 and 64 (tokens a second, milliseconds a step, share of the memory roofline) and the
+holds decoding at batch 1 and 64 (tokens a second, milliseconds a step, share of the memory roofline), the
 whole way of batch 8 from 512-token prompts to the 2,048-token context (mean tokens a second, its share of the
-roofline at the mean context, and the percentiles of the time between two steps). The measuring follows the reference's own benchmark
+roofline at the mean context, and the percentiles of the time between two steps), a continuous-batching mix at
+OPT-350m's sizes and, where the device has room, decoding and a prompt at OPT-66B's; `ceilings` is what this
+device reaches at best, measured here (a kernel that only reads memory, a loop of matrix instructions on
+registers), and `roofline` / `prefill` give their shares of these beside the shares of the published peaks;
+`check` compares the bfloat16 engine with a float32 engine on the same weights at full depth, by the
+reference's own yardstick (generation_demo.py:437-443). The measuring follows the reference's own benchmark
 (generation_demo.py:107-187: warm-up runs, then timed ones; random token ids as prompts,
 :492-494). Weights and prompts are synthetic and seeded; there are no published numbers of
 the reference to compare with, so `vs_baseline` is null.
+
+The model is any registered architecture's: `--model` takes a name of the table below (config.json contents of
+the OPT family), a model folder or a config.json file. Bytes and flops come from what the model's parts
+declare, not from formulas of one architecture.
 """
 import argparse
+import gc
 import json
 import os
 import sys
@@ -23,125 +33,126 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-# OPT-6.7B: the measurement of record
-MODEL = dict(architectures=["OPTForCausalLM"], model_type="opt", vocab_size=50272, hidden_size=4096,
-             num_hidden_layers=32, num_attention_heads=32, ffn_dim=16384, max_position_embeddings=2048,
-             word_embed_proj_dim=4096, do_layer_norm_before=True, activation_function="relu", enable_bias=True,
-             layer_norm_elementwise_affine=True, init_std=0.02, torch_dtype="bfloat16")
-# More members of the family, for `--model` (the default run and its JSON line stay OPT-6.7B)
-OTHER_MODELS = {
-    "350m": dict(hidden_size=1024, num_hidden_layers=24, num_attention_heads=16, ffn_dim=4096, word_embed_proj_dim=512,
+# config.json contents by name: the measurement of record is OPT-6.7B
+_OPT = dict(architectures=["OPTForCausalLM"], model_type="opt", vocab_size=50272, max_position_embeddings=2048,
+            do_layer_norm_before=True, activation_function="relu", enable_bias=True,
+            layer_norm_elementwise_affine=True, init_std=0.02, torch_dtype="bfloat16")
+PRESETS = {
+    "6.7b": dict(_OPT, hidden_size=4096, num_hidden_layers=32, num_attention_heads=32, ffn_dim=16384, word_embed_proj_dim=4096),
+    "350m": dict(_OPT, hidden_size=1024, num_hidden_layers=24, num_attention_heads=16, ffn_dim=4096, word_embed_proj_dim=512,
                  do_layer_norm_before=False),
-    "1.3b": dict(hidden_size=2048, num_hidden_layers=24, num_attention_heads=32, ffn_dim=8192, word_embed_proj_dim=2048),
-    "2.7b": dict(hidden_size=2560, num_hidden_layers=32, num_attention_heads=32, ffn_dim=10240, word_embed_proj_dim=2560),
-    "13b": dict(hidden_size=5120, num_hidden_layers=40, num_attention_heads=40, ffn_dim=20480, word_embed_proj_dim=5120),
-    "30b": dict(hidden_size=7168, num_hidden_layers=48, num_attention_heads=56, ffn_dim=28672, word_embed_proj_dim=7168),
-    "66b": dict(hidden_size=9216, num_hidden_layers=64, num_attention_heads=72, ffn_dim=36864, word_embed_proj_dim=9216),
+    "1.3b": dict(_OPT, hidden_size=2048, num_hidden_layers=24, num_attention_heads=32, ffn_dim=8192, word_embed_proj_dim=2048),
+    "2.7b": dict(_OPT, hidden_size=2560, num_hidden_layers=32, num_attention_heads=32, ffn_dim=10240, word_embed_proj_dim=2560),
+    "13b": dict(_OPT, hidden_size=5120, num_hidden_layers=40, num_attention_heads=40, ffn_dim=20480, word_embed_proj_dim=5120),
+    "30b": dict(_OPT, hidden_size=7168, num_hidden_layers=48, num_attention_heads=56, ffn_dim=28672, word_embed_proj_dim=7168),
+    "66b": dict(_OPT, hidden_size=9216, num_hidden_layers=64, num_attention_heads=72, ffn_dim=36864, word_embed_proj_dim=9216),
 }
-CONTEXT = 2048
 PREFILL_TOKENS = 2048
 PEAK_HBM_GBS = 8000.0                      # MI355X, published
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 
-def prefill_flops(cfg, tokens):
-    """Multiply-adds times two of one whole prompt: the matrix products of every layer, causal
-    attention (half of the square), and the head for the last token."""
-    h, f, l = cfg["hidden_size"], cfg["ffn_dim"], cfg["num_hidden_layers"]
-    linear = 2 * tokens * l * (4 * h * h + 2 * h * f)
-    attention = l * 2 * 2 * h * tokens * (tokens + 1) / 2
-    head = 2 * cfg["vocab_size"] * cfg["word_embed_proj_dim"]
-    return linear + attention + head
+def log(text):
+    print(f"[bench] {text}", file=sys.stderr, flush=True)
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=64)
-    ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
-    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
-    ap.add_argument("--prefill-only", action="store_true", help="measure the prompt step alone (for profiles)")
-    ap.add_argument("--model", default="6.7b", choices=["6.7b"] + sorted(OTHER_MODELS),
-                    help="layer sizes: OPT-6.7B (the measurement of record) or another member of the family")
-    ap.add_argument("--do-sample", action="store_true",
-                    help="decode with temperature 0.8, top-k 50 and top-p 0.95 instead of greedily")
-    ap.add_argument("--mix", action="store_true",
-                    help="instead: 64 requests with prompts of 16 to 1,024 tokens and 256 new tokens each, all "
-                         "queued at once (a continuous-batching workload); prints its own line")
-    ap.add_argument("--own-products", action="store_true",
-                    help="every matrix product on our own kernels (none goes to the vendor library)")
-    ap.add_argument("--tune-all", action="store_true",
-                    help="time the vendor library's candidates for the many-rows products too")
-    ap.add_argument("--big-batch", type=int, default=64, help="the larger batch of `points` (cut to what fits the device at the full context)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
-        return 2
+def raw_config(model: str) -> dict:
+    """config.json contents for `--model`: a name of the table, a model folder or a config.json file."""
+    if model in PRESETS:
+        return dict(PRESETS[model], name="OPT-" + model.upper())
+    path = os.path.join(model, "config.json") if os.path.isdir(model) else model
+    with open(path) as fp:
+        raw = json.load(fp)
+    raw.setdefault("name", os.path.basename(os.path.dirname(os.path.abspath(path))))
+    return raw
 
-    import torch
-    from transformers_neuronx_amd.config import EngineConfig
-    from transformers_neuronx_amd.opt.config import OPTConfig
-    from transformers_neuronx_amd.engine.engine import LLMEngine
-    from transformers_neuronx_amd.engine.factory import runner_from_random
-    from transformers_neuronx_amd.sampling import SamplingParams
 
-    if args.own_products:
-        from transformers_neuronx_amd.kernels.hip import HipOps
-        HipOps.library_rows = 0
-    if args.tune_all:
-        from transformers_neuronx_amd.kernels.hip import HipOps
-        HipOps.library_tune = 2
-    raw = dict(MODEL)
-    raw.update(OTHER_MODELS.get(args.model, {}))
-    layers_full = raw["num_hidden_layers"]
-    if args.layers:
-        raw["num_hidden_layers"] = args.layers
-    cfg = OPTConfig.from_dict(raw)
-    dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
-    item = 2 if dtype == torch.bfloat16 else 4
-    kv_bytes_per_token = 2 * cfg.num_hidden_layers * cfg.hidden_size * item
-    # the larger batch of `points` is cut to what the device holds beside the weights at the full context
-    weights = item * (cfg.num_hidden_layers * (4 * cfg.hidden_size ** 2 + 2 * cfg.hidden_size * cfg.ffn_dim)
-                      + (cfg.vocab_size + cfg.max_position_embeddings) * cfg.hidden_size)
-    # (the random weights are drawn apart and fused afterwards: a quarter of them is held twice meanwhile, and
-    # what that leaves free again is in pieces too small for the cache's blocks)
-    room = int(0.95 * torch.cuda.mem_get_info()[1]) - int(1.27 * weights) - (4 << 30)
-    fits = max(1, room // (kv_bytes_per_token * CONTEXT))
-    if args.big_batch > fits and not (args.no_points or args.prefill_only):
-        print(f"[bench] {args.big_batch} requests of {CONTEXT} tokens do not fit beside {weights / 1e9:.0f} GB of "
-              f"weights; the larger batch is {fits}", file=sys.stderr, flush=True)
-        args.big_batch = fits
-    if args.batch > fits:
-        print(f"bench.py: {args.batch} requests of {CONTEXT} tokens do not fit beside {weights / 1e9:.0f} GB of weights "
-              f"on this device ({fits} do)")
-        return 2
-    max_batch = args.batch if args.no_points or args.prefill_only else max(args.batch, args.big_batch)
-    ecfg = EngineConfig(dtype=dtype, page_size=64, max_tokens=max_batch * CONTEXT, max_num_seqs=max_batch,
-                        max_num_batched_tokens=max(2048, PREFILL_TOKENS), max_model_len=CONTEXT,
-                        prompts_first=True)
-    t0 = time.time()
-    runner = runner_from_random(cfg, seed=0, cfg=ecfg)
-    torch.cuda.synchronize()
-    print(f"[bench] model ready in {time.time() - t0:.1f} s "
-          f"({runner.model.weight_bytes / 1e9:.2f} GB of weights"
-          + (f", {runner.ops.copy_bytes / 1e9:.1f} GB of them a second time in tile order" if getattr(runner.ops, "copy_bytes", None) is not None else "")
-          + ")", file=sys.stderr, flush=True)
-    engine = LLMEngine(runner, ecfg)
-    gen = torch.Generator().manual_seed(1)
+def measured_ceilings(ops, torch):
+    """What a kernel of ours reaches on this device at best: GB/s of a kernel that only reads 8 GB of memory,
+    TFLOP/s of a loop of bfloat16 matrix instructions whose operands stay in registers."""
+    dev = ops.device
+    buf = torch.empty(8 << 30, dtype=torch.uint8, device=dev)
+    buf.view(torch.int32).fill_(1)
+    units = ops.compute_units
+    out = torch.zeros(units * 16 * 256, dtype=torch.float32, device=dev)
 
-    def decode(batch, steps, warmup, prompt_len=None, latencies=None):
+    def timed(fn, repeats):
+        fn()
+        torch.cuda.synchronize(dev)
+        best = float("inf")
+        for _ in range(repeats):
+            start = torch.cuda.Event(enable_timing=True)
+            end = torch.cuda.Event(enable_timing=True)
+            start.record()
+            fn()
+            end.record()
+            end.synchronize()
+            best = min(best, start.elapsed_time(end) * 1e-3)
+        return best
+
+    read = timed(lambda: ops.call("probe", "tnx_probe_stream_read", buf.data_ptr(), buf.numel(), out.data_ptr(),
+                                  units * 8, ops.stream()), 5)
+    iterations, blocks = 20000, units * 8
+    loop = timed(lambda: ops.call("probe", "tnx_probe_mfma_loop", blocks, iterations, out.data_ptr(), ops.stream()), 3)
+    del buf, out
+    torch.cuda.empty_cache()
+    return {"hbm_read_gbs_measured": round(8 * (1 << 30) / read / 1e9, 1),
+            "mfma_tflops_measured": round(blocks * 4 * iterations * 4 * 2 * 32 * 32 * 16 / loop / 1e12, 1)}
+
+
+class Bench:
+    """One model on the device and the measurements over it."""
+
+    def __init__(self, raw, dtype_name, max_batch, context, layers=None, layers_key="num_hidden_layers", storage=None,
+                 max_tokens=None):
+        import torch
+        from transformers_neuronx_amd.config import EngineConfig
+        from transformers_neuronx_amd.config.registry import resolve
+        from transformers_neuronx_amd.engine.engine import LLMEngine
+        from transformers_neuronx_amd.engine.factory import runner_from_random
+        self.torch = torch
+        raw = {k: v for k, v in raw.items() if k != "name"}
+        self.layers_full = raw.get(layers_key)
+        if layers:
+            raw[layers_key] = layers
+        self.cfg = resolve(raw).config_class.from_dict(raw)
+        self.dtype_name = dtype_name
+        self.dtype = torch.bfloat16 if dtype_name == "bf16" else torch.float32
+        self.context = context
+        self.ecfg = EngineConfig(dtype=self.dtype, page_size=64, max_tokens=max_tokens or max_batch * context,
+                                 max_num_seqs=max_batch, max_num_batched_tokens=max(2048, PREFILL_TOKENS),
+                                 max_model_len=context, prompts_first=True)
+        t0 = time.time()
+        self.runner = runner_from_random(self.cfg, seed=0, cfg=self.ecfg, storage=storage)
+        torch.cuda.synchronize()
+        self.model = self.runner.model
+        copies = getattr(self.runner.ops, "copy_bytes", None)
+        log(f"model ready in {time.time() - t0:.1f} s ({self.model.weight_bytes / 1e9:.2f} GB of weights"
+            + (f", {copies / 1e9:.1f} GB of them a second time in tile order" if copies is not None else "") + ")")
+        self.engine = LLMEngine(self.runner, self.ecfg)
+        self.gen = torch.Generator().manual_seed(1)
+        self.vocab = self.model.spec.vocab_size
+
+    def close(self):
+        self.engine = self.runner = self.model = None
+        gc.collect()
+        self.torch.cuda.empty_cache()
+
+    def prompt(self, n):
+        return self.torch.randint(3, self.vocab, (n,), generator=self.gen).tolist()
+
+    def decode(self, batch, steps, warmup, prompt_len=None, latencies=None, do_sample=False):
         """Tokens per second, seconds per step and bytes per step of `steps` decode steps that end at
         the full context (or begin after prompts of `prompt_len` tokens)."""
+        from transformers_neuronx_amd.sampling import SamplingParams
+        torch, engine = self.torch, self.engine
         engine.reset()
         if prompt_len is None:
-            prompt_len = CONTEXT - (steps + warmup) - 1
+            prompt_len = self.context - (steps + warmup) - 1
         for i in range(batch):
-            params = SamplingParams(max_new_tokens=steps + warmup + 1, do_sample=args.do_sample, temperature=0.8,
+            params = SamplingParams(max_new_tokens=steps + warmup + 1, do_sample=do_sample, temperature=0.8,
                                     top_k=50, top_p=0.95, seed=i, ignore_eos=True)
-            engine.add_request(torch.randint(3, cfg.vocab_size, (prompt_len,), generator=gen).tolist(), params)
+            engine.add_request(self.prompt(prompt_len), params)
         while any(not r.decoding for r in engine.requests.values()):
             engine.step()                 # prompts first: nothing decodes until every prompt is in
         assert all(len(r.output) == 1 for r in engine.requests.values())
@@ -161,32 +172,38 @@ def main():
         torch.cuda.synchronize()
         sec = (time.perf_counter() - start) / steps
         assert made == batch * steps, f"{made} tokens in {steps} steps of batch {batch}"
-        read = runner.model.weight_bytes + lens / steps * kv_bytes_per_token
+        # every weight once, and of each live request the cache that its token reads (at the mean length)
+        read = self.model.weight_bytes + batch * self.model.cache_bytes_read(lens / steps / batch, self.dtype)
         return made / (sec * steps), sec, read
 
-    def prefill(tokens):
+    def prefill(self, tokens):
+        """Seconds of one whole prompt in one step (the median of five, after one warm-up) and its flops."""
+        from transformers_neuronx_amd.sampling import SamplingParams
+        torch, engine = self.torch, self.engine
         engine.reset()
         params = SamplingParams(max_new_tokens=1, do_sample=False, ignore_eos=True)
         times = []
         for i in range(6):
-            engine.add_request(torch.randint(3, cfg.vocab_size, (tokens,), generator=gen).tolist(), params)
+            engine.add_request(self.prompt(tokens), params)
             torch.cuda.synchronize()
             start = time.perf_counter()
             engine.step()
             torch.cuda.synchronize()
             times.append(time.perf_counter() - start)
-        return sorted(times[1:])[2]       # the median of five, after one warm-up
+        return sorted(times[1:])[2], self.model.step_flops(tokens, (tokens + 1) / 2, 1)
 
-    if args.mix:
-        # every request is there at the start; the scheduler mixes portions of prompts with decoding. The
-        # workload runs twice with other tokens and the second run is timed: the first loads the vendor
-        # library and lets it choose its algorithms, which a server does once in its life
-        params = SamplingParams(max_new_tokens=256, do_sample=False, ignore_eos=True)
+    def mix(self, requests=64, new_tokens=256):
+        """Every request is there at the start; the scheduler mixes portions of prompts with decoding. The
+        workload runs twice with other tokens and the second run is timed: the first loads the vendor
+        library and lets it choose its algorithms, which a server does once in its life."""
+        from transformers_neuronx_amd.sampling import SamplingParams
+        torch, engine = self.torch, self.engine
+        params = SamplingParams(max_new_tokens=new_tokens, do_sample=False, ignore_eos=True)
         for timed in (False, True):
             engine.reset()
-            lengths = torch.randint(16, 1025, (64,), generator=torch.Generator().manual_seed(2)).tolist()
+            lengths = torch.randint(16, 1025, (requests,), generator=torch.Generator().manual_seed(2)).tolist()
             for n in lengths:
-                engine.add_request(torch.randint(3, cfg.vocab_size, (n,), generator=gen).tolist(), params)
+                engine.add_request(self.prompt(n), params)
             preempted = engine.scheduler.num_preemptions
             torch.cuda.synchronize()
             start = time.perf_counter()
@@ -198,69 +215,241 @@ def main():
                 steps += 1
             torch.cuda.synchronize()
             sec = time.perf_counter() - start
-            assert made == 64 * 256, made
-        print(json.dumps({"metric": f"OPT-{args.model.upper()} continuous batching: 64 requests, prompts 16-1,024, "
-                                    "256 new tokens each", "value": round(made / sec, 1), "unit": "generated tokens/s",
-                          "seconds": round(sec, 3), "steps": steps, "prompt_tokens": sum(lengths),
-                          "mean_time_to_first_token_ms": round(1e3 * sum(first.values()) / len(first), 2),
-                          "preemptions": engine.scheduler.num_preemptions - preempted, "dtype": args.dtype,
-                          "warmup": "the same workload once, untimed"}))
+            assert made == requests * new_tokens, made
+        return {"tokens_per_s": round(made / sec, 1), "seconds": round(sec, 3), "steps": steps,
+                "prompt_tokens": sum(lengths),
+                "mean_time_to_first_token_ms": round(1e3 * sum(first.values()) / len(first), 2),
+                "preemptions": engine.scheduler.num_preemptions - preempted}
+
+
+def room_for(raw, args, context, torch):
+    """How many requests of `context` tokens the device holds beside the model's weights, from what the model
+    declares (nothing is loaded)."""
+    from transformers_neuronx_amd.config.registry import resolve
+    from transformers_neuronx_amd.engine.model import DecoderModel
+    raw = {k: v for k, v in raw.items() if k != "name"}
+    if args.layers:
+        raw[args.layers_key] = args.layers
+    arch = resolve(raw)
+    model = DecoderModel(arch.build_spec(arch.config_class.from_dict(raw)))
+    dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    item = 2 if args.dtype == "bf16" else 4
+    weights = sum(item * int(torch.Size(d.shape).numel()) for d in model.param_decls() if d.tied_to is None)
+    # (the random weights are drawn apart and fused afterwards: a quarter of them is held twice meanwhile, and
+    # what that leaves free again is in pieces too small for the cache's blocks)
+    room = int(0.95 * torch.cuda.mem_get_info()[1]) - int(1.27 * weights) - (4 << 30)
+    return max(1, int(room // (model.cache_bytes_read(1, dtype) * context)))
+
+
+def flat_config(cfg, extra):
+    """The sizes of a run in one flat dictionary of at most 20 keys: the run's own first, then the typed
+    configuration's sizes (integers), then its options (strings and truth values) while there is room."""
+    out = dict(extra)
+    raw = cfg.to_dict()
+    skip = ("_token_id", "torch_dtype", "model_type", "init_std", "architectures")
+    fields = [(k, v) for k, v in raw.items() if not any(s in k for s in skip) and not isinstance(v, (list, dict))
+              and v is not None]
+    for wanted in ((int,), (str, bool)):
+        for k, v in fields:
+            if len(out) < 20 and k not in out and type(v) in wanted and not k.startswith("_"):
+                out[k] = v
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=None,
+                    help="the context length decoding ends at (default: the model's positions); a longer one than "
+                         "the configuration names is written into it, random weights allow any")
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
+    ap.add_argument("--layers-key", default="num_hidden_layers", help="the config.json key that --layers sets")
+    ap.add_argument("--positions-key", default="max_position_embeddings", help="the config.json key that --context raises")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--no-points", action="store_true", help="skip everything but the headline decode measurement")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the measurements at other models' sizes (the OPT-350m mix, OPT-66B) and the full-depth check")
+    ap.add_argument("--prefill-only", action="store_true", help="measure the prompt step alone (for profiles)")
+    ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS)
+    ap.add_argument("--model", default="6.7b",
+                    help="a name of " + ", ".join(PRESETS) + " (OPT-6.7B is the measurement of record), a model "
+                         "folder or a config.json file of any registered architecture; weights are random")
+    ap.add_argument("--do-sample", action="store_true",
+                    help="decode with temperature 0.8, top-k 50 and top-p 0.95 instead of greedily")
+    ap.add_argument("--mix", action="store_true",
+                    help="instead: 64 requests with prompts of 16 to 1,024 tokens and 256 new tokens each, all "
+                         "queued at once (a continuous-batching workload); prints its own line")
+    ap.add_argument("--own-products", action="store_true",
+                    help="every matrix product on our own kernels (none goes to the vendor library)")
+    ap.add_argument("--tune-all", action="store_true",
+                    help="time the vendor library's candidates for the many-rows products too")
+    ap.add_argument("--big-batch", type=int, default=None,
+                    help="the larger batch of `points` (64; cut to what fits the device at the full context)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
+        return 2
+
+    import torch
+    from transformers_neuronx_amd.kernels.hip import HipOps
+    if args.own_products:
+        HipOps.library_rows = 0
+    if args.tune_all:
+        HipOps.library_tune = 2
+    raw = raw_config(args.model)
+    name = raw["name"]
+    if args.context and args.context > raw.get(args.positions_key, 0):
+        raw[args.positions_key] = args.context
+    context = args.context or raw[args.positions_key]
+    tokens = args.prefill_tokens
+    peak_flops = PEAK_FLOPS[args.dtype]
+
+    # the larger batch of `points` is cut to what the device holds beside the weights at the full context
+    only = args.no_points or args.prefill_only or args.mix
+    big = args.big_batch or 64
+    if not only:
+        fits = room_for(raw, args, context, torch)
+        if big > fits:
+            log(f"{big} requests of {context} tokens do not fit beside the weights; the larger batch is {fits}")
+            big = fits
+        if args.batch > fits:
+            print(f"bench.py: {args.batch} requests of {context} tokens do not fit on this device ({fits} do)")
+            return 2
+    max_batch = args.batch if only else max(args.batch, big)
+    if args.mix:
+        max_batch = 64
+    bench = Bench(raw, args.dtype, max_batch, context, args.layers, args.layers_key)
+    cfg = bench.cfg
+
+    if args.mix:
+        got = bench.mix()
+        print(json.dumps(dict({"metric": f"{name} continuous batching: 64 requests, prompts 16-1,024, 256 new tokens each",
+                               "value": got.pop("tokens_per_s"), "unit": "generated tokens/s"}, **got,
+                              dtype=args.dtype, warmup="the same workload once, untimed")))
         return 0
     if args.prefill_only:
-        sec_p = prefill(PREFILL_TOKENS)
-        print(json.dumps({"prefill_ms": round(sec_p * 1e3, 3), "tokens": PREFILL_TOKENS,
-                          "frac": round(prefill_flops(raw, PREFILL_TOKENS) / sec_p / PEAK_FLOPS[args.dtype], 4)}))
+        sec_p, flops = bench.prefill(tokens)
+        print(json.dumps({"prefill_ms": round(sec_p * 1e3, 3), "tokens": tokens,
+                          "frac": round(flops / sec_p / peak_flops, 4)}))
         return 0
-    value, sec, read = decode(args.batch, args.steps, args.warmup)
-    print(f"[bench] decode batch {args.batch}: {value:.1f} tok/s, {sec * 1e3:.2f} ms/step", file=sys.stderr, flush=True)
+
+    ceilings = measured_ceilings(bench.runner.ops, torch) if not args.no_points else None
+    if ceilings:
+        log(f"this device at best: {ceilings}")
+    value, sec, read = bench.decode(args.batch, args.steps, args.warmup, do_sample=args.do_sample)
+    log(f"decode batch {args.batch}: {value:.1f} tok/s, {sec * 1e3:.2f} ms/step")
     achieved = read / sec / 1e9
     out = {
-        "metric": f"OPT-{args.model.upper()} decode tok/s @ batch 1/8/{args.big_batch}; prefill tok/s @ 2,048 tokens",
+        "metric": f"{name} decode tok/s @ batch 1/8/{big}; prefill tok/s @ {tokens:,} tokens",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic (seeded random weights and token ids)"
                                       + (", sampled (temperature 0.8, top-k 50, top-p 0.95)" if args.do_sample else ""),
-        "config": {"model": "OPT-" + args.model.upper(), "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "none",
-                   "layers": cfg.num_hidden_layers, "layers_of_model": layers_full, "hidden_size": cfg.hidden_size,
-                   "heads": cfg.num_attention_heads, "head_size": cfg.head_size, "ffn_dim": cfg.ffn_dim,
-                   "vocab_size": cfg.vocab_size, "max_positions": cfg.max_position_embeddings,
-                   "prompt_len": CONTEXT - args.steps - args.warmup - 1, "page_size": ecfg.page_size,
-                   "activation": cfg.activation_function, "pre_norm": cfg.do_layer_norm_before,
-                   "prefill_tokens": PREFILL_TOKENS},
+        "config": flat_config(cfg, {"model": name, "global_batch": args.batch, "seq_len": context, "parallelism": "none",
+                                    "layers_of_model": bench.layers_full, "page_size": bench.ecfg.page_size,
+                                    "prompt_len": context - args.steps - args.warmup - 1, "prefill_tokens": tokens}),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
     }
+    if ceilings:
+        out["ceilings"] = ceilings
+        out["roofline"]["peak_measured"] = ceilings["hbm_read_gbs_measured"]
+        out["roofline"]["frac_of_measured"] = round(achieved / ceilings["hbm_read_gbs_measured"], 4)
     if not args.no_points:
-        sec_p = prefill(PREFILL_TOKENS)
-        flops = prefill_flops(raw, PREFILL_TOKENS)
-        out["prefill"] = {"value": round(PREFILL_TOKENS / sec_p, 1), "tokens": PREFILL_TOKENS,
-                          "ms": round(sec_p * 1e3, 3), "frac": round(flops / sec_p / PEAK_FLOPS[args.dtype], 4)}
-        print(f"[bench] prefill: {out['prefill']}", file=sys.stderr, flush=True)
+        sec_p, flops = bench.prefill(tokens)
+        out["prefill"] = {"value": round(tokens / sec_p, 1), "tokens": tokens, "ms": round(sec_p * 1e3, 3),
+                          "frac": round(flops / sec_p / peak_flops, 4)}
+        if args.dtype == "bf16":
+            out["prefill"]["peak_measured_tflops"] = ceilings["mfma_tflops_measured"]
+            out["prefill"]["frac_of_measured"] = round(flops / sec_p / 1e12 / ceilings["mfma_tflops_measured"], 4)
+        log(f"prefill: {out['prefill']}")
         points = {}
-        for b, k, w in ((1, min(args.steps, 64), args.warmup),
-                        (args.big_batch, min(args.steps, 32), min(args.warmup, 4))):
-            v, s, rd = decode(b, k, w)
+        for b, k, w in ((1, min(args.steps, 64), args.warmup), (big, min(args.steps, 32), min(args.warmup, 4))):
+            v, s, rd = bench.decode(b, k, w, do_sample=args.do_sample)
             points[f"decode_b{b}"] = round(v, 2)
             points[f"decode_b{b}_ms"] = round(s * 1e3, 4)
             points[f"decode_b{b}_hbm_frac"] = round(rd / s / 1e9 / PEAK_HBM_GBS, 4)
-            print(f"[bench] decode batch {b}: {v:.1f} tok/s, {s * 1e3:.2f} ms/step", file=sys.stderr, flush=True)
+            log(f"decode batch {b}: {v:.1f} tok/s, {s * 1e3:.2f} ms/step")
         # the whole way from 512-token prompts to the full context, as the reference's benchmark generates whole
         # sequences (generation_demo.py:159-187) and reports the percentiles of their latency
         lat = []
-        first = 512
-        k = CONTEXT - first - 1 - 4
-        v, s, rd = decode(args.batch, k, 4, prompt_len=first, latencies=lat)
+        first = min(512, context // 4)
+        k = context - first - 1 - 4
+        v, s, rd = bench.decode(args.batch, k, 4, prompt_len=first, latencies=lat, do_sample=args.do_sample)
         lat.sort()
-        points["decode_512_to_2048"] = round(v, 2)
-        points["decode_512_to_2048_ms"] = round(s * 1e3, 4)
-        points["decode_512_to_2048_hbm_frac"] = round(rd / s / 1e9 / PEAK_HBM_GBS, 4)
+        tag = f"decode_{first}_to_{context}"
+        points[tag] = round(v, 2)
+        points[tag + "_ms"] = round(s * 1e3, 4)
+        points[tag + "_hbm_frac"] = round(rd / s / 1e9 / PEAK_HBM_GBS, 4)
         for q in (0, 50, 90, 95, 99, 100):
             points[f"step_latency_p{q}_ms"] = round(lat[min(len(lat) - 1, int(len(lat) * q / 100))] * 1e3, 4)
-        print(f"[bench] decode batch {args.batch}, 512 -> 2,048: {v:.1f} tok/s, {s * 1e3:.2f} ms/step",
-              file=sys.stderr, flush=True)
+        log(f"decode batch {args.batch}, {first} -> {context:,}: {v:.1f} tok/s, {s * 1e3:.2f} ms/step")
         out["points"] = points
+        if not args.no_extras and args.dtype == "bf16":
+            extras(out, bench, raw, args, context)
     print(json.dumps(out))
     return 0
+
+
+def extras(out, bench, raw, args, context):
+    """What the line carries beyond its own model: the full-depth check against a float32 engine, and the other
+    workloads the family is measured on. None of them may cost the line: what fails is named and left out."""
+    import torch
+    from transformers_neuronx_amd.testing import compare_precisions
+    points = out["points"]
+    try:
+        # the float32 engine on the very weights of the bfloat16 one (drawn in bfloat16 from the same seed)
+        wide = Bench(raw, "fp32", 1, context, args.layers, args.layers_key, storage=torch.bfloat16, max_tokens=384)
+        report = compare_precisions(wide.engine, bench.engine, bench.prompt(300), 21)
+        wide.close()
+        out["check"] = {k: (round(v, 6) if isinstance(v, float) else v) for k, v in report.items()}
+        out["check"]["what"] = ("bfloat16 engine against the float32 engine on the same weights, all layers: a 300-token "
+                                "prompt and 20 decode steps; allclose is atol 1.0, rtol 1e-3")
+        log(f"check: {out['check']}")
+    except Exception as e:                                   # noqa: BLE001
+        out["check"] = {"error": f"{type(e).__name__}: {e}"[:200]}
+    bench.close()
+    try:
+        small = Bench(raw_config("350m"), "bf16", 64, 2048)
+        got = small.mix()
+        small.close()
+        for k, v in got.items():
+            points[f"mix_350m_{k}"] = v
+        log(f"OPT-350m mix: {got}")
+    except Exception as e:                                   # noqa: BLE001
+        points["mix_350m_error"] = f"{type(e).__name__}: {e}"[:200]
+    try:
+        free = torch.cuda.mem_get_info()[0]
+        if free < 262e9:
+            points["opt66b_skipped"] = f"{free / 1e9:.0f} GB free"
+            return
+        # Twice: with the cache of 8 requests most matrices get their tile-ordered copy beside the 131 GB of
+        # weights; then with the largest batch that fits at the full context (the family's is 32), where
+        # hardly any does.
+        def decode_points(large, batches):
+            for b, k, w in batches:
+                v, s, rd = large.decode(b, k, w)
+                points[f"opt66b_decode_b{b}"] = round(v, 2)
+                points[f"opt66b_decode_b{b}_ms"] = round(s * 1e3, 3)
+                points[f"opt66b_decode_b{b}_hbm_frac"] = round(rd / s / 1e9 / PEAK_HBM_GBS, 4)
+                log(f"OPT-66B decode batch {b}: {v:.1f} tok/s, {s * 1e3:.2f} ms/step")
+
+        large = Bench(raw_config("66b"), "bf16", 8, 2048)
+        decode_points(large, ((8, 16, 4), (1, 16, 4)))
+        large.close()
+        most = min(32, room_for(raw_config("66b"), argparse.Namespace(layers=None, layers_key="", dtype="bf16"), 2048, torch))
+        large = Bench(raw_config("66b"), "bf16", most, 2048)
+        decode_points(large, ((most, 12, 3),))
+        sec_p, flops = large.prefill(PREFILL_TOKENS)
+        points["opt66b_prefill_ms"] = round(sec_p * 1e3, 2)
+        points["opt66b_prefill_frac"] = round(flops / sec_p / PEAK_FLOPS["bf16"], 4)
+        log(f"OPT-66B prefill: {sec_p * 1e3:.1f} ms")
+        large.close()
+    except Exception as e:                                   # noqa: BLE001
+        points["opt66b_error"] = f"{type(e).__name__}: {e}"[:200]
 
 
 if __name__ == "__main__":

@@ -14,6 +14,7 @@ from transformers_neuronx_amd.config import EngineConfig
 from transformers_neuronx_amd.opt.config import OPTConfig
 from transformers_neuronx_amd.engine import StepEntry
 from transformers_neuronx_amd.engine.engine import LLMEngine
+from transformers_neuronx_amd.engine.scheduler import PENDING
 from transformers_neuronx_amd.engine.factory import runner_from_folder
 from transformers_neuronx_amd.sampling import SamplingParams
 
@@ -191,6 +192,27 @@ def test_a_step_that_plans_nothing_while_work_waits_raises(tiny_folders):
     engine.scheduler.schedule = lambda: []          # a scheduler that has work and plans none of it
     with pytest.raises(RuntimeError, match="no progress"):
         engine.run()
+    with pytest.raises(RuntimeError, match="no progress"):      # a caller's own loop over step() meets it too
+        while engine.has_work:
+            engine.step()
+    # the entry point's loop: a pool that the scheduler cannot plan the batch into
+    from transformers_neuronx_amd import OPTForSampling
+    model = OPTForSampling.from_pretrained(folder, batch_size=1, amp="f32", n_positions=32, kernels="reference",
+                                           device="cpu").load()
+    model.engine.scheduler.schedule = lambda: []
+    with pytest.raises(RuntimeError, match="no progress"):
+        model.sample(torch.tensor([[5, 6, 7]]), 8)
+
+
+def test_end_tokens_of_any_integer_type():
+    import numpy as np
+    assert SamplingParams(eos_token_id=np.int64(7)).eos_ids == (7,)
+    assert SamplingParams(eos_token_id=torch.tensor(7)).eos_ids == (7,)
+    assert SamplingParams(eos_token_id=[np.int32(7), 9]).eos_ids == (7, 9)
+    assert SamplingParams(eos_token_id=None).eos_ids == ()
+    for bad in (7.5, "seven", [7, 1.5]):
+        with pytest.raises(ValueError, match="eos_token_id"):
+            SamplingParams(eos_token_id=bad)
 
 
 def test_sampled_tokens_follow_the_plain_sampler(tiny_folders):
@@ -301,6 +323,13 @@ def test_entry_point_in_the_reference_manner(tiny_folders, tmp_path):
     torch.testing.assert_close(logits[0, 2:], plain_opt.forward_logits(weights, cfg, [5, 9]), atol=1e-5, rtol=1e-5)
     torch.testing.assert_close(logits[1], plain_opt.forward_logits(weights, cfg, [7, 7, 100, 3]), atol=1e-5, rtol=1e-5)
     model.neuron_config.output_all_logits = False
+    # a smaller batch after a larger one: the rows it does not name give back what they held
+    model(ids)
+    assert sorted(model.engine.runner.cache.requests) == [("row", 0), ("row", 1)]
+    logits = model(ids[1:])
+    assert sorted(model.engine.runner.cache.requests) == [("row", 0)]
+    model.engine.runner.cache.check()
+    torch.testing.assert_close(logits[0], plain_opt.forward_logits(weights, cfg, ids[1].tolist())[-1], atol=1e-5, rtol=1e-5)
     model.reset()
     assert not model.engine.runner.cache.requests
     # a streamer gets one token of every row at a time and is told the end (sampling.py:159-160, :172-173),
@@ -635,6 +664,28 @@ def test_a_request_taken_out_midway(tiny_folders, run_ahead):
     assert got[late] == [] and ids[1] not in engine.requests
     with pytest.raises(KeyError):
         engine.abort_request("nobody")
+    # a request that has ended by its length while its last token is still in a step under way: taken out, it
+    # keeps no placeholder and reports nothing more; handed over in the ordinary way, only once the token is there
+    for take_out in (True, False):
+        rid = engine.add_request(prompts[0], SamplingParams(max_new_tokens=2, do_sample=False, ignore_eos=True))
+        seen = []
+        while not engine.requests[rid].finished:
+            seen += [o.token for o in engine.step()]
+        want = plain_opt.greedy(weights, cfg, prompts[0], 2)[len(prompts[0]):]
+        if take_out:
+            req = engine.abort_request(rid)
+            assert PENDING not in req.output and req.output == seen and req.finish_reason == "length"
+            while engine.has_work:
+                assert engine.step() == []
+        else:
+            if run_ahead:
+                assert PENDING in engine.requests[rid].output
+                with pytest.raises(ValueError, match="under way"):
+                    engine.pop_request(rid)
+            while engine.has_work:
+                seen += [o.token for o in engine.step()]
+            assert engine.pop_request(rid).output == seen == want
+        assert not runner.cache.requests
 
 
 def test_several_tokens_end_a_request(tiny_folders):

@@ -397,6 +397,34 @@ def test_full_layer_sizes_against_plain(size):
         assert bool((got.argmax(-1) == want.argmax(-1))[clear].all())
 
 
+def test_full_depth_bfloat16_against_float32():
+    """All 32 layers of OPT-6.7B's sizes on the same random weights (drawn in bfloat16): the float32 engine and
+    the bfloat16 engine generate from a 300-token prompt through `LLMEngine`, one step over the prompt and
+    20 decode steps (recorded ones, with running ahead), the bfloat16 engine held to the float32 engine's
+    tokens. The yardstick is the reference's own for a low-precision run against a float32 one
+    (generation_demo.py:437-443: allclose(atol=1.0, rtol=1e-3) and the same token, step by step) with the
+    plain distance beside it: a bfloat16 kernel that loses part of a sum over the depth shows here, where a
+    two-layer model hides it. The float32 engine at this size holds 26.6 GB of weights."""
+    from transformers_neuronx_amd.config import EngineConfig
+    from transformers_neuronx_amd.engine.engine import LLMEngine
+    from transformers_neuronx_amd.engine.factory import runner_from_random
+    from transformers_neuronx_amd.opt.config import OPTConfig
+    from transformers_neuronx_amd.testing import compare_precisions
+    cfg = OPTConfig.from_dict(dict(FULL_SIZES["6.7b"], num_hidden_layers=32))
+    prompt = torch.randint(3, cfg.vocab_size, (300,), generator=torch.Generator().manual_seed(11)).tolist()
+    engines = []
+    for dtype in (torch.float32, torch.bfloat16):
+        ecfg = EngineConfig(dtype=dtype, page_size=64, max_tokens=384, max_num_seqs=1)
+        engines.append(LLMEngine(runner_from_random(cfg, 5, ecfg, storage=torch.bfloat16), ecfg))
+    report = compare_precisions(engines[0], engines[1], prompt, 21)
+    print("full depth, bfloat16 against float32:", report)
+    assert engines[1].runner.graph_replays >= 19
+    assert report["rows"] == report["allclose_rows"] == 21, report
+    assert report["rel"] <= TOL["bfloat16"], report
+    assert report["clear_rows"] >= 5, report          # the comparison of choices is not empty
+    assert report["clear_same"] == report["clear_rows"], report
+
+
 def _odd(v, heads, hs, layers, ffn, proj, pre, act, bias, affine, eps):
     return dict(architectures=["OPTForCausalLM"], model_type="opt", vocab_size=v, hidden_size=heads * hs,
                 num_hidden_layers=layers, num_attention_heads=heads, ffn_dim=ffn, max_position_embeddings=200,

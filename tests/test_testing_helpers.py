@@ -57,3 +57,40 @@ def test_validate_on_the_gpu(tiny_folders):
     inputs = batch_varying_lengths(cfg["vocab_size"], 4, 9, 1, torch.Generator().manual_seed(7))
     model = OPTForSampling.from_pretrained(folder, batch_size=4, amp="f32", n_positions=40, page_size=16)
     validate(_golden(weights, cfg), model, inputs, sequence_length=20)
+
+
+def test_compare_precisions_on_the_host(tiny_folders):
+    """The full-depth check's helper on the torch rendition of the kernels: an engine against itself differs
+    nowhere, a bfloat16 engine held to the float32 engine's tokens differs by bfloat16 rounding and no more,
+    and the logits the helper keeps are the plain implementation's at the followed tokens."""
+    from transformers_neuronx_amd.config import EngineConfig
+    from transformers_neuronx_amd.engine.engine import LLMEngine
+    from transformers_neuronx_amd.engine.factory import runner_from_folder
+    from transformers_neuronx_amd.testing import compare_logits, compare_precisions, greedy_logits
+    folder, cfg, weights = tiny_folders["A"]
+
+    def engine(dtype):
+        ecfg = EngineConfig(dtype=dtype, kernels="reference", device="cpu", page_size=16, max_tokens=128, max_num_seqs=2,
+                            cast_float32_weights=True)
+        return LLMEngine(runner_from_folder(folder, ecfg), ecfg)
+
+    wide, narrow = engine(torch.float32), engine(torch.bfloat16)
+    prompt = torch.randint(3, 512, (21,), generator=torch.Generator().manual_seed(3)).tolist()
+    same = compare_precisions(wide, wide, prompt, 6)
+    assert same["rel"] == 0.0 and same["rows"] == same["same_argmax"] == same["clear_rows"] == same["clear_same"] == 6
+    got = compare_precisions(wide, narrow, prompt, 6)
+    assert 0.0 < got["rel"] < 3e-2 and got["allclose_rows"] == 6 and got["clear_same"] == got["clear_rows"]
+    tokens, rows = greedy_logits(wide, prompt, 6)
+    assert tokens == plain_opt.greedy(weights, cfg, prompt, 6)[len(prompt):]
+    forced = [7, 9, 11, 13, 15, 17]
+    tokens, rows = greedy_logits(narrow, prompt, 6, follow=forced)
+    assert tokens == forced
+    want = plain_opt.forward_logits(weights, cfg, prompt + forced[:-1])[len(prompt) - 1:]
+    assert compare_logits(rows, want)["rel"] < 3e-2
+    # a row whose winner changes where the golden one leads clearly is counted as such
+    bad = want.clone()
+    bad[2, int(want[2].argmax())] -= 1.0
+    report = compare_logits(bad, want)
+    assert report["same_argmax"] == 5 and report["max_abs_diff"] == 1.0 and report["clear_rows"] == report["clear_same"]
+    top2 = want[2].topk(2).values
+    assert float(top2[0] - top2[1]) < 2.0         # (the changed row is no clear one: its winner led by less than 2 x 1.0)

@@ -117,7 +117,7 @@ class CausalLMForSampling:
         from .kernels import build
         os.makedirs(directory, exist_ok=True)
         with open(os.path.join(directory, "kernels.json"), "w") as fp:
-            json.dump({m: build.compile_module(m) for m in build.MODULES}, fp, indent=1)
+            json.dump({m: build.compile_module(m) for m in build.modules()}, fp, indent=1)   # also those that parts brought
 
     def is_compiled(self) -> bool:
         """base.py:143-151: whether the model is ready to run."""
@@ -159,8 +159,9 @@ class CausalLMForSampling:
             return self._forward_sequences(input_ids, cache_ids, start_ids)
         rows = self._rows(input_ids, start_ids)
         if cache_ids is None:
-            for b in range(len(rows)):
-                runner.finish(("row", b))
+            # every row starts afresh, also rows of an earlier, larger batch that this one does not name
+            for key in [k for k in runner.cache.requests if isinstance(k, tuple) and k[:1] == ("row",)]:
+                runner.finish(key)
         else:
             first = int(torch.as_tensor(cache_ids).flatten()[0])
             for b, toks in enumerate(rows):

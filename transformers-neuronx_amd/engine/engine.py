@@ -146,15 +146,25 @@ class LLMEngine:
         the step it ran, or with `run_ahead` those of the step started by the call before."""
         # a request that may not repeat its n-grams needs its last token on the host before the next is chosen
         in_step = any(q.params.no_repeat_ngram_size and not q.finished for q in self.requests.values())
+        idle = self._started is None
         if not self.run_ahead or self.record_timings or in_step:
             out = self._finish(self._started) if self._started is not None else []
             self._started = None
             started = self._start()
+            self._check_progress(idle)
             return out + (self._finish(started) if started is not None else [])
         started = self._start()
         out = self._finish(self._started) if self._started is not None else []
         self._started = started
+        self._check_progress(idle)
         return out
+
+    def _check_progress(self, idle: bool) -> None:
+        """Requests wait, no step was under way when this call began and the scheduler has planned none: no
+        later call would do better (a pool too small for a lone request raises `OutOfPages` where it is
+        found; this is what is left, and every loop over `step()` meets it)."""
+        if idle and not self._planned and self.scheduler.has_work:
+            raise RuntimeError("no progress: requests wait, the scheduler plans no step and none is under way")
 
     def profile(self, steps: int = 1):
         """Run `steps` steps with events around every kernel launch (no recording, no running ahead) and
@@ -176,11 +186,7 @@ class LLMEngine:
     def run(self, on_token: Optional[Callable[[StepOutput], None]] = None) -> None:
         """Step until every request has ended."""
         while self.has_work:
-            idle = self._started is None
-            outs = self.step()
-            if idle and not self._planned and self.scheduler.has_work:
-                raise RuntimeError("no progress: requests wait, the scheduler plans no step and none is under way")
-            for out in outs:
+            for out in self.step():
                 if on_token:
                     on_token(out)
 
@@ -208,6 +214,9 @@ class LLMEngine:
         req = self.requests[req_id]
         if not req.finished:
             raise ValueError(f"request {req_id!r} has not ended")
+        if PENDING in req.output:
+            raise ValueError(f"request {req_id!r} has ended, but its last token is in a step under way: "
+                             "the next call of step() delivers it")
         return self.requests.pop(req_id)
 
     def reset(self) -> None:

@@ -94,13 +94,16 @@ def runner_from_folder(folder: str, cfg: EngineConfig) -> ModelRunner:
     return build_runner(model_config, Checkpoint(folder), cfg)
 
 
-def runner_from_random(model_config, seed: int, cfg: EngineConfig) -> ModelRunner:
+def runner_from_random(model_config, seed: int, cfg: EngineConfig, storage: Optional[torch.dtype] = None) -> ModelRunner:
     """Random weights drawn on the device, without a folder (for models too large
-    to write for a measurement)."""
+    to write for a measurement). `storage` is the precision the matrices are drawn in (the engine's own
+    if not given): a float32 engine on bfloat16-drawn matrices has the very weights of a bfloat16 engine
+    with the same seed."""
     device = _device_of(cfg)
     arch = resolve(model_config.to_dict())
     spec = arch.build_spec(model_config)
     decls = DecoderModel(spec).param_decls()
-    storage = torch.float32 if cfg.dtype == torch.float32 else torch.bfloat16
+    if storage is None:
+        storage = torch.float32 if cfg.dtype == torch.float32 else torch.bfloat16
     source = TensorDict(random_tensors(decls, spec.init_std, seed, storage, device))
     return build_runner(model_config, source, cfg)       # the source alone holds the tensors, and lets go of them

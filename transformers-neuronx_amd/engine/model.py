@@ -80,6 +80,31 @@ class DecoderModel:
         """{cache id: need} of the calls that write a cache."""
         return {cid: self.layers[layer].mixer.cache_need() for layer, cid, writes in self.schedule if writes}
 
+    # ---------------------------------------------------------------- accounting (for measurements)
+
+    def step_flops(self, tokens: float, keys: float, wanted: float) -> float:
+        """Multiply-adds times two of a step of `tokens` tokens that see `keys` cached tokens each on
+        average (a whole prompt of T tokens: (T + 1) / 2) and ask for `wanted` rows of logits."""
+        per_token = self.embedding.flops_per_token(keys)
+        for layer, _, _ in self.schedule:
+            l = self.layers[layer]
+            per_token += sum(p.flops_per_token(keys) for p in (l.mixer, l.feed_forward, l.mixer_norm, l.feed_forward_norm))
+        return tokens * per_token + wanted * self.head.flops_per_token(keys)
+
+    def cache_bytes_read(self, keys: float, dtype: torch.dtype, page_size: int = 1) -> float:
+        """Bytes of its request's cache that one decoded token reads at a context of `keys` tokens: every call
+        of the run order reads the cache it names (a windowed one up to its window)."""
+        needs = {cid: self.layers[layer].mixer.cache_need() for layer, cid, writes in self.schedule if writes}
+        total = 0.0
+        for _, cid, _ in self.schedule:
+            need = needs.get(cid)
+            if need is None or need.kind != "paged":
+                continue
+            from ..cache.manager import CacheManager
+            per_token = CacheManager.bytes_per_page({0: need}, page_size, dtype) / page_size
+            total += per_token * (min(keys, need.window) if need.window else keys)
+        return total
+
     # ---------------------------------------------------------------- weights
 
     def load(self, source, ops, dtype: torch.dtype, device, cast_float32: bool = False,

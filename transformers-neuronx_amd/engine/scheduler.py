@@ -266,11 +266,10 @@ class Scheduler:
         """Take a request out, wherever it stands: it ends with the reason "aborted" and gives back what it
         holds. A token that a step under way is still to deliver for it is dropped when it comes (`resolve`
         finds the request shorter than the place the token was meant for)."""
-        if req.finished:
-            return
-        if PENDING in req.output:
+        if PENDING in req.output:          # also of a request that has ended by its length with its last token under way
             del req.output[req.output.index(PENDING):]
-        self._end(req, "aborted", [])
+        if not req.finished:
+            self._end(req, "aborted", [])
 
     def record(self, runs: List[ScheduledRun]) -> List[Request]:
         """What the step computes, before its tokens are known: every run that samples gets `PENDING` as

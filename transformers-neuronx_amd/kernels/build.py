@@ -18,7 +18,7 @@ import time
 from typing import Dict, List, Optional
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
-MODULES = ("elementwise", "gemm", "attention", "sampling")
+MODULES = ("elementwise", "gemm", "attention", "sampling", "probe")
 ARCH = "gfx950"
 FLAGS = ["-O3", f"--offload-arch={ARCH}", "-shared", "-fPIC", "-std=c++17",
          # packed float32 instructions are kept out of the generated code

@@ -76,6 +76,10 @@ _SIGNATURES = {
         "tnx_sample": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                        _c_int, _c_void_p],
     },
+    "probe": {
+        "tnx_probe_stream_read": [_c_void_p, ctypes.c_size_t, _c_void_p, _c_int, _c_void_p],
+        "tnx_probe_mfma_loop": [_c_int, _c_int, _c_void_p, _c_void_p],
+    },
 }
 
 

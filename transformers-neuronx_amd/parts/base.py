@@ -61,6 +61,20 @@ class Part:
         self.ops = ops
         self.dtype = dtype
 
+    def flops_per_token(self, keys: float = 0.0) -> float:
+        """Multiply-adds times two that one token costs in this part, for a measurement's accounting; `keys`
+        is the number of cached tokens of its request that the token sees. By default every declared
+        matrix meets every token once; a part that does otherwise (experts of which a token takes some,
+        products over the cache) says so."""
+        count = 0
+        for d in self.param_decls(""):
+            if d.role == "matrix":
+                n = 1
+                for dim in d.shape:
+                    n *= dim
+                count += n
+        return 2.0 * count
+
 
 class Mixer(Part):
     """Mixes information between the tokens of a request.

@@ -86,6 +86,10 @@ class Attention(Mixer):
     def first_weight(self):
         return self.w_qkv
 
+    def flops_per_token(self, keys: float = 0.0) -> float:
+        seen = min(keys, self.window) if self.window else keys
+        return super().flops_per_token(keys) + 4.0 * self.num_heads * self.head_size * seen   # q k^T and p v
+
     def forward(self, h, ctx, cache, residual):
         if cache.writes != self.own_kv:
             raise ValueError("an attention mixer with own_kv writes its cache; one without reads another's")

@@ -1,4 +1,5 @@
 """What a request asks of the sampler."""
+import operator
 from dataclasses import dataclass
 from typing import Optional, Sequence, Tuple, Union
 
@@ -58,6 +59,17 @@ class SamplingParams:
             raise ValueError(f"`ngram_size` has to be a strictly positive integer, but is {self.no_repeat_ngram_size}")
         if float(self.temperature) < 0:
             raise ValueError("temperature has to be a non-negative float (0 is greedy).")
+        # one token or several, of any integer type (a numpy or tensor scalar too): settled here, not when
+        # the first token is compared with it
+        if self.eos_token_id is not None:
+            try:
+                self.eos_token_id = operator.index(self.eos_token_id)
+            except TypeError:
+                try:
+                    self.eos_token_id = tuple(operator.index(t) for t in self.eos_token_id)
+                except TypeError:
+                    raise ValueError(f"eos_token_id has to be an integer or a sequence of integers, got "
+                                     f"{self.eos_token_id!r}") from None
 
     @property
     def eos_ids(self) -> Tuple[int, ...]:
