@@ -91,7 +91,7 @@ def measured_ceilings(ops, torch):
         return best
 
     read = timed(lambda: ops.call("probe", "tnx_probe_stream_read", buf.data_ptr(), buf.numel(), out.data_ptr(),
-                                  units * 8, ops.stream()), 5)
+                                  units * 32, ops.stream()), 5)
     iterations, blocks = 20000, units * 8
     loop = timed(lambda: ops.call("probe", "tnx_probe_mfma_loop", blocks, iterations, out.data_ptr(), ops.stream()), 3)
     del buf, out

@@ -180,7 +180,10 @@ def test_save_notes_the_built_kernels(tiny_folders, tmp_path):
     model = OPTForSampling.from_pretrained(tiny_folders["A"][0], batch_size=1, amp="bf16", n_positions=32).load()
     model.save(str(tmp_path / "artifacts"))
     noted = json.load(open(tmp_path / "artifacts" / "kernels.json"))
-    assert set(noted) == {"elementwise", "gemm", "attention", "sampling"} and all(os.path.exists(p) for p in noted.values())
+    from transformers_neuronx_amd.kernels import build
+    # every registered module, those that parts of the tests brought among them
+    assert set(noted) == set(build.modules()) >= {"elementwise", "gemm", "attention", "sampling", "probe"}
+    assert all(os.path.exists(p) for p in noted.values())
     again = OPTForSampling.from_pretrained(tiny_folders["A"][0], batch_size=1, amp="bf16", n_positions=32)
     again.load(str(tmp_path / "artifacts")).to_neuron()
     assert again.is_compiled() and again.sample(torch.tensor([[5, 6, 7]]), 6).shape == (1, 6)

@@ -61,6 +61,14 @@ __device__ __forceinline__ float from_f32<float>(float x) { return x; }
 template <>
 __device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) { return (bf16_t)x; }
 
+// 16 bytes that are read once and by no one else (a weight in a decode step, a key or value of a request):
+// the load is marked as streaming, so that the lines it brings in are the first to leave the caches again.
+// A kernel that only reads memory reaches 6.8 TB/s on an MI355X with such loads and 5.8 to 6.1 with plain ones.
+typedef __attribute__((ext_vector_type(4))) unsigned tnx_u32x4;
+__device__ __forceinline__ bf16x8 load_once(const bf16_t* p) {
+  return __builtin_bit_cast(bf16x8, __builtin_nontemporal_load((const tnx_u32x4*)p));
+}
+
 // Element `i` of an array whose dtype is known at run time only.
 __device__ __forceinline__ float load_any(const void* p, int dtype, size_t i) {
   return dtype == TNX_F32 ? ((const float*)p)[i] : (float)((const bf16_t*)p)[i];
@@ -180,6 +188,13 @@ inline int tnx_compute_units() {
 // these loads must have no other instruction that reads M0, which holds for every kernel of ours.
 __device__ __forceinline__ void load_to_lds(const void* base, unsigned offset, unsigned lds) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds), "v"(offset), "s"(base)
+               : "memory");
+}
+// the same for bytes that are read once (see `load_once`)
+__device__ __forceinline__ void load_to_lds_once(const void* base, unsigned offset, unsigned lds) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
                :
                : "s"(lds), "v"(offset), "s"(base)
                : "memory");

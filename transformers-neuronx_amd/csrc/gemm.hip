@@ -609,7 +609,7 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
 #pragma unroll
       for (int j = 0; j < RT; ++j)
 #pragma unroll
-        for (int s = 0; s < 4; ++s) wf[slot][j][s] = *(const bf16x8*)(wrow[j] + (size_t)k * W_STEP + W_LOAD * s);
+        for (int s = 0; s < 4; ++s) wf[slot][j][s] = load_once(wrow[j] + (size_t)k * W_STEP + W_LOAD * s);
     };
     // NORMED: the float32 elements wait in registers as they came and are shifted, summed and rounded when
     // their step is multiplied, a step after they were asked for (used at once they would make the wave
@@ -1005,7 +1005,7 @@ gemm_bf16_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w_
     for (int u = 0; u < MT; ++u) load_to_lds(xbase, xoff[u], x_lds + stage * XSTAGE + (wave + 4 * u) * 1024);
     const char* wbase = wtile + (size_t)st * (128 * 16 * 2);
 #pragma unroll
-    for (int s = 0; s < 4; ++s) load_to_lds(wbase + 1024 * s, (unsigned)((r * 4 + g) * 16), w_lds + stage * WSTAGE + 1024 * s);
+    for (int s = 0; s < 4; ++s) load_to_lds_once(wbase + 1024 * s, (unsigned)((r * 4 + g) * 16), w_lds + stage * WSTAGE + 1024 * s);
   };
   f32x4 acc[MT];
 #pragma unroll

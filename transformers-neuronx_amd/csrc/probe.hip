@@ -5,25 +5,29 @@
 
 TNX_DEFINE_ERROR_API
 
-// Every block reads its share of the buffer 16 bytes a lane, four loads in flight a lane, and leaves the
-// exclusive-or of what it read, so that no load can be left out.
+// Every block reads its share of the buffer 16 bytes a lane, eight loads in flight a lane, marked as streaming
+// (of the forms tried, plain or streaming loads, four or eight in flight, 4 to 32 blocks a compute unit,
+// strided or in runs, this one read fastest: 6.8 TB/s against 5.5 to 6.3), and leaves the exclusive-or of what
+// it read, so that no load can be left out.
 __global__ void __launch_bounds__(256)
-stream_read_kernel(const uint4* __restrict__ data, size_t vectors, unsigned* __restrict__ out) {
+stream_read_kernel(const tnx_u32x4* __restrict__ data, size_t vectors, unsigned* __restrict__ out) {
   const size_t stride = (size_t)gridDim.x * 256;
   size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  uint4 a = {0, 0, 0, 0}, b = a, c = a, d = a;
-  for (; i + 3 * stride < vectors; i += 4 * stride) {
-    const uint4 v0 = data[i], v1 = data[i + stride], v2 = data[i + 2 * stride], v3 = data[i + 3 * stride];
-    a.x ^= v0.x, a.y ^= v0.y, a.z ^= v0.z, a.w ^= v0.w;
-    b.x ^= v1.x, b.y ^= v1.y, b.z ^= v1.z, b.w ^= v1.w;
-    c.x ^= v2.x, c.y ^= v2.y, c.z ^= v2.z, c.w ^= v2.w;
-    d.x ^= v3.x, d.y ^= v3.y, d.z ^= v3.z, d.w ^= v3.w;
+  tnx_u32x4 acc[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) acc[u] = (tnx_u32x4){0, 0, 0, 0};
+  for (; i + 7 * stride < vectors; i += 8 * stride) {
+    tnx_u32x4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(data + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc[u] ^= v[u];
   }
-  for (; i < vectors; i += stride) {
-    const uint4 v = data[i];
-    a.x ^= v.x, a.y ^= v.y, a.z ^= v.z, a.w ^= v.w;
-  }
-  const unsigned x = a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+  for (; i < vectors; i += stride) acc[0] ^= __builtin_nontemporal_load(data + i);
+  tnx_u32x4 a = acc[0];
+#pragma unroll
+  for (int u = 1; u < 8; ++u) a ^= acc[u];
+  const unsigned x = a[0] ^ a[1] ^ a[2] ^ a[3];
   if (x == 0x9E3779B9u) out[blockIdx.x] = x;      // (all but never: the sums have to be made for it)
 }
 
@@ -31,7 +35,7 @@ stream_read_kernel(const uint4* __restrict__ data, size_t vectors, unsigned* __r
 extern "C" int tnx_probe_stream_read(const void* data, size_t bytes, void* out, int blocks, hipStream_t stream) {
   TNX_REQUIRE(bytes % 16 == 0 && ((uintptr_t)data & 15) == 0, "stream_read: the buffer must be whole 16-byte vectors");
   TNX_REQUIRE(blocks > 0 && blocks <= 65536, "stream_read: %d blocks", blocks);
-  stream_read_kernel<<<blocks, 256, 0, stream>>>((const uint4*)data, bytes / 16, (unsigned*)out);
+  stream_read_kernel<<<blocks, 256, 0, stream>>>((const tnx_u32x4*)data, bytes / 16, (unsigned*)out);
   TNX_CHECK_LAUNCH("stream_read");
   return 0;
 }
