@@ -303,6 +303,56 @@ def test_recorded_decode_steps_equal_open_ones(tiny_folders, tiny_folders_bf16, 
         assert float((rec_rows[key] - want).abs().max() / expected[rid].abs().max()) <= TOL[dtype]
 
 
+LONG = dict(architectures=["OPTForCausalLM"], model_type="opt", vocab_size=300, hidden_size=128, num_hidden_layers=2,
+            num_attention_heads=2, ffn_dim=256, max_position_embeddings=1100, init_std=0.08)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("batch", [2, 9])
+def test_recorded_decoding_across_the_marks_of_256_keys(tmp_path, dtype, batch):
+    """Requests about as long as one another are decoded in blocks of 256 keys, and a recorded step is
+    recorded again when the longest of them needs another block: from 250 to 1,030 tokens that happens four
+    times. Every step is a recorded one; the logits at every mark (the three steps around it) and at every
+    50th position are compared with the plain implementation, for the first and the last request. Nine requests
+    of two heads are 18 (request, head) pairs, which the kernel cuts further than two requests."""
+    from safetensors.torch import load_file
+    from transformers_neuronx_amd.config import EngineConfig
+    from transformers_neuronx_amd.engine import StepEntry
+    from transformers_neuronx_amd.engine.factory import runner_from_folder
+    from transformers_neuronx_amd.opt.config import OPTConfig
+    from transformers_neuronx_amd.weights import write_random_model
+    folder = str(tmp_path / "long")
+    write_random_model(OPTConfig.from_dict(LONG), folder, seed=8, dtype=dtype)
+    weights = {k: v.float() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    cfg = OPTConfig.from_dict(LONG).to_dict()
+    total, first = 1030, 250
+    requests = _requests(cfg, [total - i % 3 for i in range(batch)], seed=batch)        # alike, not equal
+    ids = list(requests)
+    watched = [ids[0], ids[-1]]
+    expected = {rid: plain_opt.forward_logits(weights, cfg, requests[rid]) for rid in watched}
+    ecfg = EngineConfig(dtype=dtype, page_size=64, max_tokens=batch * 1088, max_num_seqs=batch, use_graphs=True)
+    runner = runner_from_folder(folder, ecfg)
+    runner.step([StepEntry(rid, requests[rid][:first], []) for rid in ids])
+    looked = set(range(first, total - 3, 50)) | {m + d for m in (256, 512, 768, 1024) for d in (-2, -1, 0, 1)}
+    worst = 0.0
+    shapes = set()
+    for pos in range(first, total - 3):
+        logits = runner.step([StepEntry(rid, [requests[rid][pos]], [0]) for rid in ids])
+        shapes.add(runner._last_ctx.plan_host["record:decode"])
+        if pos in looked:
+            got = logits.float().cpu()
+            for rid in watched:
+                want = expected[rid][pos]
+                err = float((got[ids.index(rid)] - want).abs().max() / expected[rid].abs().max())
+                worst = max(worst, err)
+                assert err <= TOL[dtype], (rid, pos, err)
+                if dtype == "float32":
+                    assert int(got[ids.index(rid)].argmax()) == int(want.argmax())
+    assert runner.graph_replays == total - 3 - first
+    assert shapes == {(k, True) for k in (1, 2, 3, 4, 5)} and len(runner._recorded) == 5
+    print(f"{dtype}, {batch} requests: worst error {worst:.2e} of the logit range")
+
+
 def test_schedules_with_library_products(tiny_folders_bf16, tmp_path, monkeypatch):
     """The path long prompts take (vendor library for the plain products, our kernels around them), forced
     on the tiny model by lowering the row count it starts at."""

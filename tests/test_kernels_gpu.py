@@ -725,6 +725,32 @@ def test_product_of_normalised_rows(m, n, k, act):
     assert torch.equal(other, plain)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 256, 1024), (8, 4096, 4096), (16, 512, 2048)])
+def test_product_of_normalised_rows_with_elements_far_from_the_rest(m, n, k):
+    """Rows of the kind a residual stream has, a few elements a thousand times the rest, among them the places the
+    kernel samples its shift from (the first, the middle and the last element, and more): what the kernel
+    subtracts before it rounds to bfloat16 must stay with the bulk of the row, or the rounding of `x - 1000`
+    wipes out everything else. Also rows whose common part is fifty times their spread, and both together."""
+    hip, _ = _ops(torch.bfloat16)
+    g = torch.Generator(device=DEV).manual_seed(m + n + k)
+    gamma = 1 + 0.2 * torch.randn(k, device=DEV, generator=g)
+    beta = 0.3 * torch.randn(k, device=DEV, generator=g)
+    w = (torch.randn(n, k, device=DEV, generator=g) / k ** 0.5).to(torch.bfloat16)
+    pw = hip.prepare_weight(w)
+    assert hip.fold_norm(pw, gamma, beta)
+    step = (k - 1) // 8
+    for places, common in (((0, k // 2), 0.0), ((0, k // 2, k - 1), 0.0), ((0, step, 2 * step), 0.0), ((k - 1, 5 * step), 50.0),
+                           ((0, 3 * step, 6 * step), 50.0), ((), 50.0), (tuple(range(0, k, 97)), 0.0)):
+        x = torch.randn(m, k, device=DEV, generator=g) + common
+        for p in places:
+            x[:, p] = 1000.0 * (1 if p % 2 == 0 else -1)
+        got = hip.linear(hip.layernorm_deferred(x, gamma, beta, 1e-5, torch.bfloat16), pw, None)
+        want = _float32_norm_then_product(x, gamma, beta, 1e-5, w, None, None)
+        # against the spread of the result: a row's result is small where its few far elements take most of the norm
+        scale = float(want.abs().max())
+        assert float((got.float() - want).abs().max()) <= 2e-2 * scale, (places, common)
+
+
 def test_product_of_normalised_rows_without_weight_and_bias():
     hip, _ = _ops(torch.bfloat16)
     g = torch.Generator(device=DEV).manual_seed(3)

@@ -592,7 +592,19 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
     const size_t row = (size_t)min(t * 16 + r, M - 1) * K;
     xrow[t] = NORMED ? nullptr : x + row + 8 * g;
     xfrow[t] = NORMED ? nf.x + row + 8 * g : nullptr;
-    x0[t] = NORMED ? __builtin_amdgcn_fmed3f(nf.x[row], nf.x[row + K / 2], nf.x[row + K - 1]) : 0.f;
+    if (NORMED) {
+      // the shift: the median of the medians of three times three elements spread over the row, which a few
+      // elements far from the rest (at most one of each three, or all three of one) do not move away from it
+      float med[3];
+#pragma unroll
+      for (int u = 0; u < 3; ++u) {
+        const float* p = nf.x + row + (size_t)(3 * u) * ((K - 1) / 8);
+        med[u] = __builtin_amdgcn_fmed3f(p[0], p[(K - 1) / 8], p[2 * ((K - 1) / 8)]);
+      }
+      x0[t] = __builtin_amdgcn_fmed3f(med[0], med[1], med[2]);
+    } else {
+      x0[t] = 0.f;
+    }
     s1[t] = s2[t] = 0.f;
   }
   constexpr int STRIDE = WAVES * 128;
