@@ -570,7 +570,8 @@ def test_a_step_planner_of_the_tests_rides_in_the_steps_integers(tiny_folders):
         ctx = runner._last_ctx
         assert ctx.plan["toy_even_runs"].tolist() == [0, 2] and ctx.plan["toy_totals"].tolist() == [6, 9, 4]
         assert ctx.plan_host["toy_count"] == 2
-        assert ctx.decode_runs.numel() == 0 and ctx.tile_run.tolist() == [1, 0, 2]     # the longest run first
+        # beside the plan that the model's attention mixers bring
+        assert ctx.plan["decode_runs"].numel() == 0 and ctx.plan["tile_run"].tolist() == [1, 0, 2]     # the longest run first
         for i, rid in enumerate(toks):
             assert float((logits[i] - want[rid]).abs().max()) < 1e-5
     finally:

@@ -9,6 +9,10 @@ pytestmark = pytest.mark.gpu
 
 DEV = "cuda:0"
 
+# the planner that an attention mixer brings to every step of its model (the kernels launch by its plan)
+from transformers_neuronx_amd.kernels.attention_plan import attention_plan  # noqa: E402
+ATTENTION_PLAN = {"attention": attention_plan}
+
 
 def _ops(dtype):
     from transformers_neuronx_amd.kernels.hip import HipOps
@@ -137,7 +141,7 @@ def _make_step(runs, cached, page_size, num_pages, seed, device=DEV):
     for i, t in enumerate(tables):
         tab[i, :len(t)] = t
     entries = [StepEntry(i, [0] * r, []) for i, r in enumerate(runs)]
-    return build_context(entries, list(cached), list(range(len(runs))), {"full": tab}, page_size, device)
+    return build_context(entries, list(cached), list(range(len(runs))), {"full": tab}, page_size, device, planners=ATTENTION_PLAN)
 
 
 ATTN_CASES = [
@@ -181,12 +185,12 @@ def _fill_cache_and_compare(dtype, heads, kv, hs, ps, runs, cached, window):
     scale = 1.0 / math.sqrt(hs)
     if live:
         ctx0 = build_context([StepEntry(i, [0] * cached[i], []) for i in live], [0] * len(live), live,
-                             {"full": tab[live]}, ps, DEV)
+                             {"full": tab[live]}, ps, DEV, planners=ATTENTION_PLAN)
         qkv0 = torch.randn(ctx0.num_tokens, width, device=DEV, generator=g).to(dtype)
         hip.qkv_write(qkv0, bias, heads, kv, hs, scale, ctx0, ctx0.groups["full"], kp, vp)
         ref.qkv_write(qkv0, bias, heads, kv, hs, scale, ctx0, ctx0.groups["full"], kp_r, vp_r)
     ctx = build_context([StepEntry(i, [0] * r, []) for i, r in enumerate(runs)], list(cached),
-                        list(range(len(runs))), {"full": tab}, ps, DEV)
+                        list(range(len(runs))), {"full": tab}, ps, DEV, planners=ATTENTION_PLAN)
     qkv = torch.randn(ctx.num_tokens, width, device=DEV, generator=g).to(dtype)
     q_h = hip.qkv_write(qkv, bias, heads, kv, hs, scale, ctx, ctx.groups["full"], kp, vp)
     q_r = ref.qkv_write(qkv, bias, heads, kv, hs, scale, ctx, ctx.groups["full"], kp_r, vp_r)

@@ -11,6 +11,10 @@ pytestmark = pytest.mark.gpu
 QKVO = ("q_proj", "k_proj", "v_proj", "out_proj")     # the names the tests' tensors carry
 DEV = "cuda:0"
 
+# the planner that an attention mixer brings to every step of its model (the kernels launch by its plan)
+from transformers_neuronx_amd.kernels.attention_plan import attention_plan  # noqa: E402
+ATTENTION_PLAN = {"attention": attention_plan}
+
 
 def _ops(dtype):
     from transformers_neuronx_amd.kernels.hip import HipOps
@@ -119,7 +123,7 @@ def test_attention_part_in_two_steps(dtype, heads, kv, hs, bias, window):
     outs = []
     for (a0, a1), (b0, b1), cached in (((0, n0), (0, 11), [0, 0]), ((n0, n0 + n1), (11, other), [n0, 11])):
         ctx = build_context([StepEntry("a", [0] * (a1 - a0), []), StepEntry("b", [0] * (b1 - b0), [])], cached,
-                            [0, 1], {"full": table}, ps, DEV)
+                            [0, 1], {"full": table}, ps, DEV, planners=ATTENTION_PLAN)
         hin = torch.cat([h[a0:a1], ho[b0:b1]])
         res = torch.zeros(hin.shape[0], width, device=DEV)
         outs.append(mixer.forward(hin, ctx, cache, res)[:a1 - a0])
@@ -144,14 +148,14 @@ def test_a_page_edge_shows(tmp_path):
     vp = torch.zeros(4, 1, hs, ps, device=DEV)
     table = np.array([[3, 1, 0]], dtype=np.int32)
     n = 40
-    ctx0 = build_context([StepEntry("a", [0] * n, [])], [0], [0], {"full": table}, ps, DEV)
+    ctx0 = build_context([StepEntry("a", [0] * n, [])], [0], [0], {"full": table}, ps, DEV, planners=ATTENTION_PLAN)
     qkv = torch.zeros(n, 3 * hs, device=DEV)
     for j in range(n):
         qkv[j, hs + (j % hs)] = 1.0 + j / 100.0           # key j points along axis j % 16, a little longer each
         qkv[j, 2 * hs:] = float(j)                         # value j is j
     ops.qkv_write(qkv, None, heads, 1, hs, 1.0, ctx0, ctx0.groups["full"], kp, vp)
     for target in (15, 16, 31, 32, 0, 39):
-        ctx = build_context([StepEntry("a", [0], [])], [n], [0], {"full": table}, ps, DEV)
+        ctx = build_context([StepEntry("a", [0], [])], [n], [0], {"full": table}, ps, DEV, planners=ATTENTION_PLAN)
         q = torch.zeros(1, hs, device=DEV)
         q[0, target % hs] = 200.0
         # keys target, target +- 16 share the axis; the longest (latest) wins unless masked: ask for it exactly
@@ -190,7 +194,7 @@ def test_block_arrangements(dtype, order):
         part.load(t, prefix, ops, dtype)
     cache = LayerCache(0, "full", True, {"k": torch.zeros(3, heads, ps, hs, device=DEV, dtype=dtype),
                                          "v": torch.zeros(3, heads, hs, ps, device=DEV, dtype=dtype)})
-    ctx = build_context([StepEntry("a", [0] * n, [])], [0], [0], {"full": np.array([[2, 0]], dtype=np.int32)}, ps, DEV)
+    ctx = build_context([StepEntry("a", [0] * n, [])], [0], [0], {"full": np.array([[2, 0]], dtype=np.int32)}, ps, DEV, planners=ATTENTION_PLAN)
     x = torch.randn(n, width, device=DEV, generator=g)
     out = block.forward(Stream(x, ops.cast(x, dtype)), ctx, cache)
     cfg = dict(num_attention_heads=heads, activation_function="relu", do_layer_norm_before=order == "pre_norm",

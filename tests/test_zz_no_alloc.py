@@ -13,6 +13,10 @@ pytestmark = pytest.mark.gpu
 
 DEV = "cuda:0"
 
+# the planner that an attention mixer brings to every step of its model (the kernels launch by its plan)
+from transformers_neuronx_amd.kernels.attention_plan import attention_plan  # noqa: E402
+ATTENTION_PLAN = {"attention": attention_plan}
+
 
 def _case(requests, lengths, heads, kv, hs, ps, splits, seed):
     """Decoding requests of the given lengths over pages drawn at random: what both entry points take."""
@@ -26,7 +30,7 @@ def _case(requests, lengths, heads, kv, hs, ps, splits, seed):
         for b in range(-(-n // ps)):
             tab[i, b] = perm.pop()
     ctx = build_context([StepEntry(i, [0], []) for i in range(requests)], [n - 1 for n in lengths],
-                        list(range(requests)), {"full": tab}, ps, DEV)
+                        list(range(requests)), {"full": tab}, ps, DEV, planners=ATTENTION_PLAN)
     g = torch.Generator(device=DEV).manual_seed(seed)
     kp = torch.randn(num_pages, kv, ps, hs, device=DEV, generator=g).to(torch.bfloat16)
     vp = torch.randn(num_pages, kv, hs, ps, device=DEV, generator=g).to(torch.bfloat16)
@@ -36,20 +40,20 @@ def _case(requests, lengths, heads, kv, hs, ps, splits, seed):
 
 def _both(lib, ctx, q, kp, vp, num_pages, heads, kv, hs, ps, splits, waves):
     view = ctx.groups["full"]
-    n = ctx.decode_runs.numel()
+    n = ctx.plan["decode_runs"].numel()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     p = lambda t: ctypes.c_void_p(t.data_ptr())
     out_ws = torch.full_like(q, float("nan"))
     part_o = torch.full((n * heads * splits * hs,), float("nan"), dtype=torch.float32, device=DEV)
     part_ml = torch.full((n * heads * splits * 2,), float("nan"), dtype=torch.float32, device=DEV)
     rc = lib.tnx_attention_decode(p(q), p(kp), p(vp), p(ctx.run_start), p(ctx.cached_lens), p(view.block_table),
-                                  view.width, ps, num_pages, p(ctx.decode_runs), n, p(out_ws), p(part_o), p(part_ml),
-                                  heads, kv, hs, 0, splits, waves, p(ctx.longest_decode), stream)
+                                  view.width, ps, num_pages, p(ctx.plan["decode_runs"]), n, p(out_ws), p(part_o), p(part_ml),
+                                  heads, kv, hs, 0, splits, waves, p(ctx.plan["longest_decode"]), stream)
     assert rc == 0, lib.tnx_last_error().decode()
     out_st = torch.full_like(q, float("nan"))
     rc = lib.tnx_attention_decode_static(p(q), p(kp), p(vp), p(ctx.run_start), p(ctx.cached_lens),
-                                         p(view.block_table), view.width, ps, num_pages, p(ctx.decode_runs), n,
-                                         p(out_st), heads, kv, hs, 0, splits, waves, p(ctx.longest_decode), stream)
+                                         p(view.block_table), view.width, ps, num_pages, p(ctx.plan["decode_runs"]), n,
+                                         p(out_st), heads, kv, hs, 0, splits, waves, p(ctx.plan["longest_decode"]), stream)
     assert rc == 0, lib.tnx_last_error().decode()
     torch.cuda.synchronize()
     return out_ws, out_st
@@ -84,8 +88,8 @@ def test_static_scratch_entry_point_refuses_what_does_not_fit():
     p = lambda t: ctypes.c_void_p(t.data_ptr())
     # 4 requests x 64 heads x 64 splits x 130 floats > 2^20: refused before anything is launched
     rc = lib.tnx_attention_decode_static(p(q), p(kp), p(vp), p(ctx.run_start), p(ctx.cached_lens),
-                                         p(view.block_table), view.width, ps, num_pages, p(ctx.decode_runs), 4,
-                                         p(q), heads, kv, hs, 0, 64, 4, p(ctx.longest_decode),
+                                         p(view.block_table), view.width, ps, num_pages, p(ctx.plan["decode_runs"]), 4,
+                                         p(q), heads, kv, hs, 0, 64, 4, p(ctx.plan["longest_decode"]),
                                          ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
     assert rc == 1
     assert "static array holds" in lib.tnx_last_error().decode()

@@ -13,13 +13,12 @@ import numpy as np
 import torch
 
 
-QUERY_TILE = 128    # queries of one run that one block of the prompt attention kernel takes
-
 # What a kernel wants to know about a step beyond its tokens, as int32 arrays that travel in the step's one
-# buffer of integers: a planner is `fn(run_lens, cached, page_size) -> ({name: int32 array}, {name: host value})`,
-# registered under a name; the arrays of all planners are laid out behind the step's own pieces and reach the
-# kernels as `ctx.plan[name]`, the host values as `ctx.plan_host[name]`. The attention kernels' planner below
-# is registered like any other; a part that brings a kernel of its own can bring a planner with it.
+# buffer of integers: a planner is `fn(run_lens, cached, page_size) -> ({name: int32 array}, {name: host value})`
+# under a name; the arrays of all planners are laid out behind the step's own pieces and reach the kernels as
+# `ctx.plan[name]`, the host values as `ctx.plan_host[name]`. A part brings its planners with it
+# (`Part.step_planners`, which the model collects and the runner hands to `pack_step`); a planner may also be
+# registered here for every step of the process.
 _PLANNERS: Dict[str, object] = {}
 
 
@@ -29,36 +28,6 @@ def register_step_planner(name: str, fn) -> None:
 
 def unregister_step_planner(name: str) -> None:
     _PLANNERS.pop(name, None)
-
-
-def attention_plan(run_lens: np.ndarray, cached: np.ndarray, page_size: int):
-    """What the attention kernels launch by: the runs of one token (each attends with one query), those with
-    the most keys first, and the most keys one of them reads; for every tile of QUERY_TILE queries of the longer runs its run and its first
-    query, those that see the most keys first (a kernel that takes them in this order starts its longest
-    blocks first)."""
-    single = run_lens == 1
-    decode_runs = np.nonzero(single)[0]
-    decode_runs = decode_runs[np.argsort(-cached[decode_runs], kind="stable")].astype(np.int32)
-    longest = int((cached[single] + 1).max()) if single.any() else 0
-    tiles = []
-    for i in np.nonzero(run_lens > 1)[0]:
-        for q0 in range(0, int(run_lens[i]), QUERY_TILE):
-            tiles.append((-(int(cached[i]) + min(q0 + QUERY_TILE, int(run_lens[i]))), int(i), q0))
-    tiles.sort()
-    arrays = {"decode_runs": decode_runs, "tile_run": np.array([t[1] for t in tiles], dtype=np.int32),
-              "tile_start": np.array([t[2] for t in tiles], dtype=np.int32),
-              "longest_decode": np.array([longest], dtype=np.int32)}
-    # What a recorded decode step is sized by beside its requests (a key that begins with "record:" is part
-    # of what two steps must share to share a recording): how many blocks of 256 keys the longest request
-    # fills, up to 8, and whether the requests are about as long as it (their mean at least 0.8 of it), which
-    # is when cutting every request into that many blocks pays.
-    mean = float((cached[single] + 1).mean()) if single.any() else 0.0
-    alike = bool(mean >= 0.8 * longest)
-    shape = (min(8, -(-longest // 256)) if alike else 0, alike)     # (requests that differ: one recording serves)
-    return arrays, {"longest_decode": longest, "record:decode": shape}
-
-
-register_step_planner("attention", attention_plan)
 
 
 @dataclass
@@ -93,7 +62,6 @@ class StepContext:
     groups: Dict[str, GroupView]
     plan: Dict[str, torch.Tensor] = field(default_factory=dict)   # int32 arrays of the registered step planners
     plan_host: Dict[str, object] = field(default_factory=dict)    # and what they say on the host
-    query_tile: int = QUERY_TILE         # queries of a tile of the attention plan
     # int32 [slots]: the token last chosen for the request in each slot, on the device. A token id -1 - s
     # in `token_ids` stands for `kept_tokens[s]`: a step can be started before the host has read the
     # tokens that the step before it chose.
@@ -106,27 +74,6 @@ class StepContext:
     cached_lens_host: np.ndarray = None
     slots_host: np.ndarray = None
     plans: Dict = field(default_factory=dict)    # launch plans the kernel backend keeps per step
-
-    # the attention kernels' plan under the names they use
-    @property
-    def decode_runs(self) -> torch.Tensor:
-        return self.plan["decode_runs"]
-
-    @property
-    def tile_run(self) -> torch.Tensor:
-        return self.plan["tile_run"]
-
-    @property
-    def tile_start(self) -> torch.Tensor:
-        return self.plan["tile_start"]
-
-    @property
-    def longest_decode(self) -> torch.Tensor:
-        return self.plan["longest_decode"]
-
-    @property
-    def longest_decode_host(self) -> int:
-        return self.plan_host["longest_decode"]
 
     @property
     def max_run(self) -> int:
@@ -153,19 +100,22 @@ class PackedStep:
     slots: np.ndarray
     plan_names: List[str]
     plan_host: Dict[str, object]
+    # set for a step that is replayed from a recording: what stands in for the requests' lengths where a
+    # launch is sized (`StepContext.length_bound`)
+    length_bound: Optional[int] = None
 
     def layout(self):
         """What two steps must share for one to reuse the other's device buffer and views."""
         return (tuple(self.offsets), tuple(self.sizes), self.num_tokens, self.num_requests,
-                tuple(self.group_names), tuple(sorted(self.widths.items())), self.page_size,
-                tuple(sorted((k, v) for k, v in self.plan_host.items() if k.startswith("record:"))))
+                tuple(self.group_names), tuple(sorted(self.widths.items())), self.page_size)
 
 
 _FIXED_PIECES = 7    # the step's own pieces, before the planners' and the per-group ones, see pack_step
 
 
 def pack_step(entries: List[StepEntry], cached: List[int], slots: List[int], tables: Dict[str, np.ndarray],
-              page_size: int) -> PackedStep:
+              page_size: int, planners: Optional[Dict[str, object]] = None) -> PackedStep:
+    """`planners`: those of the model's parts; the registered ones are added to them."""
     run_lens = np.array([len(e.tokens) for e in entries], dtype=np.int32)
     cached_np = np.array(cached, dtype=np.int32)
     r, t = len(entries), int(run_lens.sum())
@@ -184,7 +134,7 @@ def pack_step(entries: List[StepEntry], cached: List[int], slots: List[int], tab
     pieces = [token_ids, positions, token_request, run_start, cached_np, np.array(slots, dtype=np.int32), rows]
     assert len(pieces) == _FIXED_PIECES
     plan_names, plan_host = [], {}
-    for planner in _PLANNERS.values():
+    for planner in {**(planners or {}), **_PLANNERS}.values():
         arrays, host = planner(run_lens, cached_np, page_size)
         for name, array in arrays.items():
             if name in plan_names:
@@ -230,7 +180,7 @@ def context_from(packed: PackedStep, dev: torch.Tensor) -> StepContext:
 
 
 def build_context(entries: List[StepEntry], cached: List[int], slots: List[int],
-                  tables: Dict[str, np.ndarray], page_size: int, device) -> StepContext:
+                  tables: Dict[str, np.ndarray], page_size: int, device, planners=None) -> StepContext:
     """Pack a step's integers into one buffer, copy it once, and slice it."""
-    packed = pack_step(entries, cached, slots, tables, page_size)
+    packed = pack_step(entries, cached, slots, tables, page_size, planners)
     return context_from(packed, torch.from_numpy(packed.flat).to(device))

@@ -64,6 +64,7 @@ class DecoderModel:
         for l in self.layers:
             parts += [l.block, l.mixer, l.feed_forward, l.mixer_norm, l.feed_forward_norm]
         self.recordable = all(getattr(p, "recordable", False) for p in parts)
+        self.parts = [p for p in parts if p is not None]
 
     # ---------------------------------------------------------------- declarations
 
@@ -79,6 +80,22 @@ class DecoderModel:
     def cache_needs(self) -> Dict[int, Optional[CacheNeed]]:
         """{cache id: need} of the calls that write a cache."""
         return {cid: self.layers[layer].mixer.cache_need() for layer, cid, writes in self.schedule if writes}
+
+    def step_planners(self) -> Dict[str, object]:
+        """The step planners that the parts bring with them."""
+        out: Dict[str, object] = {}
+        for part in self.parts:
+            out.update(part.step_planners())
+        return out
+
+    def launch_shape(self, step) -> tuple:
+        """What the parts' launches of a decode step are sized by, beyond its layout (`Part.launch_shape`)."""
+        shapes = []
+        for part in self.parts:
+            shape = part.launch_shape(step)
+            if shape is not None and shape not in shapes:
+                shapes.append(shape)
+        return tuple(shapes)
 
     # ---------------------------------------------------------------- accounting (for measurements)
 

@@ -65,7 +65,7 @@ class _RecordedStep:
         self.staging = _Staging(runner.ops, packed.flat.size)
         self.static = torch.from_numpy(packed.flat).to(dev)
         self.ctx = context_from(packed, self.static)
-        self.ctx.length_bound = runner.max_positions
+        self.ctx.length_bound = packed.length_bound
         self.ctx.kept_tokens = runner.kept_tokens
         side = torch.cuda.Stream(device=dev)
         side.wait_stream(torch.cuda.current_stream(dev))
@@ -74,11 +74,17 @@ class _RecordedStep:
         torch.cuda.current_stream(dev).wait_stream(side)
         torch.cuda.synchronize(dev)
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
+        # Every recording of a runner draws on one pool of memory: recordings are replayed one after the other
+        # on one stream, so what a step needs in between may lie where another recording's lay; what a
+        # recording hands out (its logits) stays its own for as long as it lives.
+        with torch.cuda.graph(self.graph, pool=runner.graph_pool()):
             self.logits = runner.model.forward(self.ctx, runner.cache.caches)
 
     def replay(self, packed: PackedStep) -> torch.Tensor:
         self.staging.send(packed.flat, self.static)
+        # what the context says of the step on the host is this step's too (the launches are the recorded ones)
+        self.ctx.plan_host = dict(packed.plan_host)
+        self.ctx.run_lens_host, self.ctx.cached_lens_host, self.ctx.slots_host = packed.run_lens, packed.cached, packed.slots
         self.graph.replay()
         return self.logits
 
@@ -90,13 +96,35 @@ class ModelRunner:
         self.max_positions = model.spec.max_positions
         # decode-only steps are recorded once per batch size and replayed (HIP kernels only)
         self.use_graphs = use_graphs and getattr(ops, "name", "") == "hip" and model.recordable
-        self._recorded: Dict[tuple, _RecordedStep] = {}
+        self._recorded: Dict[tuple, _RecordedStep] = {}       # in the order of their last use
+        self._graph_pool = None
+        self._planners = model.step_planners()
         self.graph_replays = 0
         # The token last chosen for the request in each slot, kept on the device: a step may name a token
         # it brings as -1 - slot, and start before the host has read what the step before it chose.
         self.kept_tokens = torch.zeros(cache.max_seqs, dtype=torch.int32, device=model.device)
         self._last_ctx: Optional[StepContext] = None
         self._staging = _Staging(ops) if hasattr(ops, "pinned_ints") else None
+
+    # The most recordings kept; the one unused longest goes when another is made. A recording is one batch size
+    # and one answer of the parts to `launch_shape` (the decode attention's: how many blocks share a request's
+    # keys), and holds its own logits, `[batch, vocabulary]` in float32, beside the pool all of them share.
+    max_recordings = 48
+
+    def graph_pool(self):
+        if self._graph_pool is None:
+            self._graph_pool = torch.cuda.graph_pool_handle()
+        return self._graph_pool
+
+    def _recording(self, packed: PackedStep) -> _RecordedStep:
+        key = (packed.layout(), self.model.launch_shape(packed))
+        rec = self._recorded.pop(key, None)
+        if rec is None:
+            while len(self._recorded) >= self.max_recordings:
+                self._recorded.pop(next(iter(self._recorded)))
+            rec = _RecordedStep(self, packed)
+        self._recorded[key] = rec          # the newest at the end
+        return rec
 
     def prepare(self, entries: List[StepEntry], fixed_width: bool = False, kept_allowed: bool = False) -> PackedStep:
         """Admit new requests, get pages for the step's tokens, lay out the batch. With `fixed_width`
@@ -133,7 +161,10 @@ class ModelRunner:
                 wide = np.full((t.shape[0], full), -1, dtype=np.int32)
                 wide[:, :t.shape[1]] = t
                 tables[g] = wide
-        return pack_step(entries, cached, slots, tables, self.cache.page_size)
+        packed = pack_step(entries, cached, slots, tables, self.cache.page_size, self._planners)
+        if fixed_width:
+            packed.length_bound = self.max_positions
+        return packed
 
     @torch.no_grad()
     def step(self, entries: List[StepEntry], kept_allowed: bool = False) -> Optional[torch.Tensor]:
@@ -145,10 +176,7 @@ class ModelRunner:
                       and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries))
         packed = self.prepare(entries, fixed_width=recordable, kept_allowed=kept_allowed)
         if recordable:
-            key = packed.layout()
-            rec = self._recorded.get(key)
-            if rec is None:
-                rec = self._recorded[key] = _RecordedStep(self, packed)
+            rec = self._recording(packed)
             logits = rec.replay(packed)
             self._last_ctx = rec.ctx
             self.graph_replays += 1

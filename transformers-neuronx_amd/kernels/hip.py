@@ -12,6 +12,7 @@ import numpy as np
 import torch
 
 from . import build
+from .attention_plan import QUERY_TILE
 from .. import debug
 
 _F32, _BF16 = 0, 1
@@ -737,13 +738,13 @@ class HipOps:
         q = torch.empty(t, num_heads * head_size, dtype=self.dtype, device=qkv.device)
         # the values of runs of several tokens are written by tiles (transposed through LDS)
         by_tiles = (self.dtype == torch.bfloat16 and self.value_tiles and num_kv_write
-                    and ctx.tile_run is not None and ctx.tile_run.numel() > 0)
+                    and ctx.plan.get("tile_run") is not None and ctx.plan["tile_run"].numel() > 0)
         self._call("attention", "tnx_qkv_write", _ptr(qkv), _code(self.dtype), _ptr(bias), float(scale),
                    _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width, view.page_size,
                    num_pages, _ptr(q), _ptr(k_pages) if num_kv_write else None,
                    _ptr(v_pages) if num_kv_write else None, t, num_heads, num_kv_write, head_size,
-                   _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(ctx.tile_run), _ptr(ctx.tile_start),
-                   ctx.tile_run.numel() if by_tiles else 0, ctx.query_tile, _stream())
+                   _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(ctx.plan["tile_run"]), _ptr(ctx.plan["tile_start"]),
+                   ctx.plan["tile_run"].numel() if by_tiles else 0, QUERY_TILE, _stream())
         return q
 
     def attention(self, q, num_heads, num_kv_heads, head_size, ctx, view, k_pages, v_pages, window=None):
@@ -756,21 +757,21 @@ class HipOps:
         out = torch.empty_like(q)
         window = int(window or 0)
         fast = (self.dtype == torch.bfloat16 and not self.force_plain_attention
-                and (ctx.decode_runs.numel() == 0
+                and (ctx.plan["decode_runs"].numel() == 0
                      or view.page_size & (view.page_size - 1) == 0))
         if not fast:
             self._call("attention", "tnx_attention_any", _ptr(q), _code(self.dtype), _ptr(k_pages), _ptr(v_pages),
                        _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width,
                        view.page_size, num_pages, _ptr(out), t, num_heads, num_kv_heads, head_size, window, _stream())
             return out
-        if ctx.tile_run.numel():
+        if ctx.plan["tile_run"].numel():
             self._call("attention", "tnx_attention_prefill", _ptr(q), _ptr(k_pages), _ptr(v_pages),
                        _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(view.block_table), view.width,
-                       view.page_size, num_pages, _ptr(ctx.tile_run), _ptr(ctx.tile_start), ctx.tile_run.numel(),
+                       view.page_size, num_pages, _ptr(ctx.plan["tile_run"]), _ptr(ctx.plan["tile_start"]), ctx.plan["tile_run"].numel(),
                        _ptr(out), num_heads, num_kv_heads, head_size, window,
-                       int(self.prefill_direct) or self._prefill_sets(ctx, num_heads, window), ctx.query_tile,
+                       int(self.prefill_direct) or self._prefill_sets(ctx, num_heads, window), QUERY_TILE,
                        _stream())
-        n_dec = ctx.decode_runs.numel()
+        n_dec = ctx.plan["decode_runs"].numel()
         if n_dec:
             splits, waves = self._decode_splits(ctx, n_dec * num_heads, window, head_size)
             part_o = part_ml = None
@@ -779,9 +780,9 @@ class HipOps:
                 part_ml = torch.empty(n_dec * num_heads * splits * 2, dtype=torch.float32, device=q.device)
             self._call("attention", "tnx_attention_decode", _ptr(q), _ptr(k_pages), _ptr(v_pages),
                        _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(view.block_table), view.width,
-                       view.page_size, num_pages, _ptr(ctx.decode_runs), n_dec, _ptr(out), _ptr(part_o),
+                       view.page_size, num_pages, _ptr(ctx.plan["decode_runs"]), n_dec, _ptr(out), _ptr(part_o),
                        _ptr(part_ml), num_heads, num_kv_heads, head_size, window, splits, waves,
-                       _ptr(ctx.longest_decode),
+                       _ptr(ctx.plan["longest_decode"]),
                        _stream())
         return out
 
@@ -802,8 +803,8 @@ class HipOps:
             lens, cached = ctx.run_lens_host, ctx.cached_lens_host
             steps = []
             for i in np.nonzero(lens > 1)[0]:
-                for q0 in range(0, int(lens[i]), ctx.query_tile):
-                    last = int(cached[i]) + min(q0 + ctx.query_tile, int(lens[i]))      # keys the tile's last query sees
+                for q0 in range(0, int(lens[i]), QUERY_TILE):
+                    last = int(cached[i]) + min(q0 + QUERY_TILE, int(lens[i]))      # keys the tile's last query sees
                     first = max(0, int(cached[i]) + q0 - window + 1) // 64 if window > 0 else 0
                     steps.append(-(-last // 64) - first)
             steps = np.array(steps)
@@ -841,8 +842,11 @@ class HipOps:
         gives every compute unit a block: most blocks of a short request would be empty (64 requests of 16
         to 1,280 tokens: 6,430 tokens a second whole, 4,760 in eight blocks each). A recorded step is sized
         by the same two facts, which are part of what it is recorded under."""
-        longest = ctx.length_bound if ctx.length_bound is not None else ctx.longest_decode_host
-        fills, alike = ctx.plan_host.get("record:decode", (0, False))
+        longest = ctx.length_bound if ctx.length_bound is not None else ctx.plan_host["longest_decode"]
+        fills, alike = ctx.plan_host.get("decode_shape", (0, False))
+        return self._splits_for(longest, fills, alike, pairs, window, head_size)
+
+    def _splits_for(self, longest: int, fills: int, alike: bool, pairs: int, window: int, head_size: int):
         if not alike:
             fills = min(8, -(-longest // 256))
         if window:
@@ -858,6 +862,19 @@ class HipOps:
         if pairs > units and -(-pairs // units) * units <= 1.05 * pairs:
             alike = False         # whole requests already come out even over the compute units
         return (max(fill_the_chip, fills) if alike else fill_the_chip), waves
+
+    def attention_launch_shape(self, step, num_heads: int, window, head_size: int):
+        """What the decode attention's launch in a recorded step is sized by beyond the number of requests: the
+        blocks that share a request's keys (and their waves), for a `PackedStep` about to be replayed. A
+        recorded step is sized for the longest request the model allows; how requests about as long as one
+        another are cut depends on how long they are now, so a batch that grows is recorded again only when
+        that changes the launch (8 requests of 32 heads: never; 9: at every 256 keys up to eight blocks)."""
+        n_dec = int((step.run_lens == 1).sum())
+        if n_dec == 0 or self.dtype != torch.bfloat16:
+            return None
+        fills, alike = step.plan_host.get("decode_shape", (0, False))
+        return ("decode", num_heads, head_size) + self._splits_for(step.length_bound, fills, alike, n_dec * num_heads,
+                                                                   int(window or 0), head_size)
 
     # ---------------------------------------------------------------- output end
 

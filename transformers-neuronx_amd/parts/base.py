@@ -7,7 +7,7 @@ step's context. Mixers also declare what they keep between steps
 from a `ModelSpec`.
 """
 from dataclasses import dataclass
-from typing import Callable, Dict, List, Optional, Tuple
+from typing import Callable, Dict, Hashable, List, Optional, Tuple
 
 from .spec import ParamDecl, PartSpec
 
@@ -60,6 +60,17 @@ class Part:
     def load(self, tensors: Dict[str, "object"], prefix: str, ops, dtype) -> None:
         self.ops = ops
         self.dtype = dtype
+
+    def step_planners(self) -> Dict[str, Callable]:
+        """{name: planner} of what this part's kernels want laid out with every step's integers
+        (`engine.batch`): `fn(run_lens, cached, page_size) -> ({name: int32 array}, {name: host value})`."""
+        return {}
+
+    def launch_shape(self, step) -> Optional[Hashable]:
+        """What this part's launches in a decode step are sized by beyond the number of requests, for a
+        `PackedStep` about to be replayed from a recording: two steps share a recording only where every
+        part gives the same answer. None: nothing."""
+        return None
 
     def flops_per_token(self, keys: float = 0.0) -> float:
         """Multiply-adds times two that one token costs in this part, for a measurement's accounting; `keys`

@@ -86,6 +86,14 @@ class Attention(Mixer):
     def first_weight(self):
         return self.w_qkv
 
+    def step_planners(self):
+        from ..kernels.attention_plan import attention_plan
+        return {"attention": attention_plan}
+
+    def launch_shape(self, step):
+        shape = getattr(self.ops, "attention_launch_shape", None)
+        return shape(step, self.num_heads, self.window, self.head_size) if shape is not None else None
+
     def flops_per_token(self, keys: float = 0.0) -> float:
         seen = min(keys, self.window) if self.window else keys
         return super().flops_per_token(keys) + 4.0 * self.num_heads * self.head_size * seen   # q k^T and p v
