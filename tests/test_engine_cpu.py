@@ -438,7 +438,7 @@ def test_toy_routed_parts_on_the_host():
     run_toy_routed_model("reference", torch.float32, "cpu", 2e-5)
 
 
-def run_toy_rotating_model(ops_kind, dtype, device, tol):
+def run_toy_rotating_model(ops_kind, dtype, device, tol, in_the_projection=False):
     """Attention whose queries and keys are turned by an encoding defined in the tests, a norm that brings a
     kernel of its own, tensor names of its own: built from the registries and stepped under every way of
     cutting, without a change to the framework."""
@@ -447,20 +447,25 @@ def run_toy_rotating_model(ops_kind, dtype, device, tol):
     from transformers_neuronx_amd.engine import DecoderModel, ModelRunner
     from transformers_neuronx_amd.kernels import make_ops
     from transformers_neuronx_amd.weights import TensorDict, random_tensors
-    spec = toy_parts.toy_spec_rotating()
+    # `in_the_projection`: the encoding hands over its pairwise tables, the projection's launch turns queries and
+    # keys, every part can be replayed from a recording (the layer with Python loops is left out of that model)
+    spec = toy_parts.toy_spec_rotating(tables=in_the_projection, latent_layer=not in_the_projection)
     model = DecoderModel(spec)
     tensors = random_tensors(model.param_decls(), spec.init_std, 6, torch.float32)
     assert "blocks.2.attn.wk.weight" in tensors and tensors["blocks.0.attn.wk.weight"].shape == (32, 96)
-    assert tensors["blocks.1.attn.down.weight"].shape == (24, 96)
     ops = make_ops(ops_kind, dtype, device)
     model.load(TensorDict(tensors), ops, dtype, device)
+    assert model.recordable == in_the_projection
     runner = ModelRunner(model, CacheManager(model.cache_needs(), 16, 12, 4, dtype, device), ops, use_graphs=True)
-    # the latent mixer's pages are of its own shape, in the same group (same page numbers) as the attention's
-    shapes = {cid: {k: tuple(v.shape) for k, v in c.pages.items()} for cid, c in runner.cache.caches.items()}
-    assert shapes[1] == {"z": (12, 16, 24)} and shapes[0] == {"k": (12, 1, 16, 32), "v": (12, 1, 32, 16)}
+    if not in_the_projection:
+        assert tensors["blocks.1.attn.down.weight"].shape == (24, 96)
+        # the latent mixer's pages are of its own shape, in the same group (same page numbers) as the attention's
+        shapes = {cid: {k: tuple(v.shape) for k, v in c.pages.items()} for cid, c in runner.cache.caches.items()}
+        assert shapes[1] == {"z": (12, 16, 24)} and shapes[0] == {"k": (12, 1, 16, 32), "v": (12, 1, 32, 16)}
     assert list(runner.cache.groups) == ["full"]
     requests = _requests(157, [70, 33, 100], 10)
-    expected = {rid: toy_parts.toy_rotating_plain_logits(tensors, toks) for rid, toks in requests.items()}
+    expected = {rid: toy_parts.toy_rotating_plain_logits(tensors, toks, latent_layer=not in_the_projection)
+                for rid, toks in requests.items()}
     for steps, place in (schedules.whole(requests), schedules.portions(requests),
                          schedules.mixed(requests, max_tokens=192, page=16, seed=2, tail=8, max_live=3)):
         for rec in steps:
@@ -474,10 +479,12 @@ def run_toy_rotating_model(ops_kind, dtype, device, tol):
                 runner.finish(rid)
             runner.cache.check()
         assert not runner.cache.requests
+    return runner
 
 
 def test_toy_rotating_parts_on_the_host():
     run_toy_rotating_model("reference", torch.float32, "cpu", 2e-5)
+    run_toy_rotating_model("reference", torch.float32, "cpu", 2e-5, in_the_projection=True)
 
 
 def test_toy_rotation_counts_distances_only():

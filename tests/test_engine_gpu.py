@@ -212,6 +212,10 @@ def test_toy_rotating_parts_on_the_gpu(dtype):
     from transformers_neuronx_amd.kernels import hip
     run_toy_rotating_model("hip", dtype, DEV, 2e-5 if dtype == torch.float32 else 3e-2)
     assert "toy_norm" in hip.loaded_libraries()
+    # the same encoding as pairwise tables: turned inside the projection's launch (the fused product of few
+    # rows, the scatter after a library product, the float32 path), and decode steps replayed from recordings
+    runner = run_toy_rotating_model("hip", dtype, DEV, 2e-5 if dtype == torch.float32 else 3e-2, in_the_projection=True)
+    assert runner.graph_replays > 10
 
 
 def test_benchmark_report_and_kernel_times(tiny_folders_bf16, capsys):

@@ -109,6 +109,69 @@ def test_fused_projection_of_small_integers_is_exact(m):
     assert int((~torch.isnan(kp.float())).sum()) == m * kv * hs            # and nothing else was written
 
 
+@pytest.mark.parametrize("m,own", [(1, True), (8, True), (16, True), (30, True), (64, True), (100, True), (200, True), (40, False),
+                                   (300, False)])
+@pytest.mark.parametrize("normed", [False, True])
+def test_projection_that_turns_pairs_is_exact(m, own, normed):
+    """Pairwise tables handed to the projection: element d of every query and key head becomes
+    a[p, d] x[d] + b[p, d] x[d ^ 1] at the token's position p, bias added, before the query's scale; values stay.
+    Integers throughout, on every way the projection can go: the fused product of few rows (with the tile-ordered
+    weight and without), our product of many rows, the library's product with the scatter after it."""
+    hip, ref = _ops(torch.bfloat16)
+    if own:
+        hip.library_rows = 0
+    heads, kv, hs, ps, k = 3, 1, 32, 16, 256
+    g = torch.Generator(device=DEV).manual_seed(m)
+    cached = [int(c) for c in torch.randint(0, 90, (m,), generator=torch.Generator().manual_seed(m))]
+    num_pages = sum(-(-(c + 1) // ps) for c in cached) + 2
+    ctx = _make_step([1] * m, cached, ps, num_pages, seed=m)
+    view = ctx.groups["full"]
+    n = (heads + 2 * kv) * hs
+    x, w, bias = _ints(g, m, k, low=-2, high=2), _ints(g, n, k, low=-2, high=2).to(torch.bfloat16), _ints(g, n, low=-8, high=8)
+    a, b = _ints(g, 100, hs, low=-2, high=2), _ints(g, 100, hs, low=-2, high=2)
+    full = x.double() @ w.double().t() + bias.double()
+    pos = torch.tensor(cached, device=DEV)
+    turned = (heads + kv) * hs
+    part = full[:, :turned].reshape(m, -1, hs)
+    beside = part.reshape(m, -1, hs // 2, 2).flip(-1).reshape(m, -1, hs)
+    part = (a[pos].double()[:, None] * part + b[pos].double()[:, None] * beside).reshape(m, turned)
+    want_q = (part[:, :heads * hs] * 0.25).float().to(torch.bfloat16).float()
+    want_k = part[:, heads * hs:].float().to(torch.bfloat16).float().view(m, kv, hs)
+    want_v = full[:, turned:].float().to(torch.bfloat16).float().view(m, kv, hs)
+    for weight in (hip.prepare_weight(w), w):
+        kp = torch.full((num_pages, kv, ps, hs), float("nan"), device=DEV, dtype=torch.bfloat16)
+        vp = torch.full((num_pages, kv, hs, ps), float("nan"), device=DEV, dtype=torch.bfloat16)
+        h = x.to(torch.bfloat16)
+        if normed:
+            # a LayerNorm that changes nothing that matters here cannot be exact: the folded form is compared below
+            break
+        q = hip.qkv_project(h, weight, bias, heads, kv, hs, 0.25, ctx, view, kp, vp, turn=(a, b))
+        torch.testing.assert_close(q.float(), want_q, **EXACT)
+        table = view.block_table.cpu()
+        for i, c in enumerate(cached):
+            page, at = int(table[i, c // ps]), c % ps
+            torch.testing.assert_close(kp[page, :, at, :].float(), want_k[i], **EXACT)
+            torch.testing.assert_close(vp[page, :, :, at].float(), want_v[i], **EXACT)
+    if normed and m <= 32:
+        # behind a folded LayerNorm (not exact: against the torch rendition, which applies the same tables)
+        gamma, beta = 1 + 0.2 * torch.randn(k, device=DEV, generator=g), 0.3 * torch.randn(k, device=DEV, generator=g)
+        xs = torch.randn(m, k, device=DEV, generator=g) * 2 + 3
+        wr = (torch.randn(n, k, device=DEV, generator=g) / 16).to(torch.bfloat16)
+        pw = hip.prepare_weight(wr)
+        assert hip.fold_norm(pw, gamma, beta)
+        kp = torch.zeros(num_pages, kv, ps, hs, device=DEV, dtype=torch.bfloat16)
+        vp = torch.zeros(num_pages, kv, hs, ps, device=DEV, dtype=torch.bfloat16)
+        kp_r, vp_r = kp.clone(), vp.clone()
+        q = hip.qkv_project(hip.layernorm_deferred(xs, gamma, beta, 1e-5, torch.bfloat16), pw, bias, heads, kv, hs, 0.25,
+                            ctx, view, kp, vp, turn=(a, b))
+        h_r = ref.layernorm(xs, gamma, beta, 1e-5, torch.bfloat16, False, True)[1]
+        q_r = ref.qkv_project(h_r, wr, bias, heads, kv, hs, 0.25, ctx, view, kp_r, vp_r, turn=(a, b))
+        scale = float(q_r.float().abs().max())
+        assert float((q.float() - q_r.float()).abs().max()) <= 2e-2 * scale
+        assert float((kp.float() - kp_r.float()).abs().max()) <= 2e-2 * float(kp_r.float().abs().max())
+        assert torch.equal(kp == 0, kp_r == 0)
+
+
 # ---------------------------------------------------------------- attention
 
 def _coded_case(heads, kv, hs, ps, runs, cached, window, seed):

@@ -260,8 +260,26 @@ class ToyRotation(PositionEncoding):
     """Turns every pair (x[2i], x[2i+1]) of each query and key head by the angle position * base^(-2i/head_size),
     so that a score depends on the distance of query and key only. Torch operations on the device: a toy."""
 
-    def __init__(self, base: float):
-        self.base = base
+    def __init__(self, base: float, tables: bool = False, positions: int = 0):
+        """`tables`: hand the attention mixer the pairwise form (`pair_tables`) for `positions` positions, which
+        the projection applies in its own launch; otherwise `on_query_key` turns the projections with torch."""
+        self.base, self.tables, self.positions = base, tables, positions
+        self.recordable = bool(tables)
+
+    def load(self, tensors, prefix, ops, dtype):
+        super().load(tensors, prefix, ops, dtype)
+        self.device = next(iter(tensors.values())).device if tensors else "cpu"
+
+    def pair_tables(self, head_size):
+        if not self.tables:
+            return None
+        freq = self.base ** (-torch.arange(head_size // 2, dtype=torch.float32) * 2 / head_size)
+        angle = torch.arange(self.positions, dtype=torch.float32)[:, None] * freq[None, :]
+        cos, sin = torch.cos(angle), torch.sin(angle)
+        # (x0, x1) -> (x0 cos - x1 sin, x1 cos + x0 sin): a = cos for both, b = -sin for the first, +sin for the second
+        a = torch.stack([cos, cos], dim=-1).reshape(self.positions, head_size)
+        b = torch.stack([-sin, sin], dim=-1).reshape(self.positions, head_size)
+        return a.contiguous().to(self.device), b.contiguous().to(self.device)
 
     def on_query_key(self, qkv, ctx, num_heads, num_kv_heads, head_size):
         t = qkv.shape[0]
@@ -347,17 +365,19 @@ class ToyLatentMixer(Mixer):
         return self.ops.linear(means.to(self.dtype), self.up, None, residual=residual, out_f32=True)
 
 
-def toy_spec_rotating(width=96, heads=3, kv_heads=1, inner=72, vocab=157, positions=150, eps=1e-3, base=100.0):
+def toy_spec_rotating(width=96, heads=3, kv_heads=1, inner=72, vocab=157, positions=150, eps=1e-3, base=100.0,
+                      tables=False, latent_layer=True):
     """Attention whose queries and keys are turned by their positions (no encoding at the input), grouped
     heads, between two such layers one whose mixer keeps a paged cache of another shape; a scale-only norm
     with its own kernel, names of its own for every tensor."""
     hs = width // heads
     norm = PartSpec("toy_scale_norm", dict(width=width, eps=eps))
     mixer = PartSpec("attention", dict(width=width, num_heads=heads, head_size=hs, num_kv_heads=kv_heads, bias=False,
-                                       names=("wq", "wk", "wv", "wo"), rotation=PartSpec("toy_rotation", dict(base=base))))
+                                       names=("wq", "wk", "wv", "wo"),
+                                       rotation=PartSpec("toy_rotation", dict(base=base, tables=tables, positions=positions))))
     ffn = PartSpec("dense", dict(width=width, inner=inner, activation="gelu", bias=False, up_name="up", down_name="down"))
     latent = PartSpec("toy_latent", dict(width=width, latent=24))
-    layers = tuple(LayerSpec(prefix=f"blocks.{i}.", block="pre_norm", mixer=latent if i == 1 else mixer, feed_forward=ffn,
+    layers = tuple(LayerSpec(prefix=f"blocks.{i}.", block="pre_norm", mixer=latent if i == 1 and latent_layer else mixer, feed_forward=ffn,
                              mixer_norm=norm, feed_forward_norm=norm, mixer_name="attn.", feed_forward_name="mlp.",
                              mixer_norm_name="attn_norm", feed_forward_norm_name="mlp_norm") for i in range(3))
     embedding = PartSpec("token_table", dict(vocab=vocab, embed_width=width, width=width, position=PartSpec("none", {}),
@@ -369,7 +389,8 @@ def toy_spec_rotating(width=96, heads=3, kv_heads=1, inner=72, vocab=157, positi
                      schedule=ModelSpec.sequential(3), head=head, init_std=0.1)
 
 
-def toy_rotating_plain_logits(w, tokens, width=96, heads=3, kv_heads=1, eps=1e-3, base=100.0, first_position=0):
+def toy_rotating_plain_logits(w, tokens, width=96, heads=3, kv_heads=1, eps=1e-3, base=100.0, first_position=0,
+                              latent_layer=True):
     """The rotating toy model on one whole sequence; `first_position` shifts every position (the logits must
     not change: only distances count)."""
     w = {k: v.float() for k, v in w.items()}
@@ -390,7 +411,7 @@ def toy_rotating_plain_logits(w, tokens, width=96, heads=3, kv_heads=1, eps=1e-3
     for i in range(3):
         p = f"blocks.{i}."
         h = norm(x, p + "attn_norm")
-        if i == 1:                                  # the layer that keeps a small vector per token and averages them
+        if i == 1 and latent_layer:                 # the layer that keeps a small vector per token and averages them
             z = plain_opt.linear(h, w[p + "attn.down.weight"])
             means = torch.cumsum(z, dim=0) / torch.arange(1, n + 1, dtype=torch.float32)[:, None]
             x = x + plain_opt.linear(means, w[p + "attn.up.weight"])

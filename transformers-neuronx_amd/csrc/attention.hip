@@ -20,7 +20,8 @@ qkv_write_kernel(const T* __restrict__ qkv, const float* __restrict__ bias, floa
                  const int* __restrict__ positions, const int* __restrict__ token_request,
                  const int* __restrict__ table, int table_width, int page_size, int num_pages, T* __restrict__ q_out,
                  T* __restrict__ k_pages, T* __restrict__ v_pages, int num_heads, int num_kv, int head_size,
-                 const int* __restrict__ run_start, int values_of_single_tokens_only) {
+                 const int* __restrict__ run_start, int values_of_single_tokens_only,
+                 const float* __restrict__ turn_a, const float* __restrict__ turn_b, int turn_rows) {
   const int t = blockIdx.x;
   const int nq = num_heads * head_size, nk = num_kv * head_size;
   const int total = nq + 2 * nk;
@@ -33,6 +34,16 @@ qkv_write_kernel(const T* __restrict__ qkv, const float* __restrict__ bias, floa
   if (bias) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) v[j] += bias[i0 + j];
+  }
+  if (turn_a && i0 < nq + nk) {
+    // a position encoding that turns queries and keys pair by pair: x[d] becomes a[p][d] x[d] + b[p][d] x[d ^ 1]
+    // (the eight elements of a thread lie in one head: head sizes are multiples of 8)
+    const size_t at = (size_t)min(max(positions[t], 0), turn_rows - 1) * head_size + i0 % head_size;
+    float w[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) w[j] = turn_a[at + j] * v[j] + turn_b[at + j] * v[j ^ 1];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = w[j];
   }
   if (i0 < nq) {
     T* dst = q_out + (size_t)t * nq + i0;
@@ -126,8 +137,10 @@ extern "C" int tnx_qkv_write(const void* qkv, int dtype, const float* bias, floa
                              int num_pages, void* q_out, void* k_pages, void* v_pages, int tokens, int num_heads,
                              int num_kv, int head_size, const int* run_start, const int* cached_lens,
                              const int* tile_run, const int* tile_q0, int num_tiles, int tile_tokens,
-                             hipStream_t stream) {
+                             const float* turn_a, const float* turn_b, int turn_rows, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && num_heads > 0 && num_kv >= 0 && head_size > 0, "qkv_write: bad sizes");
+  TNX_REQUIRE((turn_a == nullptr) == (turn_b == nullptr) && (!turn_a || turn_rows > 0),
+              "qkv_write: the pair-turning tables come both or not at all, with their number of rows");
   TNX_REQUIRE(page_size > 0 && table_width > 0, "qkv_write: bad page table");
   if (tokens == 0) return 0;
   TNX_REQUIRE(head_size % 8 == 0, "qkv_write: head size %d is not a multiple of 8", head_size);
@@ -145,12 +158,13 @@ extern "C" int tnx_qkv_write(const void* qkv, int dtype, const float* bias, floa
     qkv_write_kernel<float><<<grid, 256, 0, stream>>>((const float*)qkv, bias, scale, positions, token_request,
                                                         table, table_width, page_size, num_pages, (float*)q_out,
                                                         (float*)k_pages, (float*)v_pages, num_heads, num_kv, head_size,
-                                                        run_start, 0);
+                                                        run_start, 0, turn_a, turn_b, turn_rows);
   else
     qkv_write_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)qkv, bias, scale, positions, token_request,
                                                          table, table_width, page_size, num_pages, (bf16_t*)q_out,
                                                          (bf16_t*)k_pages, (bf16_t*)v_pages, num_heads, num_kv,
-                                                         head_size, run_start, by_tiles ? 1 : 0);
+                                                         head_size, run_start, by_tiles ? 1 : 0, turn_a, turn_b,
+                                                         turn_rows);
   TNX_CHECK_LAUNCH("qkv_write");
   if (by_tiles) {
     value_tiles_kernel<<<dim3(num_tiles, num_kv), 256, 0, stream>>>(

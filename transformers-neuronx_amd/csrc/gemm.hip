@@ -23,6 +23,10 @@ __device__ __forceinline__ void epilogue_store(float v, int m, int n, int N, con
 // Where the fused query/key/value projection puts its output: queries (scaled) into a dense matrix, the
 // keys and values of token m into the cache page `token_page[m]` at place `token_off[m]`
 // (keys [pages, kv_heads, page_size, head_size], values [pages, kv_heads, head_size, page_size]).
+// `turn_a`, `turn_b` (both or neither): a position encoding that turns queries and keys pair by pair, as
+// tables [turn_rows, head_size] of float32. Element d of a query or key head of the token at position p
+// becomes a[p][d] x[d] + b[p][d] x[d ^ 1], bias added, before the query's scale: any map of each pair
+// (2i, 2i + 1) of a head that depends on the position alone (a rotation: a = cos, b = -sin and +sin).
 struct QkvScatter {
   const int* token_page;
   const int* token_off;
@@ -31,10 +35,19 @@ struct QkvScatter {
   bf16_t* v_pages;
   float scale;
   int nq, nk, head_size, num_kv, page_size, num_pages;
+  const float* turn_a;
+  const float* turn_b;
+  const int* positions;
+  int turn_rows;
 };
 
-__device__ __forceinline__ void qkv_store(float v, int m, int n, const float* bias, const QkvScatter& sc) {
-  if (bias) v += bias[n];
+// `v`: element n of token m's projections with its bias; `beside`: element n ^ 1 with its bias (read only
+// where the scatter turns pairs)
+__device__ __forceinline__ void qkv_store(float v, float beside, int m, int n, const QkvScatter& sc) {
+  if (sc.turn_a && n < sc.nq + sc.nk) {
+    const size_t at = (size_t)min(max(sc.positions[m], 0), sc.turn_rows - 1) * sc.head_size + n % sc.head_size;
+    v = sc.turn_a[at] * v + sc.turn_b[at] * beside;
+  }
   if (n < sc.nq) {
     sc.q_out[(size_t)m * sc.nq + n] = (bf16_t)(v * sc.scale);
     return;
@@ -277,10 +290,13 @@ gemm_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, con
       for (int e = 0; e < 16; ++e) {
         const int m = m0 + wm + i * 32 + 8 * (e >> 2) + 4 * lhalf + (e & 3);
         if (m < M) {
-          if (QKV)
-            qkv_store(acc[i][j][e], m, n, bias, sc);
-          else
+          if (QKV) {
+            // (the element beside this one is the neighbouring lane's: N is even, so both are there or neither)
+            const float v = acc[i][j][e] + (bias ? bias[n] : 0.f);
+            qkv_store(v, lane_dpp<TNX_DPP_XOR1>(v), m, n, sc);
+          } else {
             epilogue_store(acc[i][j][e], m, n, N, bias, residual, out, out_dtype, act);
+          }
         }
       }
     }
@@ -734,6 +750,13 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
 #pragma unroll
     for (int wv = 0; wv < WAVES; ++wv) v += red[wv][t][j][i][l];
     const int n = n0 + 16 * j + 4 * (l >> 4) + i, m = t * 16 + (l & 15);
+    // where the scatter turns pairs, the element beside this one (column n ^ 1: the same lane's, i ^ 1) as well
+    const bool pairs = QKV && sc.turn_a != nullptr;
+    float beside = 0.f;
+    if (pairs) {
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv) beside += red[wv][t][j][i ^ 1][l];
+    }
     if (NORMED && n < N) {
       float a1 = 0.f, a2 = 0.f;
 #pragma unroll
@@ -743,13 +766,20 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
       }
       const float mean = a1 / (float)K;                       // of x - x0
       const float var = fmaxf(a2 / (float)K - mean * mean, 0.f);
-      v = rsqrtf(var + nf.eps) * (v - mean * nf.c[n]) + nf.d[n];
+      const float rstd = rsqrtf(var + nf.eps);
+      v = rstd * (v - mean * nf.c[n]) + nf.d[n];
+      if (pairs) beside = rstd * (beside - mean * nf.c[n ^ 1]) + nf.d[n ^ 1];
     }
     if (n < N && m < M) {
-      if (QKV)
-        qkv_store(v, m, n, bias, sc);
-      else
+      if (QKV) {
+        if (bias) {
+          v += bias[n];
+          if (pairs) beside += bias[n ^ 1];
+        }
+        qkv_store(v, beside, m, n, sc);
+      } else {
         epilogue_store(v, m, n, N, bias, residual, out, out_dtype, act);
+      }
     }
   }
 }
@@ -907,11 +937,24 @@ extern "C" int tnx_gemm_bf16(const void* x, const void* w, const void* w_tiles, 
 
 // The fused projection of queries, keys and values: `x w^T + bias` with w = [Wq; Wk; Wv] stacked by rows,
 // queries scaled and written densely, keys and values written straight into their cache pages.
+// What both forms of the fused projection check and fill in of the pair-turning tables.
+static int qkv_turn(QkvScatter& sc, const float* turn_a, const float* turn_b, const int* positions, int turn_rows) {
+  TNX_REQUIRE((turn_a == nullptr) == (turn_b == nullptr), "gemm_bf16_qkv: the pair-turning tables come both or not at all");
+  TNX_REQUIRE(!turn_a || (positions && turn_rows > 0 && sc.head_size % 2 == 0),
+              "gemm_bf16_qkv: pair-turning tables need the tokens' positions, rows, and an even head size");
+  sc.turn_a = turn_a;
+  sc.turn_b = turn_b;
+  sc.positions = positions;
+  sc.turn_rows = turn_rows;
+  return 0;
+}
+
 extern "C" int tnx_gemm_bf16_qkv(const void* x, const void* w, const void* w_tiles, const float* bias, int M, int K,
                                  const int* token_page,
                                  const int* token_off, void* q_out, void* k_pages, void* v_pages, float scale,
                                  int num_heads, int num_kv, int head_size, int page_size, int num_pages,
-                                 int force_tiled, hipStream_t stream) {
+                                 int force_tiled, const float* turn_a, const float* turn_b, const int* positions,
+                                 int turn_rows, hipStream_t stream) {
   TNX_REQUIRE(num_heads > 0 && num_kv >= 0 && head_size > 0 && page_size > 0, "gemm_bf16_qkv: bad sizes");
   QkvScatter sc;
   sc.token_page = token_page;
@@ -926,6 +969,7 @@ extern "C" int tnx_gemm_bf16_qkv(const void* x, const void* w, const void* w_til
   sc.num_kv = num_kv;
   sc.page_size = page_size;
   sc.num_pages = num_pages;
+  if (int rc = qkv_turn(sc, turn_a, turn_b, positions, turn_rows)) return rc;
   const int N = sc.nq + 2 * sc.nk;
   return gemm_bf16_dispatch(x, w, w_tiles, bias, nullptr, nullptr, TNX_BF16, TNX_ACT_NONE, M, N, K, force_tiled, &sc,
                             stream);
@@ -945,7 +989,9 @@ extern "C" int tnx_gemm_bf16_qkv_normed(const float* x, const void* w_folded, co
                                         const float* fold_d, float eps, const float* bias, int M, int K,
                                         const int* token_page, const int* token_off, void* q_out, void* k_pages,
                                         void* v_pages, float scale, int num_heads, int num_kv, int head_size,
-                                        int page_size, int num_pages, int force_tiled, hipStream_t stream) {
+                                        int page_size, int num_pages, int force_tiled, const float* turn_a,
+                                        const float* turn_b, const int* positions, int turn_rows,
+                                        hipStream_t stream) {
   TNX_REQUIRE(num_heads > 0 && num_kv >= 0 && head_size > 0 && page_size > 0, "gemm_bf16_qkv: bad sizes");
   QkvScatter sc;
   sc.token_page = token_page;
@@ -960,6 +1006,7 @@ extern "C" int tnx_gemm_bf16_qkv_normed(const float* x, const void* w_folded, co
   sc.num_kv = num_kv;
   sc.page_size = page_size;
   sc.num_pages = num_pages;
+  if (int rc = qkv_turn(sc, turn_a, turn_b, positions, turn_rows)) return rc;
   const int N = sc.nq + 2 * sc.nk;
   const NormFold nf{x, fold_c, fold_d, eps};
   return gemm_bf16_dispatch(nullptr, nullptr, w_folded, bias, nullptr, nullptr, TNX_BF16, TNX_ACT_NONE, M, N, K,

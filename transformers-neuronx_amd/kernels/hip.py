@@ -40,7 +40,7 @@ _SIGNATURES = {
                           _c_int, _c_int, _c_int, _c_void_p],
         "tnx_gemm_bf16_qkv": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
                               _c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int,
-                              _c_int, _c_void_p],
+                              _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p],
         "tnx_gemm_skinny_tiles_per_block": [_c_int, _c_int],
         "tnx_gemm_bf16_mid": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                               _c_int, _c_void_p, ctypes.c_size_t, _c_int, _c_int, _c_void_p],
@@ -50,12 +50,12 @@ _SIGNATURES = {
                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_gemm_bf16_qkv_normed": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int,
                                      _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int,
-                                     _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                                     _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p],
     },
     "attention": {
         "tnx_qkv_write": [_c_void_p, _c_int, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                           _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p,
-                          _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+                          _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p],
         "tnx_attention_any": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                               _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_attention_prefill": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
@@ -658,10 +658,26 @@ class HipOps:
                              f"{(n, num_kv, head_size, page_size)}")
         return n
 
+    @staticmethod
+    def _turn_args(turn, head_size, ctx):
+        """(a, b, positions, rows) of pair-turning tables as the entry points take them; all None / 0 without."""
+        if turn is None:
+            return None, None, None, 0
+        a, b = turn
+        _want(a, "turn a", torch.float32)
+        _want(b, "turn b", torch.float32, tuple(a.shape))
+        if a.dim() != 2 or a.shape[1] != head_size or head_size % 2:
+            raise ValueError(f"pair-turning tables are [positions, head_size] with an even head size, got {tuple(a.shape)} "
+                             f"for a head of {head_size}")
+        return a, b, ctx.positions, a.shape[0]
+
     def qkv_project(self, h, w, bias, num_heads, num_kv_write, head_size, scale, ctx, view, k_pages, v_pages,
-                    force_tiled=0):
+                    force_tiled=0, turn=None):
         """Queries, keys and values of the step's tokens: one matrix product whose epilogue scales the
-        queries and stores keys and values in their pages (bfloat16), or product and `qkv_write` apart."""
+        queries and stores keys and values in their pages (bfloat16), or product and `qkv_write` apart.
+        `turn` = (a, b), float32 `[positions, head_size]`: element d of every query and key head of a token at
+        position p becomes a[p, d] x[d] + b[p, d] x[d ^ 1] (bias added, before the scale), in the same launch."""
+        turn_a, turn_b, turn_pos, turn_rows = self._turn_args(turn, head_size, ctx)
         if isinstance(h, DeferredNorm):
             folded = self._folded_for(h, w) if force_tiled != 1 else None
             if folded is not None and (ctx.num_tokens >= 128 or self._library_product(
@@ -690,7 +706,8 @@ class HipOps:
                            _ptr(folded.d), float(h.eps), _ptr(bias), t, h.x.shape[1], _ptr(view.token_page),
                            _ptr(view.token_offset), _ptr(q), _ptr(k_pages) if num_kv_write else None,
                            _ptr(v_pages) if num_kv_write else None, float(scale), num_heads, num_kv_write, head_size,
-                           view.page_size, num_pages, int(force_tiled), _stream())
+                           view.page_size, num_pages, int(force_tiled), _ptr(turn_a), _ptr(turn_b), _ptr(turn_pos),
+                           turn_rows, _stream())
                 return q
         tiles = None
         if isinstance(w, PreparedWeight):
@@ -703,10 +720,10 @@ class HipOps:
             # and values are cached with the same rounding whichever path a token took; the queries are
             # scaled after that
             return self.qkv_write(self.linear(h, w, bias), None, num_heads, num_kv_write, head_size, scale, ctx,
-                                  view, k_pages, v_pages)
+                                  view, k_pages, v_pages, turn)
         if self.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
             return self.qkv_write(self.linear(h, w, None), bias, num_heads, num_kv_write, head_size, scale, ctx,
-                                  view, k_pages, v_pages)
+                                  view, k_pages, v_pages, turn)
         t = ctx.num_tokens
         total = (num_heads + 2 * num_kv_write) * head_size
         _want(h, "h", torch.bfloat16, (t, w.shape[1]))
@@ -722,10 +739,12 @@ class HipOps:
         self._call("gemm", "tnx_gemm_bf16_qkv", _ptr(h), _ptr(w), _ptr(tiles), _ptr(bias), t, h.shape[1],
                    _ptr(view.token_page), _ptr(view.token_offset), _ptr(q),
                    _ptr(k_pages) if num_kv_write else None, _ptr(v_pages) if num_kv_write else None, float(scale),
-                   num_heads, num_kv_write, head_size, view.page_size, num_pages, int(force_tiled), _stream())
+                   num_heads, num_kv_write, head_size, view.page_size, num_pages, int(force_tiled), _ptr(turn_a),
+                   _ptr(turn_b), _ptr(turn_pos), turn_rows, _stream())
         return q
 
-    def qkv_write(self, qkv, bias, num_heads, num_kv_write, head_size, scale, ctx, view, k_pages, v_pages):
+    def qkv_write(self, qkv, bias, num_heads, num_kv_write, head_size, scale, ctx, view, k_pages, v_pages, turn=None):
+        turn_a, turn_b, _, turn_rows = self._turn_args(turn, head_size, ctx)
         t = ctx.num_tokens
         total = (num_heads + 2 * num_kv_write) * head_size
         _want(qkv, "qkv", self.dtype, (t, total))
@@ -744,7 +763,8 @@ class HipOps:
                    num_pages, _ptr(q), _ptr(k_pages) if num_kv_write else None,
                    _ptr(v_pages) if num_kv_write else None, t, num_heads, num_kv_write, head_size,
                    _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(ctx.plan["tile_run"]), _ptr(ctx.plan["tile_start"]),
-                   ctx.plan["tile_run"].numel() if by_tiles else 0, QUERY_TILE, _stream())
+                   ctx.plan["tile_run"].numel() if by_tiles else 0, QUERY_TILE, _ptr(turn_a), _ptr(turn_b), turn_rows,
+                   _stream())
         return q
 
     def attention(self, q, num_heads, num_kv_heads, head_size, ctx, view, k_pages, v_pages, window=None):

@@ -116,20 +116,28 @@ class ReferenceOps:
 
     # ---------------------------------------------------------------- attention
 
-    def qkv_project(self, h, w, bias, num_heads, num_kv_write, head_size, scale, ctx, view, k_pages, v_pages):
+    def qkv_project(self, h, w, bias, num_heads, num_kv_write, head_size, scale, ctx, view, k_pages, v_pages, turn=None):
         """The projection to queries, keys and values (`w` holds the three stacked by rows), then
         `qkv_write`."""
         return self.qkv_write(self.linear(h, w, None), bias, num_heads, num_kv_write, head_size, scale, ctx, view,
-                              k_pages, v_pages)
+                              k_pages, v_pages, turn)
 
-    def qkv_write(self, qkv, bias, num_heads, num_kv_write, head_size, scale, ctx, view, k_pages, v_pages):
-        """Bias, query scale, and the step's keys and values into their pages:
-        page `table[run][position // page_size]`, place `position % page_size`."""
+    def qkv_write(self, qkv, bias, num_heads, num_kv_write, head_size, scale, ctx, view, k_pages, v_pages, turn=None):
+        """Bias, then `turn` = (a, b), float32 `[positions, head_size]`: element d of every query and key head
+        of a token at position p becomes a[p, d] x[d] + b[p, d] x[d ^ 1]; then the query scale, and the step's
+        keys and values into their pages: page `table[run][position // page_size]`, place `position % page_size`."""
         t = qkv.shape[0]
         y = qkv.float()
         if bias is not None:
             y = y + bias.float()
         nq = num_heads * head_size
+        if turn is not None:
+            a, b = turn
+            turned = nq + num_kv_write * head_size
+            at = ctx.positions.long().clamp(0, a.shape[0] - 1)
+            x = y[:, :turned].reshape(t, -1, head_size)
+            beside = x.reshape(t, -1, head_size // 2, 2).flip(-1).reshape(t, -1, head_size)
+            y = torch.cat([(a[at][:, None, :] * x + b[at][:, None, :] * beside).reshape(t, turned), y[:, turned:]], dim=1)
         q = (y[:, :nq] * scale).to(self.dtype)
         if num_kv_write:
             nk = num_kv_write * head_size

@@ -144,13 +144,24 @@ class PositionEncoding(Part):
     num_kv_heads, head_size)` is the hook of encodings that turn queries and keys inside a mixer: the
     attention mixer calls it, when its spec names such an encoding as `rotation`, with the step's
     `[T, (num_heads + 2 num_kv_heads) * head_size]` projections (bias added, query not yet scaled) and
-    `ctx.positions`, and stores what it returns. A part leaves the hook it does not use as it is."""
+    `ctx.positions`, and stores what it returns; or, for the common pairwise form, with nothing at all:
+    see `pair_tables`. A part leaves the hook it does not use as it is."""
 
     def at_input(self, x, positions, want_compute: bool):
         return None
 
     def on_query_key(self, qkv, ctx, num_heads: int, num_kv_heads: int, head_size: int):
         return qkv
+
+    def pair_tables(self, head_size: int):
+        """For an encoding that turns queries and keys pair by pair: float32 tables `(a, b)`, both
+        `[positions, head_size]`, such that element d of a head of the token at position p becomes
+        a[p, d] x[d] + b[p, d] x[d ^ 1]; asked once, after loading. The attention mixer then hands them to the
+        projection, which applies them where it adds the bias, in the same launch, and `on_query_key` is not
+        called; such a part may be `recordable`. None (the default): the encoding is not of that form. An
+        encoding that pairs element d with d + head_size / 2 is of that form once the rows of the query and
+        key projections are put in the order (0, h/2, 1, h/2 + 1, ...) in every head, which changes no score."""
+        return None
 
 
 class Block(Part):

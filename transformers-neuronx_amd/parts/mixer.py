@@ -23,8 +23,9 @@ class Attention(Mixer):
     `num_kv_heads < num_heads` groups query heads over shared key/value heads.
     `own_kv=False` builds a mixer without key/value projections that reads the
     cache another call of the run order writes. `rotation` names a position
-    encoding (a `PartSpec` of the position registry) whose `on_query_key` turns
-    the queries and keys before they are scaled and stored; OPT has none.
+    encoding (a `PartSpec` of the position registry) that turns the queries and
+    keys before they are scaled and stored: through its `pair_tables`, inside the
+    projection's launch, or else through its `on_query_key`; OPT has none.
     """
 
     recordable = True
@@ -80,8 +81,10 @@ class Attention(Mixer):
                       if self.has_bias else None)
         self.w_out = ops.prepare_weight(tensors[f"{prefix}{on}.weight"])
         self.b_out = tensors[f"{prefix}{on}.bias"] if self.has_bias else None
+        self.turn = None
         if self.rotation is not None:
             self.rotation.load(tensors, prefix + "rotation", ops, dtype)
+            self.turn = self.rotation.pair_tables(self.head_size)     # the pairwise form: applied by the projection
 
     def first_weight(self):
         return self.w_qkv
@@ -103,7 +106,7 @@ class Attention(Mixer):
             raise ValueError("an attention mixer with own_kv writes its cache; one without reads another's")
         view = ctx.groups[cache.group]
         kv_write = self.num_kv_heads if self.own_kv else 0
-        if self.rotation is not None:
+        if self.rotation is not None and self.turn is None:
             # the projections with their bias, turned by the encoding, then scaled and stored
             qkv = self.ops.linear(h, self.w_qkv, self.b_qkv)
             qkv = self.rotation.on_query_key(qkv, ctx, self.num_heads, kv_write, self.head_size)
@@ -114,7 +117,7 @@ class Attention(Mixer):
             return self.ops.linear(c, self.w_out, self.b_out, residual=residual, out_f32=True)
         q = self.ops.qkv_project(h, self.w_qkv, self.b_qkv, self.num_heads,
                                  self.num_kv_heads if self.own_kv else 0, self.head_size, self.scale, ctx, view,
-                                 cache.k_pages, cache.v_pages)
+                                 cache.k_pages, cache.v_pages, **({"turn": self.turn} if self.turn is not None else {}))
         c = self.ops.attention(q, self.num_heads, self.num_kv_heads, self.head_size, ctx, view,
                                cache.k_pages, cache.v_pages, self.window)
         return self.ops.linear(c, self.w_out, self.b_out, residual=residual, out_f32=True)
