@@ -247,6 +247,12 @@ CODED_CASES = [
     (2, 1, 128, 16, [60, 1], [70, 129], 40),
     (1, 1, 256, 16, [33, 1], [0, 200], None),
     (2, 2, 16, 16, [1, 30], [800, 0], None),                 # ten bits of position in a head of sixteen
+    # heads that share keys and values are taken together when decoding: a group of 20 (16 and 4), of 8 at the
+    # largest head size (one block's worth), of 8 over many tiles, of 5 with a window
+    (40, 2, 64, 64, [1, 1], [700, 300], None),
+    (24, 3, 256, 16, [1, 3], [300, 10], None),
+    (8, 1, 128, 64, [1, 1, 1], [2000, 17, 255], None),
+    (10, 2, 96, 32, [1, 1], [400, 90], 70),
 ]
 
 

@@ -341,6 +341,23 @@ def test_windowed_attention_over_pages_given_back(mode):
     torch.testing.assert_close(got.float(), want.float(), rtol=2e-2, atol=2e-2)
 
 
+def test_a_page_size_that_is_no_power_of_two_is_said_once(capfd):
+    """Pages of 48 tokens send decoding to the general kernel: correct, several times slower, and said so once."""
+    from transformers_neuronx_amd.kernels.hip import HipOps
+    hip, ref = _ops(torch.bfloat16)
+    HipOps._warned_page_size = False
+    ctx = _make_step([1, 1], [100, 47], 48, 8, seed=1)
+    g = torch.Generator(device=DEV).manual_seed(2)
+    q = torch.randn(2, 2 * 32, device=DEV, generator=g).to(torch.bfloat16)
+    kp = torch.randn(8, 2, 48, 32, device=DEV, generator=g).to(torch.bfloat16)
+    vp = torch.randn(8, 2, 32, 48, device=DEV, generator=g).to(torch.bfloat16)
+    for _ in range(2):
+        got = hip.attention(q, 2, 2, 32, ctx, ctx.groups["full"], kp, vp, None)
+    torch.testing.assert_close(got.float(), ref.attention(q, 2, 2, 32, ctx, ctx.groups["full"], kp, vp, None).float(),
+                               rtol=2e-2, atol=2e-2)
+    assert capfd.readouterr().err.count("no power of two") == 1
+
+
 def test_attention_refuses_bad_head_size():
     hip, _ = _ops(torch.float32)
     ctx = _make_step([1], [0], 16, 2, seed=1)

@@ -1490,7 +1490,11 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
 // every lane), which do not queue behind the tile data; the next tile's keys are asked for as soon as this
 // tile's scores are made, its values as soon as this tile's are used (NDB <= 8; beyond that the registers
 // hold one of the two at a time).
-template <int NDB, int NW>
+// PACK: for query heads that share their keys and values (fewer kv heads than heads). A block then takes one
+// kv head of one request, and the 16 columns hold up to 16 (8 at the largest head size) different query heads
+// of its group, so the keys and values are read once for all of them and not once a head; the maxima, sums and
+// results are a column's own throughout (a column is the lanes with the same lane % 16).
+template <int NDB, int NW, bool PACK>
 __global__ void __launch_bounds__(64 * NW, (NDB <= 8 ? 8 / NW : 1))
 attention_decode_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                              const bf16_t* __restrict__ v_pages, const int* __restrict__ run_start,
@@ -1502,12 +1506,19 @@ attention_decode_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   constexpr int NKS = (NDB + 1) / 2;  // steps of 32 over the head size
   constexpr int DH = 16 * NDB;        // the registers are laid out for this head size; `head_size` <= DH
   constexpr bool PIPE = NDB <= 8;     // keys and values of different tiles are in registers together
-  __shared__ float sm_o[NW][DH];
-  __shared__ float sm_m[NW], sm_l[NW];
+  constexpr int COLS = !PACK ? 1 : NDB <= 8 ? 16 : 8;     // query heads a block takes (what LDS holds of results)
+  __shared__ float sm_o[NW][COLS][DH];
+  __shared__ float sm_m[NW][COLS], sm_l[NW][COLS];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, g = lane >> 4;
-  const int split = blockIdx.x, h = blockIdx.y, dz = blockIdx.z;
-  const int kvh = h / (num_heads / num_kv);
+  const int split = blockIdx.x, dz = blockIdx.z;
+  const int group = num_heads / num_kv;
+  // h: the query head of this lane's column; kvh: the kv head of the block
+  const int chunks = PACK ? (group + COLS - 1) / COLS : 1;
+  const int kvh = PACK ? blockIdx.y / chunks : blockIdx.y / group;
+  const int col0 = PACK ? (blockIdx.y % chunks) * COLS : 0;          // the group's first head in this block
+  const bool col_on = !PACK || (r < COLS && col0 + r < group);
+  const int h = PACK ? kvh * group + min(col0 + r, group - 1) : blockIdx.y;
   const int run = decode_runs[dz];
   const int longest_given = longest_ptr[0];
   const int t = run_start[run];
@@ -1579,7 +1590,7 @@ attention_decode_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
 #pragma unroll
   for (int ks = 0; ks < NKS; ++ks) {
     const bf16x8 qv = *(const bf16x8*)(q + (size_t)t * nq + h * head_size + min(32 * ks + 8 * g, dlast));
-    qf[ks] = (32 * ks + 8 * g < head_size) ? qv : zero8;
+    qf[ks] = (32 * ks + 8 * g < head_size && col_on) ? qv : zero8;
   }
   float m = -INFINITY, l = 0.f;       // `l`: this lane's share of the sum (its own 16 keys a tile)
   f32x4 o[NDB];
@@ -1669,35 +1680,39 @@ attention_decode_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
     }
     tile0 = next;
   }
-  // o[db][i] of a lane is element 16 db + 4 g + i of the weighted values, the same in the 16 lanes of a row group
+  // o[db][i] of a lane is element 16 db + 4 g + i of the weighted values of its column (without PACK the same in
+  // the 16 lanes of a row group)
   l = rows_sum(l);
-  if (r == 0) {
+  if (PACK ? r < COLS : r == 0) {
 #pragma unroll
     for (int db = 0; db < NDB; ++db)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) sm_o[wave][16 * db + 4 * g + i] = o[db][i];
+      for (int i = 0; i < 4; ++i) sm_o[wave][PACK ? r : 0][16 * db + 4 * g + i] = o[db][i];
   }
-  if (lane == 0) {
-    sm_m[wave] = m;
-    sm_l[wave] = l;
+  if (PACK ? (g == 0 && r < COLS) : lane == 0) {
+    sm_m[wave][PACK ? r : 0] = m;
+    sm_l[wave][PACK ? r : 0] = l;
   }
   __syncthreads();
-  for (int d = threadIdx.x; d < head_size; d += 64 * NW) {
-    float mm = sm_m[0];
+  for (int idx = threadIdx.x; idx < COLS * head_size; idx += 64 * NW) {
+    const int col = idx / head_size, d = idx - col * head_size;
+    if (PACK && col0 + col >= group) break;          // (columns beyond the group: none follows that is within it)
+    const int hh = PACK ? kvh * group + col0 + col : h;
+    float mm = sm_m[0][col];
 #pragma unroll
-    for (int w = 1; w < NW; ++w) mm = fmaxf(mm, sm_m[w]);
+    for (int w = 1; w < NW; ++w) mm = fmaxf(mm, sm_m[w][col]);
     const float ms = mm == -INFINITY ? 0.f : mm;
     float ll = 0.f, oo = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
-      const float f = __expf(sm_m[w] - ms);
-      ll += sm_l[w] * f;
-      oo += sm_o[w][d] * f;
+      const float f = __expf(sm_m[w][col] - ms);
+      ll += sm_l[w][col] * f;
+      oo += sm_o[w][col][d] * f;
     }
     if (num_splits == 1) {
-      out[(size_t)t * nq + h * head_size + d] = (bf16_t)(oo / ll);
+      out[(size_t)t * nq + hh * head_size + d] = (bf16_t)(oo / ll);
     } else {
-      const size_t pi = ((size_t)dz * num_heads + h) * num_splits + split;
+      const size_t pi = ((size_t)dz * num_heads + hh) * num_splits + split;
       part_o[pi * head_size + d] = oo;
       if (d == 0) {
         part_ml[pi * 2] = mm;
@@ -1747,18 +1762,24 @@ static int attention_decode_run(const void* q, const void* k_pages, const void* 
   TNX_REQUIRE(waves == 4 || (waves == 8 && head_size <= 128),
               "attention_decode: blocks have 4 waves, or 8 up to head size 128; not %d at head size %d", waves, head_size);
   if (num_decode <= 0) return 0;
-  dim3 grid(num_splits, num_heads, num_decode);
-#define LAUNCH_MFMA(NDB)                                                                                          \
-  if (waves == 8)                                                                                                 \
-    attention_decode_mfma_kernel<NDB, 8><<<grid, 512, 0, stream>>>(                                               \
-        (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table,          \
-        table_width, page_shift, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window, \
-        num_splits, longest, head_size);                                                                          \
-  else                                                                                                            \
-    attention_decode_mfma_kernel<NDB, 4><<<grid, 256, 0, stream>>>(                                               \
-        (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table,          \
-        table_width, page_shift, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window, \
-        num_splits, longest, head_size)
+  // query heads that share keys and values are taken together, up to 16 a block (8 at head sizes beyond 128)
+  const int group = num_heads / num_kv;
+  const bool pack = group > 1;
+  const int cols = head_size <= 128 ? 16 : 8;
+  dim3 grid(num_splits, pack ? num_kv * ((group + cols - 1) / cols) : num_heads, num_decode);
+#define MFMA_ARGS                                                                                                 \
+  (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, table_width,    \
+      page_shift, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window, num_splits,    \
+      longest, head_size
+#define LAUNCH_MFMA(NDB)                                                                         \
+  if (waves == 8 && pack)                                                                        \
+    attention_decode_mfma_kernel<NDB, 8, true><<<grid, 512, 0, stream>>>(MFMA_ARGS);             \
+  else if (waves == 8)                                                                           \
+    attention_decode_mfma_kernel<NDB, 8, false><<<grid, 512, 0, stream>>>(MFMA_ARGS);            \
+  else if (pack)                                                                                 \
+    attention_decode_mfma_kernel<NDB, 4, true><<<grid, 256, 0, stream>>>(MFMA_ARGS);             \
+  else                                                                                           \
+    attention_decode_mfma_kernel<NDB, 4, false><<<grid, 256, 0, stream>>>(MFMA_ARGS)
     // the registers are laid out for the next of these sizes; a smaller head repeats its last chunk there
     if (head_size <= 32) {
       LAUNCH_MFMA(2);
@@ -1768,12 +1789,12 @@ static int attention_decode_run(const void* q, const void* k_pages, const void* 
       LAUNCH_MFMA(6);
     } else if (head_size <= 128) {
       LAUNCH_MFMA(8);
+    } else if (pack) {
+      attention_decode_mfma_kernel<16, 4, true><<<grid, 256, 0, stream>>>(MFMA_ARGS);
     } else {
-      attention_decode_mfma_kernel<16, 4><<<grid, 256, 0, stream>>>(
-          (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table,
-          table_width, page_shift, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window,
-          num_splits, longest, head_size);
+      attention_decode_mfma_kernel<16, 4, false><<<grid, 256, 0, stream>>>(MFMA_ARGS);
     }
+#undef MFMA_ARGS
 #undef LAUNCH_MFMA
   TNX_CHECK_LAUNCH("attention_decode");
   if (num_splits > 1) {

@@ -779,6 +779,11 @@ class HipOps:
         fast = (self.dtype == torch.bfloat16 and not self.force_plain_attention
                 and (ctx.plan["decode_runs"].numel() == 0
                      or view.page_size & (view.page_size - 1) == 0))
+        if self.dtype == torch.bfloat16 and not fast and not self.force_plain_attention and not HipOps._warned_page_size:
+            HipOps._warned_page_size = True
+            build._log(f"a page size of {view.page_size} is no power of two: steps with decoding requests run on the "
+                       "general attention kernel (one wave a query), several times slower than the matrix-unit "
+                       "kernels that pages of 16, 32, 64, ... tokens get")
         if not fast:
             self._call("attention", "tnx_attention_any", _ptr(q), _code(self.dtype), _ptr(k_pages), _ptr(v_pages),
                        _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width,
@@ -793,7 +798,8 @@ class HipOps:
                        _stream())
         n_dec = ctx.plan["decode_runs"].numel()
         if n_dec:
-            splits, waves = self._decode_splits(ctx, n_dec * num_heads, window, head_size)
+            splits, waves = self._decode_splits(ctx, n_dec * self._decode_blocks(num_heads, num_kv_heads, head_size),
+                                                window, head_size)
             part_o = part_ml = None
             if splits > 1:
                 part_o = torch.empty(n_dec * num_heads * splits * head_size, dtype=torch.float32, device=q.device)
@@ -837,6 +843,7 @@ class HipOps:
             plan = ctx.plans[("prefill_sets", window)] = 0 if two < one else 2
         return plan
 
+    _warned_page_size = False         # said once a process
     value_tiles = True                # tests clear it to write every value token by token
     prefill_direct = False            # tests set it: True, the prompt kernel that reads pages without LDS staging;
                                       # 2, the staged one with one set of four waves a block; 3, with two
@@ -844,6 +851,15 @@ class HipOps:
     decode_waves = 4                  # waves of a decode attention block (8 is kept for head sizes up to 128)
     decode_blocks_wanted = None       # the keys of decoding requests are split until about this many blocks run;
                                       # None: one block a compute unit
+
+    @staticmethod
+    def _decode_blocks(num_heads: int, num_kv_heads: int, head_size: int) -> int:
+        """Blocks of the decode attention a request and a share of its keys: one a head, or, where heads share
+        keys and values, one for every 16 heads of a group (8 at head sizes beyond 128), which read them once."""
+        group = num_heads // num_kv_heads
+        if group == 1:
+            return num_heads
+        return num_kv_heads * -(-group // (16 if head_size <= 128 else 8))
 
     def _decode_splits(self, ctx, pairs: int, window: int, head_size: int = 128):
         """(splits, waves): how many blocks share the keys of one decoding (request, head), and how many
@@ -883,7 +899,7 @@ class HipOps:
             alike = False         # whole requests already come out even over the compute units
         return (max(fill_the_chip, fills) if alike else fill_the_chip), waves
 
-    def attention_launch_shape(self, step, num_heads: int, window, head_size: int):
+    def attention_launch_shape(self, step, num_heads: int, window, head_size: int, num_kv_heads: Optional[int] = None):
         """What the decode attention's launch in a recorded step is sized by beyond the number of requests: the
         blocks that share a request's keys (and their waves), for a `PackedStep` about to be replayed. A
         recorded step is sized for the longest request the model allows; how requests about as long as one
@@ -893,8 +909,9 @@ class HipOps:
         if n_dec == 0 or self.dtype != torch.bfloat16:
             return None
         fills, alike = step.plan_host.get("decode_shape", (0, False))
-        return ("decode", num_heads, head_size) + self._splits_for(step.length_bound, fills, alike, n_dec * num_heads,
-                                                                   int(window or 0), head_size)
+        blocks = self._decode_blocks(num_heads, num_kv_heads or num_heads, head_size)
+        return ("decode", blocks, head_size) + self._splits_for(step.length_bound, fills, alike, n_dec * blocks,
+                                                                int(window or 0), head_size)
 
     # ---------------------------------------------------------------- output end
 

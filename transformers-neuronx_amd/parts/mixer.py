@@ -95,7 +95,7 @@ class Attention(Mixer):
 
     def launch_shape(self, step):
         shape = getattr(self.ops, "attention_launch_shape", None)
-        return shape(step, self.num_heads, self.window, self.head_size) if shape is not None else None
+        return shape(step, self.num_heads, self.window, self.head_size, self.num_kv_heads) if shape is not None else None
 
     def flops_per_token(self, keys: float = 0.0) -> float:
         seen = min(keys, self.window) if self.window else keys
