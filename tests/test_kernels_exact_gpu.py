@@ -22,6 +22,16 @@ def _ints(g, *shape, low=-4, high=4):
     return torch.randint(low, high + 1, shape, device=DEV, generator=g).float()
 
 
+def _apart(pages, pad):
+    """The same pages with `pad` elements between one page and the next, as a cache with `page_pad_bytes` lays
+    them out; what lies between them is NaN."""
+    n = pages.shape[0]
+    count = pages[0].numel()
+    whole = torch.full((n, count + pad), float("nan"), dtype=pages.dtype, device=pages.device)
+    whole[:, :count] = pages.reshape(n, count)
+    return whole[:, :count].view(pages.shape)
+
+
 # ---------------------------------------------------------------- products
 
 def _exact_product(x, w, bias, residual, act, out_dtype):
@@ -94,8 +104,8 @@ def test_fused_projection_of_small_integers_is_exact(m):
     view = ctx.groups["full"]
     n = (heads + 2 * kv) * hs
     x, w, bias = _ints(g, m, k).to(torch.bfloat16), _ints(g, n, k).to(torch.bfloat16), _ints(g, n, low=-64, high=64)
-    kp = torch.full((num_pages, kv, ps, hs), float("nan"), device=DEV, dtype=torch.bfloat16)
-    vp = torch.full((num_pages, kv, hs, ps), float("nan"), device=DEV, dtype=torch.bfloat16)
+    kp = _apart(torch.full((num_pages, kv, ps, hs), float("nan"), device=DEV, dtype=torch.bfloat16), 8 * m)
+    vp = _apart(torch.full((num_pages, kv, hs, ps), float("nan"), device=DEV, dtype=torch.bfloat16), 8 * m)
     q = hip.qkv_project(x, hip.prepare_weight(w), bias, heads, kv, hs, 0.125, ctx, view, kp, vp)
     full = x.double() @ w.double().t() + bias.double()
     torch.testing.assert_close(q.float(), (full[:, :heads * hs] * 0.125).float().to(torch.bfloat16).float(), **EXACT)
@@ -139,8 +149,8 @@ def test_projection_that_turns_pairs_is_exact(m, own, normed):
     want_k = part[:, heads * hs:].float().to(torch.bfloat16).float().view(m, kv, hs)
     want_v = full[:, turned:].float().to(torch.bfloat16).float().view(m, kv, hs)
     for weight in (hip.prepare_weight(w), w):
-        kp = torch.full((num_pages, kv, ps, hs), float("nan"), device=DEV, dtype=torch.bfloat16)
-        vp = torch.full((num_pages, kv, hs, ps), float("nan"), device=DEV, dtype=torch.bfloat16)
+        kp = _apart(torch.full((num_pages, kv, ps, hs), float("nan"), device=DEV, dtype=torch.bfloat16), 64)
+        vp = _apart(torch.full((num_pages, kv, hs, ps), float("nan"), device=DEV, dtype=torch.bfloat16), 64)
         h = x.to(torch.bfloat16)
         if normed:
             # a LayerNorm that changes nothing that matters here cannot be exact: the folded form is compared below
@@ -278,6 +288,10 @@ def test_attention_with_two_tied_keys_is_exact(case):
         got = ops.attention(q, heads, kv, hs, ctx, view, kp, vp, window)
         worst = float((got.float() - want).abs().max())
         assert worst <= 1e-6, f"{name}: differs by {worst}"
+        # and with the pages some way apart in memory, as the engine's cache lays them out
+        got = ops.attention(q, heads, kv, hs, ctx, view, _apart(kp, 136), _apart(vp, 136), window)
+        worst = float((got.float() - want).abs().max())
+        assert worst <= 1e-6, f"{name}, pages apart: differs by {worst}"
     # the comparison can fail, and pages belong to whom the table says: one more in every value of the first
     # request's pages is one more in every result of that request and nothing in the others'
     pages = view.block_table[0][view.block_table[0] >= 0].long()

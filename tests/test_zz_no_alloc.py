@@ -48,7 +48,7 @@ def _both(lib, ctx, q, kp, vp, num_pages, heads, kv, hs, ps, splits, waves):
     part_ml = torch.full((n * heads * splits * 2,), float("nan"), dtype=torch.float32, device=DEV)
     rc = lib.tnx_attention_decode(p(q), p(kp), p(vp), p(ctx.run_start), p(ctx.cached_lens), p(view.block_table),
                                   view.width, ps, num_pages, p(ctx.plan["decode_runs"]), n, p(out_ws), p(part_o), p(part_ml),
-                                  heads, kv, hs, 0, splits, waves, p(ctx.plan["longest_decode"]), stream)
+                                  heads, kv, hs, 0, splits, waves, p(ctx.plan["longest_decode"]), 0, stream)
     assert rc == 0, lib.tnx_last_error().decode()
     out_st = torch.full_like(q, float("nan"))
     rc = lib.tnx_attention_decode_static(p(q), p(kp), p(vp), p(ctx.run_start), p(ctx.cached_lens),

@@ -71,8 +71,15 @@ class CacheManager:
     """
 
     def __init__(self, needs: Dict[int, CacheNeed], page_size: int, num_pages, max_seqs: int,
-                 dtype: torch.dtype, device, allocate: bool = True):
+                 dtype: torch.dtype, device, allocate: bool = True, page_pad_bytes: int = 0):
+        """`page_pad_bytes`: memory left between one page and the next in every page tensor (a multiple of 32).
+        Pages whose size is a power of two lie at distances that are powers of two, and so do the requests
+        that fill them side by side: the kernels that read all requests at once then meet the same memory
+        channels at the same time. A few hundred bytes between pages take that regularity away."""
         self.page_size, self.max_seqs, self.dtype, self.device = page_size, max_seqs, dtype, device
+        if page_pad_bytes < 0 or page_pad_bytes % 32:
+            raise ValueError(f"page_pad_bytes must be a multiple of 32 from 0 up, got {page_pad_bytes}")
+        self.page_pad_bytes = page_pad_bytes
         self.slots = SlotPool(max_seqs)
         self.groups: Dict[str, PageGroup] = {}
         self.caches: Dict[int, LayerCache] = {}
@@ -94,9 +101,12 @@ class CacheManager:
                 g.cache_ids.append(cid)
                 lc = LayerCache(cid, g.name)
                 if allocate:
+                    item = torch.empty(0, dtype=dtype).element_size()
                     for name, shape in need.tensors_of_a_page():
                         dims = [page_size if d == "page" else d for d in shape]
-                        lc.pages[name] = torch.empty(g.pool.num_pages, *dims, dtype=dtype, device=device)
+                        count = int(np.prod(dims))
+                        whole = torch.empty(g.pool.num_pages, count + page_pad_bytes // item, dtype=dtype, device=device)
+                        lc.pages[name] = whole[:, :count].view(g.pool.num_pages, *dims)
                 self.caches[cid] = lc
             elif need.kind == "state":
                 lc = LayerCache(cid, None)
@@ -111,7 +121,7 @@ class CacheManager:
     # ---------------------------------------------------------------- sizes
 
     @staticmethod
-    def bytes_per_page(needs: Dict[int, CacheNeed], page_size: int, dtype: torch.dtype) -> int:
+    def bytes_per_page(needs: Dict[int, CacheNeed], page_size: int, dtype: torch.dtype, page_pad_bytes: int = 0) -> int:
         item = torch.empty(0, dtype=dtype).element_size()
         total = 0
         for n in needs.values():
@@ -121,7 +131,7 @@ class CacheManager:
                 count = 1
                 for d in shape:
                     count *= page_size if d == "page" else d
-                total += count * item
+                total += count * item + page_pad_bytes
         return total
 
     # ---------------------------------------------------------------- requests

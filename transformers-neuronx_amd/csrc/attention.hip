@@ -21,7 +21,8 @@ qkv_write_kernel(const T* __restrict__ qkv, const float* __restrict__ bias, floa
                  const int* __restrict__ table, int table_width, int page_size, int num_pages, T* __restrict__ q_out,
                  T* __restrict__ k_pages, T* __restrict__ v_pages, int num_heads, int num_kv, int head_size,
                  const int* __restrict__ run_start, int values_of_single_tokens_only,
-                 const float* __restrict__ turn_a, const float* __restrict__ turn_b, int turn_rows) {
+                 const float* __restrict__ turn_a, const float* __restrict__ turn_b, int turn_rows, int page_pad) {
+  const size_t page_stride = (size_t)num_kv * page_size * head_size + page_pad;     // elements from page to page
   const int t = blockIdx.x;
   const int nq = num_heads * head_size, nk = num_kv * head_size;
   const int total = nq + 2 * nk;
@@ -58,7 +59,7 @@ qkv_write_kernel(const T* __restrict__ qkv, const float* __restrict__ bias, floa
   if (page < 0 || page >= num_pages) return;
   if (i0 < nq + nk) {
     const int j0 = i0 - nq, h = j0 / head_size, d = j0 % head_size;
-    T* dst = k_pages + (((size_t)page * num_kv + h) * page_size + off) * head_size + d;
+    T* dst = k_pages + (size_t)page * page_stride + ((size_t)h * page_size + off) * head_size + d;
 #pragma unroll
     for (int j = 0; j < 8; ++j) dst[j] = from_f32<T>(v[j]);
   } else {
@@ -67,7 +68,7 @@ qkv_write_kernel(const T* __restrict__ qkv, const float* __restrict__ bias, floa
       if (run_start[r + 1] - run_start[r] > 1) return;
     }
     const int j0 = i0 - nq - nk, h = j0 / head_size, d = j0 % head_size;
-    T* dst = v_pages + (((size_t)page * num_kv + h) * head_size + d) * page_size + off;
+    T* dst = v_pages + (size_t)page * page_stride + ((size_t)h * head_size + d) * page_size + off;
 #pragma unroll
     for (int j = 0; j < 8; ++j) dst[(size_t)j * page_size] = from_f32<T>(v[j]);
   }
@@ -84,8 +85,9 @@ value_tiles_kernel(const bf16_t* __restrict__ qkv, const float* __restrict__ bia
                    const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
                    int page_size, int num_pages, const int* __restrict__ tile_run,
                    const int* __restrict__ tile_q0, bf16_t* __restrict__ v_pages, int num_heads, int num_kv,
-                   int head_size) {
+                   int head_size, int page_pad) {
   __shared__ __attribute__((aligned(16))) bf16_t sm[VT_TOKENS * VT_ROW];
+  const size_t page_stride = (size_t)num_kv * page_size * head_size + page_pad;
   const int run = tile_run[blockIdx.x], q0 = tile_q0[blockIdx.x], kvh = blockIdx.y;
   const int t0 = run_start[run] + q0;
   const int n = min(VT_TOKENS, run_start[run + 1] - t0);
@@ -113,7 +115,7 @@ value_tiles_kernel(const bf16_t* __restrict__ qkv, const float* __restrict__ bia
       const int blk = pos / page_size;
       const int page = blk < table_width ? tab[blk] : -1;
       if (page < 0 || page >= num_pages) continue;
-      bf16_t* dst = v_pages + (((size_t)page * num_kv + kvh) * head_size + dc + d) * page_size + pos % page_size;
+      bf16_t* dst = v_pages + (size_t)page * page_stride + ((size_t)kvh * head_size + dc + d) * page_size + pos % page_size;
       const int i0 = pos - p0;                         // the group's first token within the tile; may be < 0
       if (i0 >= 0 && i0 + 8 <= n) {
         bf16x8 v;
@@ -137,8 +139,11 @@ extern "C" int tnx_qkv_write(const void* qkv, int dtype, const float* bias, floa
                              int num_pages, void* q_out, void* k_pages, void* v_pages, int tokens, int num_heads,
                              int num_kv, int head_size, const int* run_start, const int* cached_lens,
                              const int* tile_run, const int* tile_q0, int num_tiles, int tile_tokens,
-                             const float* turn_a, const float* turn_b, int turn_rows, hipStream_t stream) {
+                             const float* turn_a, const float* turn_b, int turn_rows, int page_pad,
+                             hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && num_heads > 0 && num_kv >= 0 && head_size > 0, "qkv_write: bad sizes");
+  TNX_REQUIRE(page_pad >= 0 && page_pad % 8 == 0, "qkv_write: pages are %d elements apart beyond their size, not a "
+              "multiple of 8 from 0 up", page_pad);
   TNX_REQUIRE((turn_a == nullptr) == (turn_b == nullptr) && (!turn_a || turn_rows > 0),
               "qkv_write: the pair-turning tables come both or not at all, with their number of rows");
   TNX_REQUIRE(page_size > 0 && table_width > 0, "qkv_write: bad page table");
@@ -158,18 +163,18 @@ extern "C" int tnx_qkv_write(const void* qkv, int dtype, const float* bias, floa
     qkv_write_kernel<float><<<grid, 256, 0, stream>>>((const float*)qkv, bias, scale, positions, token_request,
                                                         table, table_width, page_size, num_pages, (float*)q_out,
                                                         (float*)k_pages, (float*)v_pages, num_heads, num_kv, head_size,
-                                                        run_start, 0, turn_a, turn_b, turn_rows);
+                                                        run_start, 0, turn_a, turn_b, turn_rows, page_pad);
   else
     qkv_write_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)qkv, bias, scale, positions, token_request,
                                                          table, table_width, page_size, num_pages, (bf16_t*)q_out,
                                                          (bf16_t*)k_pages, (bf16_t*)v_pages, num_heads, num_kv,
                                                          head_size, run_start, by_tiles ? 1 : 0, turn_a, turn_b,
-                                                         turn_rows);
+                                                         turn_rows, page_pad);
   TNX_CHECK_LAUNCH("qkv_write");
   if (by_tiles) {
     value_tiles_kernel<<<dim3(num_tiles, num_kv), 256, 0, stream>>>(
         (const bf16_t*)qkv, bias, run_start, cached_lens, table, table_width, page_size, num_pages, tile_run, tile_q0,
-        (bf16_t*)v_pages, num_heads, num_kv, head_size);
+        (bf16_t*)v_pages, num_heads, num_kv, head_size, page_pad);
     TNX_CHECK_LAUNCH("value_tiles");
   }
   return 0;
@@ -188,8 +193,10 @@ __global__ void __launch_bounds__(256)
 attention_any_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                      const int* __restrict__ positions, const int* __restrict__ token_request,
                      const int* __restrict__ table, int table_width, int page_size, int num_pages,
-                     T* __restrict__ out, int tokens, int num_heads, int num_kv, int head_size, int window) {
+                     T* __restrict__ out, int tokens, int num_heads, int num_kv, int head_size, int window,
+                     int page_pad) {
   __shared__ float qs[4][256];
+  const size_t page_stride = (size_t)num_kv * page_size * head_size + page_pad;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const long long idx = (long long)blockIdx.x * 4 + wave;
   const bool active = idx < (long long)tokens * num_heads;
@@ -214,7 +221,7 @@ attention_any_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, con
     if (valid) {
       const int page = tab[key / page_size];
       if (page >= 0 && page < num_pages) {
-        const T* kp = k_pages + (((size_t)page * num_kv + kvh) * page_size + key % page_size) * head_size;
+        const T* kp = k_pages + (size_t)page * page_stride + ((size_t)kvh * page_size + key % page_size) * head_size;
         float a = 0.f;
         for (int d = 0; d < head_size; d += 4) {
           a = fmaf(qs[wave][d], to_f32(kp[d]), a);
@@ -240,7 +247,7 @@ attention_any_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, con
       const int page = tab[key0 / page_size];
       if (page < 0 || page >= num_pages) continue;
       const int off0 = key0 % page_size;
-      const T* vbase = v_pages + ((size_t)page * num_kv + kvh) * head_size * page_size + off0;
+      const T* vbase = v_pages + (size_t)page * page_stride + (size_t)kvh * head_size * page_size + off0;
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         const float pj = __shfl(p, 16 * grp + j, 64);
@@ -265,8 +272,9 @@ attention_any_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, con
 extern "C" int tnx_attention_any(const void* q, int dtype, const void* k_pages, const void* v_pages,
                                  const int* positions, const int* token_request, const int* table, int table_width,
                                  int page_size, int num_pages, void* out, int tokens, int num_heads, int num_kv,
-                                 int head_size, int window, hipStream_t stream) {
+                                 int head_size, int window, int page_pad, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && num_heads > 0 && num_kv > 0 && num_heads % num_kv == 0, "attention: bad head counts");
+  TNX_REQUIRE(page_pad >= 0 && page_pad % 8 == 0, "attention: bad distance between pages");
   TNX_REQUIRE(head_size % 16 == 0 && head_size >= 16 && head_size <= 256,
               "attention: head size %d is not a multiple of 16 in [16, 256]", head_size);
   TNX_REQUIRE(page_size % 16 == 0 && page_size > 0, "attention: page size %d is not a multiple of 16", page_size);
@@ -277,11 +285,11 @@ extern "C" int tnx_attention_any(const void* q, int dtype, const void* k_pages, 
   if (dtype == TNX_F32)
     attention_any_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>(
         (const float*)q, (const float*)k_pages, (const float*)v_pages, positions, token_request, table, table_width,
-        page_size, num_pages, (float*)out, tokens, num_heads, num_kv, head_size, window);
+        page_size, num_pages, (float*)out, tokens, num_heads, num_kv, head_size, window, page_pad);
   else
     attention_any_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>(
         (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, positions, token_request, table,
-        table_width, page_size, num_pages, (bf16_t*)out, tokens, num_heads, num_kv, head_size, window);
+        table_width, page_size, num_pages, (bf16_t*)out, tokens, num_heads, num_kv, head_size, window, page_pad);
   TNX_CHECK_LAUNCH("attention_any");
   return 0;
 }
@@ -307,8 +315,9 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict_
                          const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
                          int page_size, int num_pages, const int* __restrict__ tile_run,
                          const int* __restrict__ tile_q0, bf16_t* __restrict__ out, int num_heads, int num_kv,
-                         int head_size, int window) {
+                         int head_size, int window, int page_pad) {
   constexpr int NKS = (NDB + 1) / 2;  // MFMA steps of 32 over the head size
+  const size_t page_stride = (size_t)num_kv * page_size * head_size + page_pad;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int tile = blockIdx.x / num_heads, h = blockIdx.x % num_heads;
@@ -357,7 +366,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict_
       if (key0 <= last_q) page = tab[key0 / page_size];
       if (page >= 0 && page < num_pages) {
         const bf16_t* kbase =
-            k_pages + (((size_t)page * num_kv + kvh) * page_size + key0 % page_size + r) * head_size;
+            k_pages + (size_t)page * page_stride + ((size_t)kvh * page_size + key0 % page_size + r) * head_size;
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
           const int d0 = 32 * ks + 8 * g;
@@ -427,7 +436,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict_
         int page = -1;
         if (key0 <= last_q) page = tab[key0 / page_size];
         vok[b] = page >= 0 && page < num_pages;
-        vbase[b] = v_pages + ((size_t)(vok[b] ? page : 0) * num_kv + kvh) * head_size * page_size +
+        vbase[b] = v_pages + (size_t)(vok[b] ? page : 0) * page_stride + (size_t)kvh * head_size * page_size +
                    key0 % page_size + 4 * g;
       }
       const bool tail = tile0 + 32 * t + 32 > total;   // some keys of this step lie beyond the request
@@ -501,7 +510,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
                              const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
                              int page_shift, int num_pages, const int* __restrict__ tile_run,
                              const int* __restrict__ tile_q0, bf16_t* __restrict__ out, int num_heads, int num_kv,
-                             int head_size, int window) {
+                             int head_size, int window, int page_pad) {
   constexpr int NKS = (NDB + 1) / 2;
   constexpr int DMAX = 16 * NDB;
   using Layout = PrefillTileLayout<NDB, FAST>;
@@ -532,6 +541,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   const int ndb = head_size / 16;
   const int cpr = head_size / 8;            // chunks per key row
   const size_t head_stride = (size_t)page_size * head_size;
+  const size_t page_stride = (size_t)num_kv * head_stride + page_pad;
 
   bf16x8 qf[2][NKS];
   int qpos[2];
@@ -603,7 +613,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
       // keys of the page beyond the request are read as they lie: their scores are masked by position and
       // their values are zeroed when the tile is staged
       const int page = min(max(tile_page, 0), num_pages - 1);
-      const size_t base = ((size_t)page * num_kv + kvh) * head_stride;
+      const size_t base = (size_t)page * page_stride + (size_t)kvh * head_stride;
       const bf16_t* kb = k_pages + base + (size_t)(tile0 & pmask) * head_size;
       const bf16_t* vb = v_pages + base + (tile0 & pmask);
 #pragma unroll
@@ -616,14 +626,14 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
     for (int j = 0; j < KCH; ++j) {
       const int key = min(tile0 + kc_key[j], total - 1);
       const int page = min(max(kpage[j], 0), num_pages - 1);
-      kreg[j] = *(const bf16x8*)(k_pages + ((size_t)page * num_kv + kvh) * head_stride +
+      kreg[j] = *(const bf16x8*)(k_pages + (size_t)page * page_stride + (size_t)kvh * head_stride +
                                  (size_t)(key & pmask) * head_size + kc_dc[j] * 8);
     }
 #pragma unroll
     for (int j = 0; j < VCH; ++j) {
       const int key = min(tile0 + 8 * vc_kc[j], (total - 1) & ~7);
       const int page = min(max(vpage[j], 0), num_pages - 1);
-      vreg[j] = *(const bf16x8*)(v_pages + ((size_t)page * num_kv + kvh) * head_stride +
+      vreg[j] = *(const bf16x8*)(v_pages + (size_t)page * page_stride + (size_t)kvh * head_stride +
                                  (size_t)vc_d[j] * page_size + (key & pmask));
     }
   };
@@ -855,7 +865,7 @@ static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, co
                               const bf16_t* v_pages, const int* run_start, const int* cached_lens, const int* table,
                               int table_width, int page_shift, int num_pages, const int* tile_run,
                               const int* tile_q0, bf16_t* out, int num_heads, int num_kv, int head_size,
-                              int window) {
+                              int window, int page_pad) {
   constexpr int DMAX = 16 * NDB;
   using Layout = PrefillTileLayout<NDB, FAST>;
   constexpr size_t bytes = GROUPS * 2 * (size_t)(Layout::KBUF + Layout::VBUF) * sizeof(bf16_t);
@@ -874,7 +884,8 @@ static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, co
   }
   attention_prefill_lds_kernel<NDB, FAST, GROUPS><<<grid, 256 * GROUPS, bytes, stream>>>(q, k_pages, v_pages, run_start, cached_lens, table,
                                                                  table_width, page_shift, num_pages, tile_run,
-                                                                 tile_q0, out, num_heads, num_kv, head_size, window);
+                                                                 tile_q0, out, num_heads, num_kv, head_size, window,
+                                                                 page_pad);
   return 0;
 }
 
@@ -905,7 +916,7 @@ attention_prefill_pipelined_kernel(const bf16_t* __restrict__ q, const bf16_t* _
                                    const int* __restrict__ cached_lens, const int* __restrict__ table,
                                    int table_width, int page_shift, int num_pages,
                                    const int* __restrict__ tile_run, const int* __restrict__ tile_q0,
-                                   bf16_t* __restrict__ out, int num_heads, int num_kv) {
+                                   bf16_t* __restrict__ out, int num_heads, int num_kv, int page_pad) {
   static_assert(NDB == 4 || NDB == 8, "head sizes 64 and 128");
   constexpr int NKS = NDB / 2, DH = 16 * NDB, CPR = 2 * NDB;   // CPR: 16-byte chunks of a key row
   constexpr int TILE_BYTES = 64 * DH * 2;                       // 64 keys, and as many values
@@ -931,6 +942,7 @@ attention_prefill_pipelined_kernel(const bf16_t* __restrict__ q, const bf16_t* _
   const int page_size = 1 << page_shift, pmask = page_size - 1;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   const size_t head_stride = (size_t)page_size * DH;
+  const size_t page_stride = (size_t)num_kv * head_stride + page_pad;
 
   bf16x8 qf[2][NKS];
   int qpos[2];
@@ -976,11 +988,11 @@ attention_prefill_pipelined_kernel(const bf16_t* __restrict__ q, const bf16_t* _
   auto lookup = [&](int tile0) { return tab[min(tile0, total - 1) >> page_shift]; };
   auto key_source = [&](int tile0, int page) -> const bf16_t* {
     const int pg = min(max(page, 0), num_pages - 1);
-    return k_pages + ((size_t)pg * num_kv + kvh) * head_stride + (size_t)(tile0 & pmask) * DH;
+    return k_pages + (size_t)pg * page_stride + (size_t)kvh * head_stride + (size_t)(tile0 & pmask) * DH;
   };
   auto value_source = [&](int tile0, int page) -> const bf16_t* {
     const int pg = min(max(page, 0), num_pages - 1);
-    return v_pages + ((size_t)pg * num_kv + kvh) * head_stride + (tile0 & pmask);
+    return v_pages + (size_t)pg * page_stride + (size_t)kvh * head_stride + (tile0 & pmask);
   };
   auto issue_key_load = [&](int j, int buf, const bf16_t* src) {
     load_to_lds(src, key_offset(j), kbuf_lds + buf * TILE_BYTES + wave * 1024 + j * 4096);
@@ -1376,7 +1388,7 @@ static int launch_prefill_pipelined(dim3 grid, hipStream_t stream, const bf16_t*
                                     const bf16_t* v_pages, const int* run_start, const int* cached_lens,
                                     const int* table, int table_width, int page_shift, int num_pages,
                                     const int* tile_run, const int* tile_q0, bf16_t* out, int num_heads, int num_kv,
-                                    int head_size, int window) {
+                                    int head_size, int window, int page_pad) {
   constexpr size_t bytes = GROUPS * 4 * (size_t)(64 * 16 * NDB * 2);
   static_assert(bytes <= 160 * 1024, "the staging buffers must fit the 160 KB of LDS");
   static_assert(GROUPS == 1 || bytes >= (4 * NDB * 2 * 4 * 64 + 4 * 2 * 2 * 64) * sizeof(float),
@@ -1395,7 +1407,7 @@ static int launch_prefill_pipelined(dim3 grid, hipStream_t stream, const bf16_t*
   (void)window;
   attention_prefill_pipelined_kernel<NDB, GROUPS><<<grid, 256 * GROUPS, bytes, stream>>>(
       q, k_pages, v_pages, run_start, cached_lens, table, table_width, page_shift, num_pages, tile_run, tile_q0, out,
-      num_heads, num_kv);
+      num_heads, num_kv, page_pad);
   return 0;
 }
 
@@ -1403,7 +1415,8 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
                                      const int* cached_lens, const int* table, int table_width, int page_size,
                                      int num_pages, const int* tile_run, const int* tile_q0, int num_tiles, void* out,
                                      int num_heads, int num_kv, int head_size, int window, int direct,
-                                     int query_tile, hipStream_t stream) {
+                                     int query_tile, int page_pad, hipStream_t stream) {
+  TNX_REQUIRE(page_pad >= 0 && page_pad % 8 == 0, "attention_prefill: bad distance between pages");
   TNX_REQUIRE(query_tile == PREFILL_Q_TILE,
               "attention_prefill: the tiles hold %d queries each, the kernels take %d: a tile's later queries would "
               "be skipped", query_tile, PREFILL_Q_TILE);
@@ -1428,7 +1441,8 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
     int rc = -1;
 #define LDS_ARGS                                                                                                 \
   grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, \
-      table_width, page_shift, num_pages, tile_run, tile_q0, (bf16_t*)out, num_heads, num_kv, head_size, window
+      table_width, page_shift, num_pages, tile_run, tile_q0, (bf16_t*)out, num_heads, num_kv, head_size, window, \
+      page_pad
 #define LAUNCH_LDS(NDB)                                                                                          \
   {                                                                                                              \
     constexpr int G = NDB <= 8 ? 2 : 1;     /* two sets of waves where LDS holds the buffers of both */          \
@@ -1459,7 +1473,7 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
 #define LAUNCH_PREFILL(NDB)                                                                                        \
   attention_prefill_kernel<NDB><<<grid, 256, 0, stream>>>(                                                         \
       (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, table_width, \
-      page_size, num_pages, tile_run, tile_q0, (bf16_t*)out, num_heads, num_kv, head_size, window)
+      page_size, num_pages, tile_run, tile_q0, (bf16_t*)out, num_heads, num_kv, head_size, window, page_pad)
   if (head_size <= 64)
     LAUNCH_PREFILL(4);
   else if (head_size <= 128)
@@ -1502,7 +1516,7 @@ attention_decode_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
                              int page_shift, int num_pages, const int* __restrict__ decode_runs,
                              bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
                              int num_heads, int num_kv, int window, int num_splits,
-                             const int* __restrict__ longest_ptr, int head_size) {
+                             const int* __restrict__ longest_ptr, int head_size, int page_pad) {
   constexpr int NKS = (NDB + 1) / 2;  // steps of 32 over the head size
   constexpr int DH = 16 * NDB;        // the registers are laid out for this head size; `head_size` <= DH
   constexpr bool PIPE = NDB <= 8;     // keys and values of different tiles are in registers together
@@ -1530,6 +1544,7 @@ attention_decode_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   const int longest = window > 0 ? min(longest_given, window + 64) : longest_given;
   const int keys_per_split = (((longest + num_splits - 1) / num_splits) + 63) & ~63;
   const size_t head_stride = (size_t)page_size * head_size;   // elements of one head of one page
+  const size_t page_stride = (size_t)num_kv * head_stride + page_pad;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
   // the pages of a tile's four blocks of 16 keys (a block of 16 lies in one page; pages of 64 keys and more
@@ -1550,7 +1565,7 @@ attention_decode_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
     for (int kb = 0; kb < 4; ++kb) {
       const int off = 32 * (kb >> 1) + 8 * (r >> 2) + 4 * (kb & 1) + (r & 3);
       const int page = (r >> 3) ? pg[2 * (kb >> 1) + 1] : pg[2 * (kb >> 1)];
-      const bf16_t* kp = k_pages + ((size_t)page * num_kv + kvh) * head_stride +
+      const bf16_t* kp = k_pages + (size_t)page * page_stride + (size_t)kvh * head_stride +
                          (size_t)((tile0 + off) & pmask) * head_size;
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) kf[kb][ks] = *(const bf16x8*)(kp + min(32 * ks + 8 * g, dlast));
@@ -1560,7 +1575,7 @@ attention_decode_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
       const int page = (g >> 1) ? pg[2 * st + 1] : pg[2 * st];
-      const bf16_t* vp = v_pages + ((size_t)page * num_kv + kvh) * head_stride + ((tile0 + 32 * st + 8 * g) & pmask);
+      const bf16_t* vp = v_pages + (size_t)page * page_stride + (size_t)kvh * head_stride + ((tile0 + 32 * st + 8 * g) & pmask);
 #pragma unroll
       for (int db = 0; db < NDB; ++db)
         vf[db][st] = *(const bf16x8*)(vp + (size_t)min(16 * db + r, head_size - 1) * page_size);
@@ -1748,8 +1763,9 @@ static int attention_decode_run(const void* q, const void* k_pages, const void* 
                                 const int* cached_lens, const int* table, int table_width, int page_size,
                                 int num_pages, const int* decode_runs, int num_decode, void* out, float* part_o,
                                 float* part_ml, int num_heads, int num_kv, int head_size, int window,
-                                int num_splits, int waves, const int* longest, hipStream_t stream) {
+                                int num_splits, int waves, const int* longest, int page_pad, hipStream_t stream) {
   TNX_REQUIRE(num_heads > 0 && num_kv > 0 && num_heads % num_kv == 0, "attention_decode: bad head counts");
+  TNX_REQUIRE(page_pad >= 0 && page_pad % 8 == 0, "attention_decode: bad distance between pages");
   TNX_REQUIRE(head_size % 16 == 0 && head_size >= 16 && head_size <= 256,
               "attention_decode: head size %d is not a multiple of 16 in [16, 256]", head_size);
   TNX_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0,
@@ -1770,7 +1786,7 @@ static int attention_decode_run(const void* q, const void* k_pages, const void* 
 #define MFMA_ARGS                                                                                                 \
   (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, table_width,    \
       page_shift, num_pages, decode_runs, (bf16_t*)out, part_o, part_ml, num_heads, num_kv, window, num_splits,    \
-      longest, head_size
+      longest, head_size, page_pad
 #define LAUNCH_MFMA(NDB)                                                                         \
   if (waves == 8 && pack)                                                                        \
     attention_decode_mfma_kernel<NDB, 8, true><<<grid, 512, 0, stream>>>(MFMA_ARGS);             \
@@ -1809,10 +1825,11 @@ extern "C" int tnx_attention_decode(const void* q, const void* k_pages, const vo
                                     const int* cached_lens, const int* table, int table_width, int page_size,
                                     int num_pages, const int* decode_runs, int num_decode, void* out, float* part_o,
                                     float* part_ml, int num_heads, int num_kv, int head_size, int window,
-                                    int num_splits, int waves, const int* longest, hipStream_t stream) {
+                                    int num_splits, int waves, const int* longest, int page_pad,
+                                    hipStream_t stream) {
   return attention_decode_run(q, k_pages, v_pages, run_start, cached_lens, table, table_width, page_size, num_pages,
                               decode_runs, num_decode, out, part_o, part_ml, num_heads, num_kv, head_size, window,
-                              num_splits, waves, longest, stream);
+                              num_splits, waves, longest, page_pad, stream);
 }
 
 // The partial results of split keys for callers that cannot allocate: one array per GPU, held until the
@@ -1862,5 +1879,5 @@ extern "C" int tnx_attention_decode_static(const void* q, const void* k_pages, c
   float* part_ml = scratch + partials * head_size;
   return attention_decode_run(q, k_pages, v_pages, run_start, cached_lens, table, table_width, page_size, num_pages,
                               decode_runs, num_decode, out, part_o, part_ml, num_heads, num_kv, head_size, window,
-                              num_splits, waves, longest, stream);
+                              num_splits, waves, longest, 0, stream);       // (pages that lie one behind the other)
 }

@@ -35,6 +35,7 @@ struct QkvScatter {
   bf16_t* v_pages;
   float scale;
   int nq, nk, head_size, num_kv, page_size, num_pages;
+  int page_pad;          // elements between the end of one page and the start of the next
   const float* turn_a;
   const float* turn_b;
   const int* positions;
@@ -58,11 +59,12 @@ __device__ __forceinline__ void qkv_store(float v, float beside, int m, int n, c
   const bool is_key = j < sc.nk;
   if (!is_key) j -= sc.nk;
   const int h = j / sc.head_size, d = j - h * sc.head_size;
-  const size_t head = (size_t)page * sc.num_kv + h;
+  const size_t head_elems = (size_t)sc.page_size * sc.head_size;
+  const size_t head = (size_t)page * ((size_t)sc.num_kv * head_elems + sc.page_pad) + (size_t)h * head_elems;
   if (is_key)
-    sc.k_pages[(head * sc.page_size + off) * sc.head_size + d] = (bf16_t)v;
+    sc.k_pages[head + (size_t)off * sc.head_size + d] = (bf16_t)v;
   else
-    sc.v_pages[(head * sc.head_size + d) * sc.page_size + off] = (bf16_t)v;
+    sc.v_pages[head + (size_t)d * sc.page_size + off] = (bf16_t)v;
 }
 
 // ------------------------------------------------------------------------------------------ float32
@@ -938,7 +940,10 @@ extern "C" int tnx_gemm_bf16(const void* x, const void* w, const void* w_tiles, 
 // The fused projection of queries, keys and values: `x w^T + bias` with w = [Wq; Wk; Wv] stacked by rows,
 // queries scaled and written densely, keys and values written straight into their cache pages.
 // What both forms of the fused projection check and fill in of the pair-turning tables.
-static int qkv_turn(QkvScatter& sc, const float* turn_a, const float* turn_b, const int* positions, int turn_rows) {
+static int qkv_turn(QkvScatter& sc, const float* turn_a, const float* turn_b, const int* positions, int turn_rows,
+                    int page_pad) {
+  TNX_REQUIRE(page_pad >= 0 && page_pad % 8 == 0, "gemm_bf16_qkv: bad distance between pages");
+  sc.page_pad = page_pad;
   TNX_REQUIRE((turn_a == nullptr) == (turn_b == nullptr), "gemm_bf16_qkv: the pair-turning tables come both or not at all");
   TNX_REQUIRE(!turn_a || (positions && turn_rows > 0 && sc.head_size % 2 == 0),
               "gemm_bf16_qkv: pair-turning tables need the tokens' positions, rows, and an even head size");
@@ -954,7 +959,7 @@ extern "C" int tnx_gemm_bf16_qkv(const void* x, const void* w, const void* w_til
                                  const int* token_off, void* q_out, void* k_pages, void* v_pages, float scale,
                                  int num_heads, int num_kv, int head_size, int page_size, int num_pages,
                                  int force_tiled, const float* turn_a, const float* turn_b, const int* positions,
-                                 int turn_rows, hipStream_t stream) {
+                                 int turn_rows, int page_pad, hipStream_t stream) {
   TNX_REQUIRE(num_heads > 0 && num_kv >= 0 && head_size > 0 && page_size > 0, "gemm_bf16_qkv: bad sizes");
   QkvScatter sc;
   sc.token_page = token_page;
@@ -969,7 +974,7 @@ extern "C" int tnx_gemm_bf16_qkv(const void* x, const void* w, const void* w_til
   sc.num_kv = num_kv;
   sc.page_size = page_size;
   sc.num_pages = num_pages;
-  if (int rc = qkv_turn(sc, turn_a, turn_b, positions, turn_rows)) return rc;
+  if (int rc = qkv_turn(sc, turn_a, turn_b, positions, turn_rows, page_pad)) return rc;
   const int N = sc.nq + 2 * sc.nk;
   return gemm_bf16_dispatch(x, w, w_tiles, bias, nullptr, nullptr, TNX_BF16, TNX_ACT_NONE, M, N, K, force_tiled, &sc,
                             stream);
@@ -990,7 +995,7 @@ extern "C" int tnx_gemm_bf16_qkv_normed(const float* x, const void* w_folded, co
                                         const int* token_page, const int* token_off, void* q_out, void* k_pages,
                                         void* v_pages, float scale, int num_heads, int num_kv, int head_size,
                                         int page_size, int num_pages, int force_tiled, const float* turn_a,
-                                        const float* turn_b, const int* positions, int turn_rows,
+                                        const float* turn_b, const int* positions, int turn_rows, int page_pad,
                                         hipStream_t stream) {
   TNX_REQUIRE(num_heads > 0 && num_kv >= 0 && head_size > 0 && page_size > 0, "gemm_bf16_qkv: bad sizes");
   QkvScatter sc;
@@ -1006,7 +1011,7 @@ extern "C" int tnx_gemm_bf16_qkv_normed(const float* x, const void* w_folded, co
   sc.num_kv = num_kv;
   sc.page_size = page_size;
   sc.num_pages = num_pages;
-  if (int rc = qkv_turn(sc, turn_a, turn_b, positions, turn_rows)) return rc;
+  if (int rc = qkv_turn(sc, turn_a, turn_b, positions, turn_rows, page_pad)) return rc;
   const int N = sc.nq + 2 * sc.nk;
   const NormFold nf{x, fold_c, fold_d, eps};
   return gemm_bf16_dispatch(nullptr, nullptr, w_folded, bias, nullptr, nullptr, TNX_BF16, TNX_ACT_NONE, M, N, K,

@@ -66,7 +66,8 @@ def build_runner(model_config, source, cfg: EngineConfig) -> ModelRunner:
     model = DecoderModel(arch.build_spec(model_config))
     ops = make_ops(cfg.kernels, cfg.dtype, device)
     needs = model.cache_needs()
-    bytes_per_page = CacheManager.bytes_per_page(needs, cfg.page_size, cfg.dtype)
+    pad = cfg.page_pad_bytes if device.type == "cuda" else 0
+    bytes_per_page = CacheManager.bytes_per_page(needs, cfg.page_size, cfg.dtype, pad)
     if hasattr(ops, "decode_copies"):
         ops.decode_copies = _room_for_weight_copies(cfg, model, bytes_per_page, device)
     later = getattr(ops, "decode_copies", None) == "later"
@@ -85,7 +86,7 @@ def build_runner(model_config, source, cfg: EngineConfig) -> ModelRunner:
         model.finish_load()
         torch.cuda.empty_cache()
     num_pages = size_page_pool(cfg, bytes_per_page, device)
-    cache = CacheManager(needs, cfg.page_size, num_pages, cfg.max_num_seqs, cfg.dtype, device)
+    cache = CacheManager(needs, cfg.page_size, num_pages, cfg.max_num_seqs, cfg.dtype, device, page_pad_bytes=pad)
     return ModelRunner(model, cache, ops, use_graphs=cfg.use_graphs)
 
 

@@ -40,7 +40,7 @@ _SIGNATURES = {
                           _c_int, _c_int, _c_int, _c_void_p],
         "tnx_gemm_bf16_qkv": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
                               _c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int,
-                              _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p],
+                              _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
         "tnx_gemm_skinny_tiles_per_block": [_c_int, _c_int],
         "tnx_gemm_bf16_mid": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                               _c_int, _c_void_p, ctypes.c_size_t, _c_int, _c_int, _c_void_p],
@@ -50,20 +50,22 @@ _SIGNATURES = {
                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_gemm_bf16_qkv_normed": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int,
                                      _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int,
-                                     _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p],
+                                     _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
+                                     _c_void_p],
     },
     "attention": {
         "tnx_qkv_write": [_c_void_p, _c_int, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                           _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p,
-                          _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p],
+                          _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int,
+                          _c_void_p],
         "tnx_attention_any": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
-                              _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                              _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_attention_prefill": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                   _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
-                                  _c_int, _c_int, _c_void_p],
+                                  _c_int, _c_int, _c_int, _c_void_p],
         "tnx_attention_decode": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                  _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
-                                 _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
+                                 _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_void_p],
         "tnx_attention_decode_static": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                                         _c_int, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                                         _c_int, _c_int, _c_void_p, _c_void_p],
@@ -647,16 +649,26 @@ class HipOps:
     # ---------------------------------------------------------------- attention
 
     def _check_pages(self, k_pages, v_pages, num_kv, head_size, page_size):
-        _want(k_pages, "key pages", self.dtype)
-        _want(v_pages, "value pages", self.dtype)
+        """The number of pages. A page's own elements lie together; from page to page there may be more than a
+        page's elements, the same for keys and values (`_page_pad`: how many more)."""
         n = k_pages.shape[0]
-        if tuple(k_pages.shape) != (n, num_kv, page_size, head_size):
-            raise ValueError(f"key pages have shape {tuple(k_pages.shape)}, expected "
-                             f"{(n, num_kv, page_size, head_size)}")
-        if tuple(v_pages.shape) != (n, num_kv, head_size, page_size):
-            raise ValueError(f"value pages have shape {tuple(v_pages.shape)}, expected "
-                             f"{(n, num_kv, head_size, page_size)}")
+        for t, name, shape in ((k_pages, "key pages", (n, num_kv, page_size, head_size)),
+                               (v_pages, "value pages", (n, num_kv, head_size, page_size))):
+            if not t.is_cuda or t.dtype != self.dtype:
+                raise TypeError(f"{name} must be {self.dtype} on the GPU, got {t.dtype} on {t.device}")
+            if tuple(t.shape) != shape:
+                raise ValueError(f"{name} have shape {tuple(t.shape)}, expected {shape}")
+            inner = (shape[2] * shape[3], shape[3], 1)
+            if tuple(t.stride()[1:]) != inner or t.stride(0) < num_kv * inner[0] or (t.stride(0) - num_kv * inner[0]) % 8:
+                raise ValueError(f"{name} must hold each page's elements together, pages a multiple of 8 elements "
+                                 f"apart; strides {tuple(t.stride())}")
+        if k_pages.stride(0) != v_pages.stride(0):
+            raise ValueError("key and value pages must lie equally far apart")
         return n
+
+    @staticmethod
+    def _page_pad(pages, num_kv, head_size, page_size) -> int:
+        return int(pages.stride(0) - num_kv * head_size * page_size) if pages is not None else 0
 
     @staticmethod
     def _turn_args(turn, head_size, ctx):
@@ -707,7 +719,8 @@ class HipOps:
                            _ptr(view.token_offset), _ptr(q), _ptr(k_pages) if num_kv_write else None,
                            _ptr(v_pages) if num_kv_write else None, float(scale), num_heads, num_kv_write, head_size,
                            view.page_size, num_pages, int(force_tiled), _ptr(turn_a), _ptr(turn_b), _ptr(turn_pos),
-                           turn_rows, _stream())
+                           turn_rows, self._page_pad(k_pages if num_kv_write else None, num_kv_write, head_size,
+                                                     view.page_size), _stream())
                 return q
         tiles = None
         if isinstance(w, PreparedWeight):
@@ -740,7 +753,8 @@ class HipOps:
                    _ptr(view.token_page), _ptr(view.token_offset), _ptr(q),
                    _ptr(k_pages) if num_kv_write else None, _ptr(v_pages) if num_kv_write else None, float(scale),
                    num_heads, num_kv_write, head_size, view.page_size, num_pages, int(force_tiled), _ptr(turn_a),
-                   _ptr(turn_b), _ptr(turn_pos), turn_rows, _stream())
+                   _ptr(turn_b), _ptr(turn_pos), turn_rows,
+                   self._page_pad(k_pages if num_kv_write else None, num_kv_write, head_size, view.page_size), _stream())
         return q
 
     def qkv_write(self, qkv, bias, num_heads, num_kv_write, head_size, scale, ctx, view, k_pages, v_pages, turn=None):
@@ -764,7 +778,7 @@ class HipOps:
                    _ptr(v_pages) if num_kv_write else None, t, num_heads, num_kv_write, head_size,
                    _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(ctx.plan["tile_run"]), _ptr(ctx.plan["tile_start"]),
                    ctx.plan["tile_run"].numel() if by_tiles else 0, QUERY_TILE, _ptr(turn_a), _ptr(turn_b), turn_rows,
-                   _stream())
+                   self._page_pad(k_pages if num_kv_write else None, num_kv_write, head_size, view.page_size), _stream())
         return q
 
     def attention(self, q, num_heads, num_kv_heads, head_size, ctx, view, k_pages, v_pages, window=None):
@@ -776,6 +790,7 @@ class HipOps:
             raise ValueError("a request is longer than its block table")
         out = torch.empty_like(q)
         window = int(window or 0)
+        pad = self._page_pad(k_pages, num_kv_heads, head_size, view.page_size)
         fast = (self.dtype == torch.bfloat16 and not self.force_plain_attention
                 and (ctx.plan["decode_runs"].numel() == 0
                      or view.page_size & (view.page_size - 1) == 0))
@@ -787,14 +802,15 @@ class HipOps:
         if not fast:
             self._call("attention", "tnx_attention_any", _ptr(q), _code(self.dtype), _ptr(k_pages), _ptr(v_pages),
                        _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width,
-                       view.page_size, num_pages, _ptr(out), t, num_heads, num_kv_heads, head_size, window, _stream())
+                       view.page_size, num_pages, _ptr(out), t, num_heads, num_kv_heads, head_size, window, pad,
+                       _stream())
             return out
         if ctx.plan["tile_run"].numel():
             self._call("attention", "tnx_attention_prefill", _ptr(q), _ptr(k_pages), _ptr(v_pages),
                        _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(view.block_table), view.width,
                        view.page_size, num_pages, _ptr(ctx.plan["tile_run"]), _ptr(ctx.plan["tile_start"]), ctx.plan["tile_run"].numel(),
                        _ptr(out), num_heads, num_kv_heads, head_size, window,
-                       int(self.prefill_direct) or self._prefill_sets(ctx, num_heads, window), QUERY_TILE,
+                       int(self.prefill_direct) or self._prefill_sets(ctx, num_heads, window), QUERY_TILE, pad,
                        _stream())
         n_dec = ctx.plan["decode_runs"].numel()
         if n_dec:
@@ -808,7 +824,7 @@ class HipOps:
                        _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(view.block_table), view.width,
                        view.page_size, num_pages, _ptr(ctx.plan["decode_runs"]), n_dec, _ptr(out), _ptr(part_o),
                        _ptr(part_ml), num_heads, num_kv_heads, head_size, window, splits, waves,
-                       _ptr(ctx.plan["longest_decode"]),
+                       _ptr(ctx.plan["longest_decode"]), pad,
                        _stream())
         return out
 
