@@ -122,7 +122,7 @@ class Bench:
     """One model on the device and the measurements over it."""
 
     def __init__(self, raw, dtype_name, max_batch, context, layers=None, layers_key="num_hidden_layers", storage=None,
-                 max_tokens=None):
+                 max_tokens=None, step_tokens=PREFILL_TOKENS):
         import torch
         from transformers_neuronx_amd.config import EngineConfig
         from transformers_neuronx_amd.config.registry import resolve
@@ -138,7 +138,7 @@ class Bench:
         self.dtype = torch.bfloat16 if dtype_name == "bf16" else torch.float32
         self.context = context
         self.ecfg = EngineConfig(dtype=self.dtype, page_size=64, max_tokens=max_tokens or max_batch * context,
-                                 max_num_seqs=max_batch, max_num_batched_tokens=max(2048, PREFILL_TOKENS),
+                                 max_num_seqs=max_batch, max_num_batched_tokens=max(2048, step_tokens),
                                  max_model_len=context, prompts_first=True)
         t0 = time.time()
         self.runner = runner_from_random(self.cfg, seed=0, cfg=self.ecfg, storage=storage)
@@ -255,8 +255,12 @@ def room_for(raw, args, context, torch):
     weights = sum(item * int(torch.Size(d.shape).numel()) for d in model.param_decls() if d.tied_to is None)
     # (the random weights are drawn apart and fused afterwards: a quarter of them is held twice meanwhile, and
     # what that leaves free again is in pieces too small for the cache's blocks)
-    room = int(0.95 * torch.cuda.mem_get_info()[1]) - int(1.27 * weights) - (4 << 30)
-    return max(1, int(room // (model.cache_bytes_read(1, dtype) * context)))
+    per_request = model.cache_bytes_read(1, dtype) * context
+    total = int(0.95 * torch.cuda.mem_get_info()[1]) - (4 << 30)
+    # beside the weights and their tile-ordered copies, which decoding at small batches reads; where not even
+    # eight requests fit beside both (the largest models), beside the weights alone
+    beside_copies = int((total - 2.3 * weights) // per_request)
+    return max(1, beside_copies if beside_copies >= 8 else int((total - 1.27 * weights) // per_request))
 
 
 def flat_config(cfg, extra):
@@ -291,7 +295,8 @@ def main():
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the measurements at other models' sizes (the OPT-350m mix, OPT-66B) and the full-depth check")
     ap.add_argument("--prefill-only", action="store_true", help="measure the prompt step alone (for profiles)")
-    ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS)
+    ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
+                    help="the length of the prompt that is taken in one step (2,048; with --context up to that)")
     ap.add_argument("--model", default="6.7b",
                     help="a name of " + ", ".join(PRESETS) + " (OPT-6.7B is the measurement of record), a model "
                          "folder or a config.json file of any registered architecture; weights are random")
@@ -339,7 +344,10 @@ def main():
     max_batch = args.batch if only else max(args.batch, big)
     if args.mix:
         max_batch = 64
-    bench = Bench(raw, args.dtype, max_batch, context, args.layers, args.layers_key)
+    if tokens > context:
+        print(f"bench.py: a prompt of {tokens} tokens is longer than the context of {context}")
+        return 2
+    bench = Bench(raw, args.dtype, max_batch, context, args.layers, args.layers_key, step_tokens=tokens)
     cfg = bench.cfg
 
     if args.mix:
