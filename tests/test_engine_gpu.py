@@ -204,6 +204,38 @@ def test_toy_routed_parts_on_the_gpu(dtype):
     run_toy_routed_model("hip", dtype, DEV, 2e-5 if dtype == torch.float32 else 3e-2)
 
 
+def test_a_norm_that_only_scales_folded_into_the_products():
+    """A model of the tests whose norms only scale (no mean, no bias) and ask the backend to fold them into the
+    products that read them: decode steps of few rows run norm and product in one launch, recorded, and the
+    logits are the plain implementation's."""
+    import toy_parts
+    from transformers_neuronx_amd.cache import CacheManager
+    from transformers_neuronx_amd.engine import DecoderModel, ModelRunner, StepEntry
+    from transformers_neuronx_amd.kernels import make_ops
+    from transformers_neuronx_amd.kernels.hip import DeferredNorm
+    from transformers_neuronx_amd.weights import TensorDict, random_tensors
+    kw = dict(width=128, heads=4, kv_heads=2)
+    spec = toy_parts.toy_spec_rotating(inner=256, vocab=160, tables=True, latent_layer=False, fold=True, **kw)
+    model = DecoderModel(spec)
+    tensors = random_tensors(model.param_decls(), spec.init_std, 4, torch.bfloat16)
+    ops = make_ops("hip", torch.bfloat16, DEV)
+    model.load(TensorDict(tensors), ops, torch.bfloat16, DEV)
+    block = model.layers[0].block
+    assert block.fold_mixer_norm and block.fold_feed_forward_norm
+    assert isinstance(model.layers[0].mixer_norm.deferred(torch.zeros(2, 128, device=DEV)), DeferredNorm)
+    runner = ModelRunner(model, CacheManager(model.cache_needs(), 16, 24, 4, torch.bfloat16, DEV), ops, use_graphs=True)
+    requests = _requests(dict(vocab_size=160), [60, 33, 90], 10)
+    expected = {rid: toy_parts.toy_rotating_plain_logits(tensors, toks, latent_layer=False, **kw) for rid, toks in requests.items()}
+    ids = list(requests)
+    runner.step([StepEntry(rid, requests[rid][:20], []) for rid in ids])
+    for pos in range(20, 33):
+        logits = runner.step([StepEntry(rid, [requests[rid][pos]], [0]) for rid in ids]).float().cpu()
+        for i, rid in enumerate(ids):
+            want = expected[rid][pos]
+            assert float((logits[i] - want).abs().max() / want.abs().max()) < 3e-2, (rid, pos)
+    assert runner.graph_replays == 13
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_toy_rotating_parts_on_the_gpu(dtype):
     """Queries and keys turned by an encoding of the tests, and a norm whose HIP kernel lives under tests/

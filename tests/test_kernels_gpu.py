@@ -772,6 +772,34 @@ def test_product_of_normalised_rows_with_elements_far_from_the_rest(m, n, k):
         assert float((got.float() - want).abs().max()) <= 2e-2 * scale, (places, common)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 256, 1024), (8, 4096, 4096), (16, 512, 2048), (30, 1024, 512)])
+def test_product_after_a_norm_that_only_scales(m, n, k):
+    """`center=False`: x / sqrt(mean(x^2) + eps) * weight, alone and folded into the product of few rows and into
+    the fused projection's: the mean stays in the rows (here it is as large as their spread)."""
+    hip, ref = _ops(torch.bfloat16)
+    g = torch.Generator(device=DEV).manual_seed(m + n + k)
+    x = torch.randn(m, k, device=DEV, generator=g) * 2 + 1.5
+    gamma = 1 + 0.2 * torch.randn(k, device=DEV, generator=g)
+    w = (torch.randn(n, k, device=DEV, generator=g) / k ** 0.5).to(torch.bfloat16)
+    bias = torch.randn(n, device=DEV, generator=g) * 0.2
+    exact = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-3) * gamma
+    f_h, c_h = hip.layernorm(x, gamma, None, 1e-3, torch.bfloat16, True, True, center=False)
+    torch.testing.assert_close(f_h, exact, rtol=2e-5, atol=2e-5)
+    torch.testing.assert_close(c_h.float(), exact, rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(ref.layernorm(x, gamma, None, 1e-3, torch.float32, True, False, center=False)[0], exact,
+                               rtol=1e-5, atol=1e-5)
+    want = exact @ w.float().T + bias
+    pw = hip.prepare_weight(w)
+    assert hip.fold_norm(pw, gamma, None, center=False)
+    got = hip.linear(hip.layernorm_deferred(x, gamma, None, 1e-3, torch.bfloat16, center=False), pw, bias)
+    assert float((got.float() - want).abs().max()) <= 2e-2 * float(want.abs().max())
+    # a norm with a mean folded into the same matrix would be another norm: the deferred rows of one do not
+    # meet the folded copy of the other, and are normalised by their own kernel
+    other = hip.linear(hip.layernorm_deferred(x, gamma, None, 1e-3, torch.bfloat16, center=True), pw, bias)
+    centred = torch.nn.functional.layer_norm(x, (k,), gamma, None, 1e-3) @ w.float().T + bias
+    assert float((other.float() - centred).abs().max()) <= 2e-2 * float(centred.abs().max())
+
+
 def test_product_of_normalised_rows_without_weight_and_bias():
     hip, _ = _ops(torch.bfloat16)
     g = torch.Generator(device=DEV).manual_seed(3)

@@ -299,11 +299,20 @@ class ToyScaleNorm(Norm):
 
     recordable = True
 
-    def __init__(self, width: int, eps: float):
-        self.width, self.eps = width, eps
+    def __init__(self, width: int, eps: float, fold: bool = False):
+        """`fold`: where a matrix product alone reads this norm, let the backend fold it into that product (its
+        `fold_norm` / `layernorm_deferred` with `center=False`, the norm that only scales) instead of running the
+        kernel this part brings."""
+        self.width, self.eps, self.fold = width, eps, fold
 
     def param_decls(self, prefix):
         return [ParamDecl(prefix + ".weight", (self.width,), "vector", "around_one")]
+
+    def fold_into(self, w):
+        return self.fold and self.ops.fold_norm(w, self.weight, None, center=False)
+
+    def deferred(self, x):
+        return self.ops.layernorm_deferred(x, self.weight, None, self.eps, self.dtype, center=False)
 
     def load(self, tensors, prefix, ops, dtype):
         super().load(tensors, prefix, ops, dtype)
@@ -366,12 +375,12 @@ class ToyLatentMixer(Mixer):
 
 
 def toy_spec_rotating(width=96, heads=3, kv_heads=1, inner=72, vocab=157, positions=150, eps=1e-3, base=100.0,
-                      tables=False, latent_layer=True):
+                      tables=False, latent_layer=True, fold=False):
     """Attention whose queries and keys are turned by their positions (no encoding at the input), grouped
     heads, between two such layers one whose mixer keeps a paged cache of another shape; a scale-only norm
     with its own kernel, names of its own for every tensor."""
     hs = width // heads
-    norm = PartSpec("toy_scale_norm", dict(width=width, eps=eps))
+    norm = PartSpec("toy_scale_norm", dict(width=width, eps=eps, fold=fold))
     mixer = PartSpec("attention", dict(width=width, num_heads=heads, head_size=hs, num_kv_heads=kv_heads, bias=False,
                                        names=("wq", "wk", "wv", "wo"),
                                        rotation=PartSpec("toy_rotation", dict(base=base, tables=tables, positions=positions))))

@@ -110,7 +110,7 @@ extern "C" int tnx_cast(const void* src, int src_dtype, void* dst, int dst_dtype
 template <int PER, bool AFFINE, bool F32_OUT, bool BF16_OUT>
 __global__ void __launch_bounds__(256)
 layernorm_kernel(const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ bias,
-                 float eps, float* __restrict__ out_f32, bf16_t* __restrict__ out_bf16, int width) {
+                 float eps, float* __restrict__ out_f32, bf16_t* __restrict__ out_bf16, int width, int center) {
   typedef __attribute__((ext_vector_type(4))) float f4;
   typedef __attribute__((ext_vector_type(4))) __bf16 b4;
   __shared__ float scratch[4];
@@ -126,11 +126,12 @@ layernorm_kernel(const float* __restrict__ x, const float* __restrict__ weight, 
     v[j] = ok ? row[i] : (f4){0.f, 0.f, 0.f, 0.f};
     if (AFFINE) {
       gw[j] = ok ? ((const f4*)weight)[i] : (f4){0.f, 0.f, 0.f, 0.f};
-      gb[j] = ok ? ((const f4*)bias)[i] : (f4){0.f, 0.f, 0.f, 0.f};
+      gb[j] = ok && bias ? ((const f4*)bias)[i] : (f4){0.f, 0.f, 0.f, 0.f};
     }
     s += (v[j].x + v[j].y) + (v[j].z + v[j].w);
   }
-  const float mean = block_sum<4>(s, scratch) / (float)width;
+  // (`center` 0: a norm that only scales, by the root of the mean square: the mean stays where it is)
+  const float mean = center ? block_sum<4>(s, scratch) / (float)width : 0.f;
   float q = 0.f;
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
@@ -160,13 +161,14 @@ layernorm_kernel(const float* __restrict__ x, const float* __restrict__ weight, 
 // Any width: three passes over the row in memory.
 __global__ void __launch_bounds__(256)
 layernorm_wide_kernel(const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ bias,
-                      float eps, float* __restrict__ out_f32, void* __restrict__ out_cd, int cd_dtype, int width) {
+                      float eps, float* __restrict__ out_f32, void* __restrict__ out_cd, int cd_dtype, int width,
+                      int center) {
   __shared__ float scratch[4];
   const int t = blockIdx.x;
   const float* row = x + (size_t)t * width;
   float s = 0.f;
   for (int i = threadIdx.x; i < width; i += 256) s += row[i];
-  const float mean = block_sum<4>(s, scratch) / (float)width;
+  const float mean = center ? block_sum<4>(s, scratch) / (float)width : 0.f;
   float q = 0.f;
   for (int i = threadIdx.x; i < width; i += 256) {
     const float d = row[i] - mean;
@@ -183,19 +185,21 @@ layernorm_wide_kernel(const float* __restrict__ x, const float* __restrict__ wei
   }
 }
 
+// `center` 1: y = (x - mean) / sqrt(var + eps) * weight + bias, the variance about the mean; 0: the same with the
+// mean taken as 0, that is x / sqrt(mean(x^2) + eps) * weight + bias. Weight and bias are each optional.
 extern "C" int tnx_layernorm(const float* x, const float* weight, const float* bias, float eps, float* out_f32,
-                             void* out_cd, int cd_dtype, int tokens, int width, hipStream_t stream) {
+                             void* out_cd, int cd_dtype, int tokens, int width, int center, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && width > 0, "layernorm: bad sizes tokens=%d width=%d", tokens, width);
   TNX_REQUIRE(eps > 0.f, "layernorm: eps must be positive");
   if (tokens == 0) return 0;
   TNX_REQUIRE(out_f32 != x, "layernorm: the float32 output may not alias the input");
   const bool affine = weight != nullptr;
-  TNX_REQUIRE((weight != nullptr) == (bias != nullptr), "layernorm: weight and bias come together or not at all");
+  TNX_REQUIRE(weight != nullptr || bias == nullptr, "layernorm: a bias comes with a weight");
   const bool vec = width % 4 == 0 && width <= 1024 * 16 && (cd_dtype == TNX_BF16 || out_cd == nullptr);
   if (vec) {
     bf16_t* ob = (bf16_t*)out_cd;
 #define LN_LAUNCH(PER, AFF, F, B) \
-  layernorm_kernel<PER, AFF, F, B><<<tokens, 256, 0, stream>>>(x, weight, bias, eps, out_f32, ob, width)
+  layernorm_kernel<PER, AFF, F, B><<<tokens, 256, 0, stream>>>(x, weight, bias, eps, out_f32, ob, width, center)
 #define LN_OUTS(PER, AFF)                                  \
   if (out_f32 && ob) LN_LAUNCH(PER, AFF, true, true);      \
   else if (ob) LN_LAUNCH(PER, AFF, false, true);           \
@@ -209,7 +213,7 @@ extern "C" int tnx_layernorm(const float* x, const float* weight, const float* b
 #undef LN_OUTS
 #undef LN_LAUNCH
   } else {
-    layernorm_wide_kernel<<<tokens, 256, 0, stream>>>(x, weight, bias, eps, out_f32, out_cd, cd_dtype, width);
+    layernorm_wide_kernel<<<tokens, 256, 0, stream>>>(x, weight, bias, eps, out_f32, out_cd, cd_dtype, width, center);
   }
   TNX_CHECK_LAUNCH("layernorm");
   return 0;

@@ -577,6 +577,7 @@ struct NormFold {
   const float* c;      // [N]
   const float* d;      // [N]
   float eps;
+  int center;          // 0: a norm that only scales (the mean is taken as 0, and nothing is shifted before rounding)
 };
 
 template <int MT, int WAVES, bool QKV, bool SHUF, int RT, bool NORMED = false>
@@ -610,7 +611,7 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
     const size_t row = (size_t)min(t * 16 + r, M - 1) * K;
     xrow[t] = NORMED ? nullptr : x + row + 8 * g;
     xfrow[t] = NORMED ? nf.x + row + 8 * g : nullptr;
-    if (NORMED) {
+    if (NORMED && nf.center) {
       // the shift: the median of the medians of three times three elements spread over the row, which a few
       // elements far from the rest (at most one of each three, or all three of one) do not move away from it
       float med[3];
@@ -766,7 +767,7 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
         a1 += stat[wv][t][0][l & 15];
         a2 += stat[wv][t][1][l & 15];
       }
-      const float mean = a1 / (float)K;                       // of x - x0
+      const float mean = nf.center ? a1 / (float)K : 0.f;     // of x - x0
       const float var = fmaxf(a2 / (float)K - mean * mean, 0.f);
       const float rstd = rsqrtf(var + nf.eps);
       v = rstd * (v - mean * nf.c[n]) + nf.d[n];
@@ -984,8 +985,8 @@ extern "C" int tnx_gemm_bf16_qkv(const void* x, const void* w, const void* w_til
 // `w_folded` is W diag(gamma) in tile order, `fold_c` its row sums, `fold_d` W beta.
 extern "C" int tnx_gemm_bf16_normed(const float* x, const void* w_folded, const float* fold_c, const float* fold_d,
                                     float eps, const float* bias, void* out, int out_dtype, int act, int M, int N,
-                                    int K, int force_tiled, hipStream_t stream) {
-  const NormFold nf{x, fold_c, fold_d, eps};
+                                    int K, int force_tiled, int center, hipStream_t stream) {
+  const NormFold nf{x, fold_c, fold_d, eps, center};
   return gemm_bf16_dispatch(nullptr, nullptr, w_folded, bias, nullptr, out, out_dtype, act, M, N, K, force_tiled,
                             nullptr, stream, &nf);
 }
@@ -996,7 +997,7 @@ extern "C" int tnx_gemm_bf16_qkv_normed(const float* x, const void* w_folded, co
                                         void* v_pages, float scale, int num_heads, int num_kv, int head_size,
                                         int page_size, int num_pages, int force_tiled, const float* turn_a,
                                         const float* turn_b, const int* positions, int turn_rows, int page_pad,
-                                        hipStream_t stream) {
+                                        int center, hipStream_t stream) {
   TNX_REQUIRE(num_heads > 0 && num_kv >= 0 && head_size > 0 && page_size > 0, "gemm_bf16_qkv: bad sizes");
   QkvScatter sc;
   sc.token_page = token_page;
@@ -1013,7 +1014,7 @@ extern "C" int tnx_gemm_bf16_qkv_normed(const float* x, const void* w_folded, co
   sc.num_pages = num_pages;
   if (int rc = qkv_turn(sc, turn_a, turn_b, positions, turn_rows, page_pad)) return rc;
   const int N = sc.nq + 2 * sc.nk;
-  const NormFold nf{x, fold_c, fold_d, eps};
+  const NormFold nf{x, fold_c, fold_d, eps, center};
   return gemm_bf16_dispatch(nullptr, nullptr, w_folded, bias, nullptr, nullptr, TNX_BF16, TNX_ACT_NONE, M, N, K,
                             force_tiled, &sc, stream, &nf);
 }

@@ -31,7 +31,7 @@ _SIGNATURES = {
         "tnx_cast": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_void_p],
         "tnx_epilogue": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_layernorm": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
-                          _c_void_p],
+                          _c_int, _c_void_p],
     },
     "gemm": {
         "tnx_gemm_f32": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
@@ -47,11 +47,11 @@ _SIGNATURES = {
         "tnx_gemm_library": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                              _c_int, _c_void_p, ctypes.c_size_t, _c_void_p, ctypes.c_size_t, _c_int, _c_void_p],
         "tnx_gemm_bf16_normed": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_int,
-                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_gemm_bf16_qkv_normed": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int,
                                      _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_int,
                                      _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
-                                     _c_void_p],
+                                     _c_int, _c_void_p],
     },
     "attention": {
         "tnx_qkv_write": [_c_void_p, _c_int, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
@@ -143,10 +143,11 @@ class DeferredNorm:
     """The input of a LayerNorm whose output only a matrix product reads: the product of few rows applies the
     norm itself (`HipOps.linear`, `HipOps.qkv_project`); whoever else gets one calls `materialize()`."""
 
-    __slots__ = ("ops", "x", "weight", "bias", "eps", "dtype")
+    __slots__ = ("ops", "x", "weight", "bias", "eps", "dtype", "center")
 
-    def __init__(self, ops, x, weight, bias, eps, dtype):
+    def __init__(self, ops, x, weight, bias, eps, dtype, center=True):
         self.ops, self.x, self.weight, self.bias, self.eps, self.dtype = ops, x, weight, bias, eps, dtype
+        self.center = center
 
     @property
     def shape(self):
@@ -155,14 +156,14 @@ class DeferredNorm:
     @property
     def key(self):
         return (self.weight.data_ptr() if self.weight is not None else 0,
-                self.bias.data_ptr() if self.bias is not None else 0)
+                self.bias.data_ptr() if self.bias is not None else 0, bool(self.center))
 
     def materialize(self):
-        return self.ops.layernorm(self.x, self.weight, self.bias, self.eps, self.dtype, False, True)[1]
+        return self.ops.layernorm(self.x, self.weight, self.bias, self.eps, self.dtype, False, True, self.center)[1]
 
     def normalised(self):
         """`(x - mean) rstd` alone, for a product with a folded copy."""
-        return self.ops.layernorm(self.x, None, None, self.eps, self.dtype, False, True)[1]
+        return self.ops.layernorm(self.x, None, None, self.eps, self.dtype, False, True, self.center)[1]
 
 
 def tile_order(w: torch.Tensor) -> torch.Tensor:
@@ -365,7 +366,8 @@ class HipOps:
 
     # ---------------------------------------------------------------- norms
 
-    def layernorm(self, x, weight, bias, eps, dtype, want_f32, want_compute):
+    def layernorm(self, x, weight, bias, eps, dtype, want_f32, want_compute, center=True):
+        """`center=False`: the norm that only scales, x / sqrt(mean(x^2) + eps) (times weight, plus bias)."""
         _want(x, "x", torch.float32)
         t, width = x.shape
         if weight is not None:
@@ -376,7 +378,7 @@ class HipOps:
         out_f32 = torch.empty_like(x) if (want_f32 or (want_compute and same)) else None
         out_cd = torch.empty(t, width, dtype=dtype, device=x.device) if (want_compute and not same) else None
         self._call("elementwise", "tnx_layernorm", _ptr(x), _ptr(weight), _ptr(bias), float(eps), _ptr(out_f32),
-                   _ptr(out_cd), _code(dtype), t, width, _stream())
+                   _ptr(out_cd), _code(dtype), t, width, int(bool(center)), _stream())
         return (out_f32 if want_f32 else None), ((out_f32 if same else out_cd) if want_compute else None)
 
     # Steps of few rows: a LayerNorm that only a matrix product reads is done by that product (`fold_norm`,
@@ -399,7 +401,7 @@ class HipOps:
         return self._tiles_per_block[key] >= 2
     few_rows = 32           # the few-rows kernel takes up to this many rows
 
-    def fold_norm(self, w, weight, bias) -> bool:
+    def fold_norm(self, w, weight, bias, center=True) -> bool:
         """Called once when a layer has its tensors, for a matrix `w` that reads a LayerNorm's output and
         nothing else does: keeps, in the place of its tile-ordered copy, the copy with the norm's weight
         folded in and the two vectors that go with it (see `FoldedNorm`). False if this matrix has no such
@@ -411,17 +413,17 @@ class HipOps:
         scaled = (full * weight.float()[None, :] if weight is not None else full).to(torch.bfloat16)
         c = scaled.float().sum(dim=1).contiguous()
         d = (full @ bias.float() if bias is not None else torch.zeros_like(c)).contiguous()
-        key = (weight.data_ptr() if weight is not None else 0, bias.data_ptr() if bias is not None else 0)
+        key = (weight.data_ptr() if weight is not None else 0, bias.data_ptr() if bias is not None else 0, bool(center))
         w.folded = FoldedNorm(tile_order(scaled), c, d, key)
         w.tiles = None          # the few-rows steps read the folded copy; the memory stays what it was
         return True
 
-    def layernorm_deferred(self, x, weight, bias, eps, dtype):
+    def layernorm_deferred(self, x, weight, bias, eps, dtype, center=True):
         """The compute-dtype output of the norm, or, in steps of few rows, a `DeferredNorm`."""
         if self.fuse_norm and dtype == torch.bfloat16 and self.dtype == torch.bfloat16 \
                 and x.shape[0] <= self.few_rows and x.shape[1] % 128 == 0 and not debug.active():
-            return DeferredNorm(self, x, weight, bias, eps, dtype)
-        return self.layernorm(x, weight, bias, eps, dtype, False, True)[1]
+            return DeferredNorm(self, x, weight, bias, eps, dtype, center)
+        return self.layernorm(x, weight, bias, eps, dtype, False, True, center)[1]
 
     def _folded_for(self, h, w):
         """The folded copy of `w` that fits the deferred norm `h`, or None."""
@@ -492,7 +494,7 @@ class HipOps:
                 out = torch.empty(m, n, dtype=self.dtype, device=x.x.device)
                 self._call("gemm", "tnx_gemm_bf16_normed", _ptr(x.x), _ptr(folded.tiles), _ptr(folded.c),
                            _ptr(folded.d), float(x.eps), _ptr(bias), _ptr(out), _code(self.dtype), _ACT[act], m, n, k,
-                           int(force_tiled), _stream())
+                           int(force_tiled), int(bool(x.center)), _stream())
                 return out
         tiles = None
         if isinstance(w, PreparedWeight):
@@ -720,7 +722,7 @@ class HipOps:
                            _ptr(v_pages) if num_kv_write else None, float(scale), num_heads, num_kv_write, head_size,
                            view.page_size, num_pages, int(force_tiled), _ptr(turn_a), _ptr(turn_b), _ptr(turn_pos),
                            turn_rows, self._page_pad(k_pages if num_kv_write else None, num_kv_write, head_size,
-                                                     view.page_size), _stream())
+                                                     view.page_size), int(bool(h.center)), _stream())
                 return q
         tiles = None
         if isinstance(w, PreparedWeight):

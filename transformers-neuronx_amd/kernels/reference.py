@@ -61,9 +61,10 @@ class ReferenceOps:
 
     # ---------------------------------------------------------------- norms
 
-    def layernorm(self, x, weight, bias, eps, dtype, want_f32, want_compute):
+    def layernorm(self, x, weight, bias, eps, dtype, want_f32, want_compute, center=True):
+        """`center=False`: the norm that only scales, x / sqrt(mean(x^2) + eps) (times weight, plus bias)."""
         x = x.float()
-        mean = x.mean(-1, keepdim=True)
+        mean = x.mean(-1, keepdim=True) if center else torch.zeros_like(x[:, :1])
         var = ((x - mean) ** 2).mean(-1, keepdim=True)
         y = (x - mean) * torch.rsqrt(var + eps)
         if weight is not None:
@@ -74,12 +75,12 @@ class ReferenceOps:
 
     # ---------------------------------------------------------------- matrix products
 
-    def layernorm_deferred(self, x, weight, bias, eps, dtype):
+    def layernorm_deferred(self, x, weight, bias, eps, dtype, center=True):
         """The norm's output for a part that only multiplies it; a backend may hand back something a
         product resolves instead (`HipOps.layernorm_deferred`)."""
-        return self.layernorm(x, weight, bias, eps, dtype, False, True)[1]
+        return self.layernorm(x, weight, bias, eps, dtype, False, True, center)[1]
 
-    def fold_norm(self, w, weight, bias) -> bool:
+    def fold_norm(self, w, weight, bias, center=True) -> bool:
         return False
 
     def prepare_weight(self, w):
