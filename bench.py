@@ -210,6 +210,40 @@ class Bench:
             times.append(time.perf_counter() - start)
         return sorted(times[1:])[2], self.model.step_flops(tokens, (tokens + 1) / 2, 1)
 
+    def kernel_rates(self, batch, tokens):
+        """What the kernels of a decode step of `batch` requests at the full context, and of a prompt step of
+        `tokens` tokens, reach: {"<step> <entry point> <sizes> us": microseconds a launch, "... GB/s" or
+        "... TFLOP/s": the bytes the launch has to move, or its flops, over that time}, for the launches that say
+        what they move (products, attention) and take a hundredth of their step or more. The steps run with
+        events around every launch, unrecorded, so a launch stands alone; the kernels are the recorded step's."""
+        from transformers_neuronx_amd.sampling import SamplingParams
+        engine, out = self.engine, {}
+        for step, count, length in ((f"decode_b{batch}", batch, self.context - 5), (f"prefill_{tokens}", 1, tokens)):
+            engine.reset()
+            new = 4 if step.startswith("decode") else 1
+            for i in range(count):
+                engine.add_request(self.prompt(length), SamplingParams(max_new_tokens=new, do_sample=False, ignore_eos=True))
+            if step.startswith("decode"):
+                while any(not r.decoding for r in engine.requests.values()):
+                    engine.step()
+                engine.profile(1)                                    # once unmeasured: what is made at first use
+            else:
+                engine.profile(1)
+                engine.reset()
+                engine.add_request(self.prompt(length), SamplingParams(max_new_tokens=1, do_sample=False, ignore_eos=True))
+            table, _ = engine.profile(1, work=True)
+            whole = sum(row[1] for row in table.values())
+            for name, (calls, ms, nbytes, flops) in table.items():
+                if nbytes and ms >= 0.01 * whole:
+                    key = f"{step} {name.replace('tnx_', '')}"
+                    out[key + " us"] = round(1e3 * ms / calls, 1)
+                    if step.startswith("decode"):
+                        out[key + " GB/s"] = round(nbytes / ms / 1e6)
+                    else:
+                        out[key + " TFLOP/s"] = round(flops / ms / 1e9, 1)
+        engine.reset()
+        return out
+
     def mix(self, requests=64, new_tokens=256):
         """Every request is there at the start; the scheduler mixes portions of prompts with decoding. The
         workload runs twice with other tokens and the second run is timed: the first loads the vendor
@@ -416,6 +450,12 @@ def main():
             points[f"decode_b{b}_hbm_frac"] = round(rd / s / 1e9 / PEAK_HBM_GBS, 4)
             log(f"decode batch {b}: {v:.1f} tok/s, {s * 1e3:.2f} ms/step")
         out["points"] = points
+        if args.dtype == "bf16":
+            try:
+                out["kernels"] = bench.kernel_rates(args.batch, tokens)
+                log(f"kernels: {out['kernels']}")
+            except Exception as e:                                   # noqa: BLE001 (never at the cost of the line)
+                out["kernels"] = {"error": f"{type(e).__name__}: {e}"[:200]}
         if not args.no_extras and args.dtype == "bf16":
             extras(out, bench, raw, args, context)
     print(json.dumps(out))

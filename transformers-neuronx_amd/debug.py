@@ -23,6 +23,11 @@ def active() -> bool:
     return _tapped is not None or _timer is not None
 
 
+def tapping() -> bool:
+    """A debug context is open: every tapped place needs its tensor as such."""
+    return _tapped is not None
+
+
 def tap(name: str, tensor):
     """Keep a copy of `tensor` under `name` if a debug context is open; returns the tensor."""
     if _tapped is not None and tensor is not None:
@@ -46,25 +51,33 @@ def debug_context():
 
 
 class KernelTimer:
-    """Events around every launch; `table()` sums them by kernel name after a synchronize."""
+    """Events around every launch; `table()` sums them by kernel name after a synchronize. A launch may say what
+    it moves and computes (`bytes`, `flops`: what it has to read and write once, and its multiply-adds times
+    two); `work_table()` then gives the rates."""
 
     def __init__(self):
         self.spans: List[tuple] = []
 
-    def start(self, name: str):
+    def start(self, name: str, bytes: float = 0.0, flops: float = 0.0):
         begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         begin.record()
-        self.spans.append((name, begin, end))
+        self.spans.append((name, begin, end, float(bytes), float(flops)))
         return end
 
-    def table(self) -> Dict[str, tuple]:
+    def work_table(self) -> Dict[str, tuple]:
+        """{name: (calls, milliseconds, bytes, flops)} by falling time."""
         torch.cuda.synchronize()
         out: Dict[str, list] = {}
-        for name, begin, end in self.spans:
-            row = out.setdefault(name, [0, 0.0])
+        for name, begin, end, nbytes, flops in self.spans:
+            row = out.setdefault(name, [0, 0.0, 0.0, 0.0])
             row[0] += 1
             row[1] += begin.elapsed_time(end)
-        return {k: (v[0], v[1]) for k, v in sorted(out.items(), key=lambda kv: -kv[1][1])}
+            row[2] += nbytes
+            row[3] += flops
+        return {k: tuple(v) for k, v in sorted(out.items(), key=lambda kv: -kv[1][1])}
+
+    def table(self) -> Dict[str, tuple]:
+        return {k: (v[0], v[1]) for k, v in self.work_table().items()}
 
 
 def timer() -> Optional[KernelTimer]:

@@ -166,9 +166,11 @@ class LLMEngine:
         if idle and not self._planned and self.scheduler.has_work:
             raise RuntimeError("no progress: requests wait, the scheduler plans no step and none is under way")
 
-    def profile(self, steps: int = 1):
+    def profile(self, steps: int = 1, work: bool = False):
         """Run `steps` steps with events around every kernel launch (no recording, no running ahead) and
-        return ({kernel: (launches, milliseconds)}, the steps' outputs). Reference: `profile`, base.py:754-759."""
+        return ({kernel: (launches, milliseconds)}, the steps' outputs); with `work` the table's entries are
+        (launches, milliseconds, bytes, flops), with what the launches said they move and compute, and its
+        names carry their sizes. Reference: `profile`, base.py:754-759."""
         from .. import debug
         ahead, self.run_ahead = self.run_ahead, False
         outs: List[StepOutput] = []
@@ -178,7 +180,7 @@ class LLMEngine:
                     if not self.has_work:
                         break
                     outs += self.step()
-                table = t.table()
+                table = t.work_table() if work else t.table()
         finally:
             self.run_ahead = ahead
         return table, outs

@@ -235,10 +235,14 @@ class HipOps:
         self._landing, self._landing_turn = [None, None], 0
         self._ints, self._ints_done, self._ints_turn = [None, None], [None, None], 0
 
-    def _call(self, module: str, fn: str, *args):
+    def _call(self, module: str, fn: str, *args, work=None):
+        """`work` = (what, bytes, flops) names the launch for a kernel timer: what it is (its sizes), what it has
+        to read and write once, and its multiply-adds times two."""
         lib = library(module)
         timer = debug.timer()
-        end = timer.start(fn) if timer is not None else None
+        end = None
+        if timer is not None:
+            end = timer.start(fn, 0, 0) if work is None else timer.start(f"{fn} {work[0]}", work[1], work[2])
         rc = getattr(lib, fn)(*args)
         if end is not None:
             end.record()
@@ -252,6 +256,25 @@ class HipOps:
 
     stream = staticmethod(_stream)
     pointer = staticmethod(_ptr)
+
+    @staticmethod
+    def _product_work(m, n, k, item=2, x_item=2, out_item=2, residual=False):
+        """What a product out[m, n] = x[m, k] w[n, k]^T is for a kernel timer: its sizes, the bytes it has to move
+        (the matrix, the rows, the result, the residual) and its flops."""
+        return (f"{m}x{n}x{k}", n * k * item + m * k * x_item + m * n * (out_item + (4 if residual else 0)), 2.0 * m * n * k)
+
+    @staticmethod
+    def _attention_work(ctx, which, num_heads, num_kv_heads, head_size, window, item):
+        """The same for the attention of a step's decoding runs (`which` "decode": bytes of the keys and values
+        they read) or of its longer runs ("prompt": flops of scores and weighted values under the causal mask)."""
+        lens, cached = ctx.run_lens_host.astype(np.float64), ctx.cached_lens_host.astype(np.float64)
+        pick = lens == 1 if which == "decode" else lens > 1
+        seen = cached[pick] + (lens[pick] + 1) / 2                     # keys a query of the run sees on average
+        if window:
+            seen = np.minimum(seen, window)
+        keys = float((lens[pick] * seen).sum())
+        nbytes = float((np.minimum(cached[pick] + lens[pick], window or 1e18)).sum()) * 2 * num_kv_heads * head_size * item
+        return (f"{which} {int(pick.sum())} runs", nbytes, 4.0 * num_heads * head_size * keys)
 
     # ---------------------------------------------------------------- input end
 
@@ -421,7 +444,7 @@ class HipOps:
     def layernorm_deferred(self, x, weight, bias, eps, dtype, center=True):
         """The compute-dtype output of the norm, or, in steps of few rows, a `DeferredNorm`."""
         if self.fuse_norm and dtype == torch.bfloat16 and self.dtype == torch.bfloat16 \
-                and x.shape[0] <= self.few_rows and x.shape[1] % 128 == 0 and not debug.active():
+                and x.shape[0] <= self.few_rows and x.shape[1] % 128 == 0 and not debug.tapping():
             return DeferredNorm(self, x, weight, bias, eps, dtype, center)
         return self.layernorm(x, weight, bias, eps, dtype, False, True, center)[1]
 
@@ -482,7 +505,8 @@ class HipOps:
                 out = torch.empty(m, n, dtype=self.dtype, device=x.x.device)
                 rows, shift = x.normalised(), folded.d_with(bias)     # held until the launch is made
                 self._call("gemm", "tnx_gemm_bf16", _ptr(rows), _ptr(w.tensor), _ptr(folded.tiles), _ptr(shift), None,
-                           _ptr(out), _code(self.dtype), _ACT[act], m, n, k, int(force_tiled), _stream())
+                           _ptr(out), _code(self.dtype), _ACT[act], m, n, k, int(force_tiled), _stream(),
+                           work=self._product_work(m, n, k))
                 return out
             else:
                 if act not in _ACT:
@@ -494,7 +518,7 @@ class HipOps:
                 out = torch.empty(m, n, dtype=self.dtype, device=x.x.device)
                 self._call("gemm", "tnx_gemm_bf16_normed", _ptr(x.x), _ptr(folded.tiles), _ptr(folded.c),
                            _ptr(folded.d), float(x.eps), _ptr(bias), _ptr(out), _code(self.dtype), _ACT[act], m, n, k,
-                           int(force_tiled), int(bool(x.center)), _stream())
+                           int(force_tiled), int(bool(x.center)), _stream(), work=self._product_work(m, n, k, x_item=4))
                 return out
         tiles = None
         if isinstance(w, PreparedWeight):
@@ -520,7 +544,7 @@ class HipOps:
             space = self._library_workspace(x.device)
             self._call("gemm", "tnx_gemm_bf16_mid", _ptr(self.cast(x, torch.bfloat16)), _ptr(tiles), _ptr(bias),
                        _ptr(residual), _ptr(out), _code(out_dtype), _ACT[act], m, n, k, _ptr(space), space.numel() // 4,
-                       0, 0, _stream())
+                       0, 0, _stream(), work=self._product_work(m, n, k, out_item=4, residual=residual is not None))
             return out
         if (self._library_product(m, n, k, w, force_tiled) and (residual is not None or not out_f32)):
             # Many rows: the product goes to the vendor library (hipBLASLt), with what follows it where the
@@ -553,11 +577,13 @@ class HipOps:
         if w.dtype == torch.float32:
             xa = self.cast(x, torch.float32)
             self._call("gemm", "tnx_gemm_f32", _ptr(xa), _ptr(w), _ptr(bias), _ptr(residual), _ptr(out),
-                       _code(out_dtype), _ACT[act], m, n, k, _stream())
+                       _code(out_dtype), _ACT[act], m, n, k, _stream(),
+                       work=self._product_work(m, n, k, 4, 4, out.element_size(), residual is not None))
         else:
             xa = self.cast(x, torch.bfloat16)
             self._call("gemm", "tnx_gemm_bf16", _ptr(xa), _ptr(w), _ptr(tiles), _ptr(bias), _ptr(residual),
-                       _ptr(out), _code(out_dtype), _ACT[act], m, n, k, int(force_tiled), _stream())
+                       _ptr(out), _code(out_dtype), _ACT[act], m, n, k, int(force_tiled), _stream(),
+                       work=self._product_work(m, n, k, out_item=out.element_size(), residual=residual is not None))
         return out
 
     library_direct = True   # many-rows products as calls of the vendor library itself, with what follows them
@@ -574,7 +600,10 @@ class HipOps:
                                         _ACT[act], m, n, k, _ptr(space), space.numel(), _ptr(flush),
                                         flush.numel() if flush is not None else 0, int(tune), _stream())
         timer = debug.timer()
-        end = timer.start("tnx_gemm_library") if timer is not None else None
+        end = None
+        if timer is not None:
+            what, nbytes, flops = self._product_work(m, n, k, out_item=out.element_size(), residual=residual is not None)
+            end = timer.start(f"tnx_gemm_library {what}", nbytes, flops)
         rc = call(None, self.library_tune)
         if end is not None:
             end.record()
@@ -722,7 +751,8 @@ class HipOps:
                            _ptr(v_pages) if num_kv_write else None, float(scale), num_heads, num_kv_write, head_size,
                            view.page_size, num_pages, int(force_tiled), _ptr(turn_a), _ptr(turn_b), _ptr(turn_pos),
                            turn_rows, self._page_pad(k_pages if num_kv_write else None, num_kv_write, head_size,
-                                                     view.page_size), int(bool(h.center)), _stream())
+                                                     view.page_size), int(bool(h.center)), _stream(),
+                           work=self._product_work(t, total, h.x.shape[1], x_item=4))
                 return q
         tiles = None
         if isinstance(w, PreparedWeight):
@@ -756,7 +786,8 @@ class HipOps:
                    _ptr(k_pages) if num_kv_write else None, _ptr(v_pages) if num_kv_write else None, float(scale),
                    num_heads, num_kv_write, head_size, view.page_size, num_pages, int(force_tiled), _ptr(turn_a),
                    _ptr(turn_b), _ptr(turn_pos), turn_rows,
-                   self._page_pad(k_pages if num_kv_write else None, num_kv_write, head_size, view.page_size), _stream())
+                   self._page_pad(k_pages if num_kv_write else None, num_kv_write, head_size, view.page_size), _stream(),
+                   work=self._product_work(t, total, h.shape[1]))
         return q
 
     def qkv_write(self, qkv, bias, num_heads, num_kv_write, head_size, scale, ctx, view, k_pages, v_pages, turn=None):
@@ -813,7 +844,8 @@ class HipOps:
                        view.page_size, num_pages, _ptr(ctx.plan["tile_run"]), _ptr(ctx.plan["tile_start"]), ctx.plan["tile_run"].numel(),
                        _ptr(out), num_heads, num_kv_heads, head_size, window,
                        int(self.prefill_direct) or self._prefill_sets(ctx, num_heads, window), QUERY_TILE, pad,
-                       _stream())
+                       _stream(), work=self._attention_work(ctx, "prompt", num_heads, num_kv_heads, head_size, window, 2)
+                       if debug.timer() is not None else None)
         n_dec = ctx.plan["decode_runs"].numel()
         if n_dec:
             splits, waves = self._decode_splits(ctx, n_dec * self._decode_blocks(num_heads, num_kv_heads, head_size),
@@ -827,7 +859,8 @@ class HipOps:
                        view.page_size, num_pages, _ptr(ctx.plan["decode_runs"]), n_dec, _ptr(out), _ptr(part_o),
                        _ptr(part_ml), num_heads, num_kv_heads, head_size, window, splits, waves,
                        _ptr(ctx.plan["longest_decode"]), pad,
-                       _stream())
+                       _stream(), work=self._attention_work(ctx, "decode", num_heads, num_kv_heads, head_size, window, 2)
+                       if debug.timer() is not None else None)
         return out
 
     # What the choice between one and two sets of waves a block rests on: the time of one 64-key step of a

@@ -165,10 +165,11 @@ def run(args):
         for row in input_ids.tolist():
             engine.add_request(row, SamplingParams(max_new_tokens=3, do_sample=False, ignore_eos=True))
         for title in ("prompt step", "decode step"):
-            table, _ = engine.profile(1)
-            print(f"{title}: {sum(ms for _, ms in table.values()):.3f} ms in kernels")
-            for name, (calls, ms) in table.items():
-                print(f"  {name:32s} {calls:5d} launches {ms:9.3f} ms")
+            table, _ = engine.profile(1, work=True)
+            print(f"{title}: {sum(row[1] for row in table.values()):.3f} ms in kernels")
+            for name, (calls, ms, nbytes, flops) in table.items():
+                rates = f"  {nbytes / ms / 1e6:8.0f} GB/s {flops / ms / 1e9:8.1f} TFLOP/s" if nbytes and ms > 0 else ""
+                print(f"  {name:48s} {calls:5d} launches {ms:9.3f} ms{rates}")
         engine.reset()
 
 
