@@ -880,7 +880,7 @@ def test_product_of_some_rows(m, n, k):
     if m > 32:
         seen = []
         inner = hip._call
-        hip._call = lambda module, fn, *a: (seen.append(fn), inner(module, fn, *a))[1]
+        hip._call = lambda module, fn, *a, **kw: (seen.append(fn), inner(module, fn, *a, **kw))[1]
         got = hip.linear(x, pw, bias, residual=res, out_f32=True)
         assert seen == ["tnx_gemm_bf16_mid"]
         torch.testing.assert_close(got, exact + bias + res, rtol=1e-3, atol=1e-3)
@@ -902,9 +902,12 @@ def test_tiles_a_block_of_the_few_rows_product():
     assert [rule(8, n) for n in (15360, 5120, 20480)] == [2, 2, 1]                     # OPT-13B
     assert rule(16, 20480) == 3 and rule(16, 28672) == 2 and rule(8, 28672) == 1       # 16 rows read twice the `x`
     assert rule(24, 12288) <= 2 and rule(33, 12288) == 1 and rule(8, 288) == 1
-    # and the norm is done by the product only where a block takes two tiles or more
-    assert hip._norm_in_the_product(8, 12288) and not hip._norm_in_the_product(8, 27648)
-    assert not hip._norm_in_the_product(9, 12288)
+    # and the norm is done by the product only where a block takes two tiles or more and the blocks between
+    # them read 40 MB of float32 rows at most
+    assert hip._norm_in_the_product(8, 12288, 4096) and not hip._norm_in_the_product(8, 27648, 9216)
+    assert not hip._norm_in_the_product(9, 12288, 4096)
+    assert hip._norm_in_the_product(4, 16384, 4096) and not hip._norm_in_the_product(8, 16384, 4096)
+    assert hip._norm_in_the_product(1, 36864, 9216) and not hip._norm_in_the_product(2, 36864, 9216)
 
 
 def test_which_products_of_some_rows_go_to_our_kernel():

@@ -411,17 +411,24 @@ class HipOps:
     # the few-rows kernel goes, the norm's kernel normalises and the folded copy does the rest.
     # Where the blocks take one tile of weight rows each (what `tnx_gemm_skinny_tiles_per_block` says), every
     # 32 bytes of weight come with 64 of float32 rows and the norm's own kernel is the cheaper way again
-    # (9,216 -> 27,648 at 8 rows: 120 us against 10 + 91).
+    # (9,216 -> 27,648 at 8 rows: 120 us against 10 + 91). And where the blocks between them read more than
+    # `fuse_norm_bytes` of rows: 4,096 -> 16,384, 512 blocks of two tiles, is 0.3 to 0.6 us quicker with the norm
+    # inside up to 4 rows, as quick at 6 (50 MB of rows) and 0.8 us slower at 8 (28.1 against 27.3 us), while
+    # 4,096 -> 12,288, 256 blocks of three, stays 0.6 us quicker at 8 rows (34 MB); 9,216 -> 36,864 at 8 rows
+    # (226 MB): 111.1 us against 106.3.
     fuse_norm = True
     fuse_norm_rows = 8
+    fuse_norm_bytes = 40 << 20
 
-    def _norm_in_the_product(self, m, n) -> bool:
+    def _norm_in_the_product(self, m, n, k) -> bool:
         if m > self.fuse_norm_rows:
             return False
         key = (m, n)
         if key not in self._tiles_per_block:
             self._tiles_per_block[key] = library("gemm").tnx_gemm_skinny_tiles_per_block(m, n)
-        return self._tiles_per_block[key] >= 2
+        tiles = self._tiles_per_block[key]
+        blocks = -(-(n // 16) // tiles)
+        return tiles >= 2 and blocks * m * k * 4 <= self.fuse_norm_bytes
     few_rows = 32           # the few-rows kernel takes up to this many rows
 
     def fold_norm(self, w, weight, bias, center=True) -> bool:
@@ -498,7 +505,7 @@ class HipOps:
                 folded = None
             if folded is None:
                 x = x.materialize()
-            elif not self._norm_in_the_product(x.shape[0], w.tensor.shape[0]):
+            elif not self._norm_in_the_product(x.shape[0], w.tensor.shape[0], w.tensor.shape[1]):
                 # the norm's kernel without weight and bias, then the plain product of the folded copy
                 m, k = x.shape
                 n = w.tensor.shape[0]
@@ -728,7 +735,7 @@ class HipOps:
                 folded = None
             if folded is None:
                 h = h.materialize()
-            elif not self._norm_in_the_product(h.shape[0], w.tensor.shape[0]):
+            elif not self._norm_in_the_product(h.shape[0], w.tensor.shape[0], w.tensor.shape[1]):
                 # the norm's kernel without weight and bias, then the fused projection of the folded copy
                 h, w, bias = h.normalised(), PreparedWeight(w.tensor, folded.tiles), folded.d_with(bias)
             else:
