@@ -181,12 +181,17 @@ def test_generation_with_few_pages_bfloat16(tiny_folders_bf16, name):
         outs = engine.generate(prompts, params)
         runner.cache.check()
         assert (engine.scheduler.num_preemptions > 0) == (max_tokens == tight)
+        allowed = []
         for prompt, out in zip(prompts, outs):
             toks = prompt + out
             logits = plain_opt.forward_logits(weights, cfg, toks[:-1])
             for pos in range(len(prompt) - 1, len(toks) - 1):
                 row = logits[pos]
-                assert float(row.max() - row[toks[pos + 1]]) <= 3e-2 * float(row.abs().max()), (pos, toks[pos + 1])
+                slack = 3e-2 * float(row.abs().max())
+                assert float(row.max() - row[toks[pos + 1]]) <= slack, (pos, toks[pos + 1])
+                allowed.append(int((row.max() - row <= slack).sum()))
+        # and that says something: of the hundreds of tokens of the vocabulary one or two pass at a place
+        assert sum(allowed) / len(allowed) < 3, sum(allowed) / len(allowed)
 
 
 def test_no_run_of_tokens_twice_on_the_gpu(tiny_folders):

@@ -41,13 +41,17 @@ def tap(name: str, tensor):
 
 @contextlib.contextmanager
 def debug_context():
-    """`with debug_context() as tensors:` runs steps with every tapped tensor kept in `tensors`."""
+    """`with debug_context() as tensors:` runs steps with every tapped tensor kept in `tensors`. Inside another
+    one, what is tapped goes to the inner one's `tensors` and, when that closes, to the outer one's as well."""
     global _tapped
-    _tapped = OrderedDict()
+    outer, mine = _tapped, OrderedDict()
+    _tapped = mine
     try:
-        yield _tapped
+        yield mine
     finally:
-        _tapped = None
+        _tapped = outer
+        for name, tensor in mine.items():
+            tap(name.split("#")[0], tensor)
 
 
 class KernelTimer:

@@ -20,6 +20,7 @@ from ..cache.manager import CacheManager
 from .. import debug
 from .batch import PackedStep, StepContext, StepEntry, context_from, pack_step
 from .model import DecoderModel
+from .snapshot import snapshots_from_environment
 
 
 class _Staging:
@@ -105,6 +106,8 @@ class ModelRunner:
         self.kept_tokens = torch.zeros(cache.max_seqs, dtype=torch.int32, device=model.device)
         self._last_ctx: Optional[StepContext] = None
         self._staging = _Staging(ops) if hasattr(ops, "pinned_ints") else None
+        # steps written to a folder for running them again alone (`engine/snapshot.py`); None: none are
+        self.snapshots = snapshots_from_environment()
 
     # The most recordings kept; the one unused longest goes when another is made. A recording is one batch size
     # and one answer of the parts to `launch_shape` (the decode attention's: how many blocks share a request's
@@ -172,9 +175,12 @@ class ModelRunner:
         their `want`; None when nothing is wanted (the step still runs)."""
         if not entries:
             return None
-        recordable = (self.use_graphs and not debug.active()
+        taking = self.snapshots is not None and self.snapshots.wanted()
+        recordable = (self.use_graphs and not debug.active() and not taking
                       and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries))
         packed = self.prepare(entries, fixed_width=recordable, kept_allowed=kept_allowed)
+        if taking:
+            self.snapshots.enter(self, entries)
         if recordable:
             rec = self._recording(packed)
             logits = rec.replay(packed)
@@ -187,8 +193,15 @@ class ModelRunner:
                 ints = torch.from_numpy(packed.flat).to(self.model.device)
             ctx = context_from(packed, ints)
             ctx.kept_tokens = self.kept_tokens
-            logits = self.model.forward(ctx, self.cache.caches)
+            if taking:
+                with debug.debug_context() as taps:
+                    logits = self.model.forward(ctx, self.cache.caches)
+                self.snapshots.exit(logits if any(len(e.want) for e in entries) else None, taps)
+            else:
+                logits = self.model.forward(ctx, self.cache.caches)
             self._last_ctx = ctx
+        if self.snapshots is not None:
+            self.snapshots.iteration += 1
         for e in entries:
             self.cache.advance(e.req, len(e.tokens))
         return logits if any(len(e.want) for e in entries) else None
