@@ -365,7 +365,7 @@ def _toy_model(ops_kind, dtype, device):
     from transformers_neuronx_amd.weights import TensorDict, random_tensors
     spec = toy_parts.toy_spec()
     model = DecoderModel(spec)
-    tensors = random_tensors(model.param_decls(), spec.init_std, 3, torch.float32)
+    tensors = random_tensors(model.param_decls(), spec.init_std, 3, dtype)    # stored as the engine computes
     ops = make_ops(ops_kind, dtype, device)
     model.load(TensorDict(tensors), ops, dtype, device)
     needs = model.cache_needs()
@@ -413,7 +413,7 @@ def run_toy_routed_model(ops_kind, dtype, device, tol):
     spec = toy_parts.toy_spec_routed()
     model = DecoderModel(spec)
     assert not model.recordable                                 # toy parts do not claim to be replayable
-    tensors = random_tensors(model.param_decls(), spec.init_std, 5, torch.float32)
+    tensors = random_tensors(model.param_decls(), spec.init_std, 5, dtype)    # stored as the engine computes
     ops = make_ops(ops_kind, dtype, device)
     model.load(TensorDict(tensors), ops, dtype, device)
     runner = ModelRunner(model, CacheManager(model.cache_needs(), 16, 12, 4, dtype, device), ops, use_graphs=True)
@@ -451,7 +451,7 @@ def run_toy_rotating_model(ops_kind, dtype, device, tol, in_the_projection=False
     # keys, every part can be replayed from a recording (the layer with Python loops is left out of that model)
     spec = toy_parts.toy_spec_rotating(tables=in_the_projection, latent_layer=not in_the_projection)
     model = DecoderModel(spec)
-    tensors = random_tensors(model.param_decls(), spec.init_std, 6, torch.float32)
+    tensors = random_tensors(model.param_decls(), spec.init_std, 6, dtype)    # stored as the engine computes
     assert "blocks.2.attn.wk.weight" in tensors and tensors["blocks.0.attn.wk.weight"].shape == (32, 96)
     ops = make_ops(ops_kind, dtype, device)
     model.load(TensorDict(tensors), ops, dtype, device)
