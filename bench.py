@@ -68,11 +68,13 @@ def raw_config(model: str) -> dict:
 
 
 def keep_busy(ops, torch, seconds):
-    """Reads memory for a while before anything is timed. A process that starts right after another has ended
-    measures its memory-bound steps some 4 % slow for its first two or three seconds on this pool, then
-    abruptly as always (seen with one and the same program started twice in a row; the cause is not
-    established: the memory the earlier process gave back may still be being cleared). A measurement that
-    is meant to say what the engine does is taken after that."""
+    """Reads memory for a while before anything is timed. Memory-bound steps measure some 4 % slow for two or
+    three seconds after a lot of device memory has been given back, by a process that has just ended or by this
+    one (an engine closed and another built): seen with one and the same program started twice in a row, and
+    with engines of OPT-6.7B's sizes built one after the other in one process, each as fast as the first once
+    the device had been kept reading for four seconds (4.37 against 4.58 ms a step). The cause is not
+    established (the memory given back may be being cleared meanwhile; a kernel that only reads one buffer does
+    not feel it). The headline is measured on the first engine of the process, after this."""
     buf = torch.empty(1 << 30, dtype=torch.uint8, device=ops.device)
     out = torch.zeros(ops.compute_units * 32, dtype=torch.float32, device=ops.device)
     end = time.time() + seconds
