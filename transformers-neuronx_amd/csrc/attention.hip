@@ -13,7 +13,32 @@ TNX_DEFINE_ERROR_API
 
 // One thread takes 8 consecutive elements of a token's [q | k | v] row: a query chunk goes to the dense
 // query matrix scaled, a key chunk to its page as it is (head-size elements are contiguous there), a value
-// chunk element by element (values lie transposed inside a page).
+// chunk element by element (values lie transposed inside a page). Chunks are read and written 16 bytes at a
+// time in bfloat16 (rows and pages are 16-byte aligned there: the launcher sees to it).
+template <typename T>
+__device__ __forceinline__ void load8(const T* p, float* v) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = to_f32(p[j]);
+}
+template <>
+__device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float* v) {
+  const bf16x8 x = *(const bf16x8*)p;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = (float)x[j];
+}
+template <typename T>
+__device__ __forceinline__ void store8(T* p, const float* v) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) p[j] = from_f32<T>(v[j]);
+}
+template <>
+__device__ __forceinline__ void store8<bf16_t>(bf16_t* p, const float* v) {
+  bf16x8 x;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) x[j] = (bf16_t)v[j];
+  *(bf16x8*)p = x;
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256)
 qkv_write_kernel(const T* __restrict__ qkv, const float* __restrict__ bias, float scale,
@@ -28,13 +53,19 @@ qkv_write_kernel(const T* __restrict__ qkv, const float* __restrict__ bias, floa
   const int total = nq + 2 * nk;
   const int i0 = (blockIdx.y * 256 + threadIdx.x) * 8;
   if (i0 >= total) return;
+  if (values_of_single_tokens_only && i0 >= nq + nk) {   // the values of longer runs are written by tiles
+    const int r = token_request[t];
+    if (run_start[r + 1] - run_start[r] > 1) return;
+  }
   float v[8];
-  const T* row = qkv + (size_t)t * total + i0;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) v[j] = to_f32(row[j]);
+  load8<T>(qkv + (size_t)t * total + i0, v);
   if (bias) {
+    const f32x4 b0 = *(const f32x4*)(bias + i0), b1 = *(const f32x4*)(bias + i0 + 4);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] += bias[i0 + j];
+    for (int j = 0; j < 4; ++j) {
+      v[j] += b0[j];
+      v[4 + j] += b1[j];
+    }
   }
   if (turn_a && i0 < nq + nk) {
     // a position encoding that turns queries and keys pair by pair: x[d] becomes a[p][d] x[d] + b[p][d] x[d ^ 1]
@@ -47,9 +78,9 @@ qkv_write_kernel(const T* __restrict__ qkv, const float* __restrict__ bias, floa
     for (int j = 0; j < 8; ++j) v[j] = w[j];
   }
   if (i0 < nq) {
-    T* dst = q_out + (size_t)t * nq + i0;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) dst[j] = from_f32<T>(v[j] * scale);
+    for (int j = 0; j < 8; ++j) v[j] *= scale;
+    store8<T>(q_out + (size_t)t * nq + i0, v);
     return;
   }
   const int pos = positions[t];
@@ -59,14 +90,8 @@ qkv_write_kernel(const T* __restrict__ qkv, const float* __restrict__ bias, floa
   if (page < 0 || page >= num_pages) return;
   if (i0 < nq + nk) {
     const int j0 = i0 - nq, h = j0 / head_size, d = j0 % head_size;
-    T* dst = k_pages + (size_t)page * page_stride + ((size_t)h * page_size + off) * head_size + d;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) dst[j] = from_f32<T>(v[j]);
+    store8<T>(k_pages + (size_t)page * page_stride + ((size_t)h * page_size + off) * head_size + d, v);
   } else {
-    if (values_of_single_tokens_only) {   // the values of longer runs are written by tiles
-      const int r = token_request[t];
-      if (run_start[r + 1] - run_start[r] > 1) return;
-    }
     const int j0 = i0 - nq - nk, h = j0 / head_size, d = j0 % head_size;
     T* dst = v_pages + (size_t)page * page_stride + ((size_t)h * head_size + d) * page_size + off;
 #pragma unroll
@@ -75,10 +100,12 @@ qkv_write_kernel(const T* __restrict__ qkv, const float* __restrict__ bias, floa
 }
 
 // The values of a tile of up to 128 consecutive tokens of one run, one kv head a block. Values lie transposed
-// in a page (consecutive positions are neighbours), so the tile goes through LDS: it is read as rows of the
-// product, 16 bytes a thread, and written 8 consecutive positions (16 bytes) a thread. Groups of 8 are
-// aligned to positions, not to the tile; a group that the tile covers in part is written element by element.
-constexpr int VT_TOKENS = 128, VT_DIMS = 64, VT_ROW = VT_DIMS + 8;
+// in a page (consecutive positions are neighbours): a thread takes 8 consecutive positions and 8 consecutive
+// elements of the head, reads them as 8 rows of the product, 16 bytes each, and writes them as 8 rows of the
+// page, 16 bytes each; the lanes of a wave are 8 groups of positions (a row of a 64-token page: 128 bytes a
+// store) by 8 chunks of elements (128 bytes of a token's row a load). Groups of 8 are aligned to positions, not
+// to the tile; a group that the tile covers in part is written element by element.
+constexpr int VT_TOKENS = 128;
 
 __global__ void __launch_bounds__(256)
 value_tiles_kernel(const bf16_t* __restrict__ qkv, const float* __restrict__ bias, const int* __restrict__ run_start,
@@ -86,7 +113,6 @@ value_tiles_kernel(const bf16_t* __restrict__ qkv, const float* __restrict__ bia
                    int page_size, int num_pages, const int* __restrict__ tile_run,
                    const int* __restrict__ tile_q0, bf16_t* __restrict__ v_pages, int num_heads, int num_kv,
                    int head_size, int page_pad) {
-  __shared__ __attribute__((aligned(16))) bf16_t sm[VT_TOKENS * VT_ROW];
   const size_t page_stride = (size_t)num_kv * page_size * head_size + page_pad;
   const int run = tile_run[blockIdx.x], q0 = tile_q0[blockIdx.x], kvh = blockIdx.y;
   const int t0 = run_start[run] + q0;
@@ -96,39 +122,46 @@ value_tiles_kernel(const bf16_t* __restrict__ qkv, const float* __restrict__ bia
   const int col0 = (num_heads + num_kv) * head_size + kvh * head_size;
   const int* tab = table + (size_t)run * table_width;
   const int groups = (p0 + n - 1) / 8 - p0 / 8 + 1;
-  for (int dc = 0; dc < head_size; dc += VT_DIMS) {
-    const int dims = min(VT_DIMS, head_size - dc);     // a multiple of 8
-    const int chunks = dims / 8;
-    for (int idx = threadIdx.x; idx < n * chunks; idx += 256) {
-      const int i = idx / chunks, c = idx % chunks;
-      bf16x8 v = *(const bf16x8*)(qkv + (size_t)(t0 + i) * total + col0 + dc + c * 8);
-      if (bias) {
+  const int chunks = head_size / 8;
+  // item = (chunk / 8, group / 8, chunk % 8, group % 8): the groups run fastest within a wave's 64 lanes
+  const int group_blocks = (groups + 7) / 8;
+  for (int item = threadIdx.x; item < group_blocks * 8 * ((chunks + 7) / 8) * 8; item += 256) {
+    const int g = (item >> 6) % group_blocks * 8 + (item & 7);
+    const int c = (item >> 6) / group_blocks * 8 + ((item >> 3) & 7);
+    if (g >= groups || c >= chunks) continue;
+    const int pos = (p0 / 8 + g) * 8;                 // first position of the group
+    const int blk = pos / page_size;
+    const int page = blk < table_width ? tab[blk] : -1;
+    if (page < 0 || page >= num_pages) continue;
+    const int i0 = pos - p0;                           // the group's first token within the tile; may be < 0
+    bf16x8 rows[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = (bf16_t)((float)v[j] + bias[col0 + dc + c * 8 + j]);
-      }
-      *(bf16x8*)(sm + i * VT_ROW + c * 8) = v;
+    for (int j = 0; j < 8; ++j) {
+      const int i = min(max(i0 + j, 0), n - 1);        // (tokens outside the tile are read somewhere and not written)
+      rows[j] = *(const bf16x8*)(qkv + (size_t)(t0 + i) * total + col0 + c * 8);
     }
-    __syncthreads();
-    for (int idx = threadIdx.x; idx < groups * dims; idx += 256) {
-      const int g = idx / dims, d = idx % dims;
-      const int pos = (p0 / 8 + g) * 8;               // first position of the group
-      const int blk = pos / page_size;
-      const int page = blk < table_width ? tab[blk] : -1;
-      if (page < 0 || page >= num_pages) continue;
-      bf16_t* dst = v_pages + (size_t)page * page_stride + ((size_t)kvh * head_size + dc + d) * page_size + pos % page_size;
-      const int i0 = pos - p0;                         // the group's first token within the tile; may be < 0
-      if (i0 >= 0 && i0 + 8 <= n) {
+    if (bias) {
+      const f32x4 b0 = *(const f32x4*)(bias + col0 + c * 8), b1 = *(const f32x4*)(bias + col0 + c * 8 + 4);
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) rows[j][e] = (bf16_t)((float)rows[j][e] + (e < 4 ? b0[e] : b1[e - 4]));
+    }
+    bf16_t* dst = v_pages + (size_t)page * page_stride + ((size_t)kvh * head_size + c * 8) * page_size + pos % page_size;
+    const bool whole = i0 >= 0 && i0 + 8 <= n;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      if (whole) {
         bf16x8 v;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = sm[(i0 + j) * VT_ROW + d];
-        *(bf16x8*)dst = v;
+        for (int j = 0; j < 8; ++j) v[j] = rows[j][e];
+        *(bf16x8*)(dst + (size_t)e * page_size) = v;
       } else {
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-          if (i0 + j >= 0 && i0 + j < n) dst[j] = sm[(i0 + j) * VT_ROW + d];
+          if (i0 + j >= 0 && i0 + j < n) dst[(size_t)e * page_size + j] = rows[j][e];
       }
     }
-    __syncthreads();
   }
 }
 
@@ -149,6 +182,8 @@ extern "C" int tnx_qkv_write(const void* qkv, int dtype, const float* bias, floa
   TNX_REQUIRE(page_size > 0 && table_width > 0, "qkv_write: bad page table");
   if (tokens == 0) return 0;
   TNX_REQUIRE(head_size % 8 == 0, "qkv_write: head size %d is not a multiple of 8", head_size);
+  TNX_REQUIRE(((uintptr_t)qkv | (uintptr_t)bias | (uintptr_t)q_out | (uintptr_t)k_pages | (uintptr_t)v_pages) % 16 == 0,
+              "qkv_write: the projections, the bias, the queries and the pages must be 16-byte aligned");
   const bool by_tiles = num_tiles > 0 && num_kv > 0;
   if (by_tiles) {
     TNX_REQUIRE(dtype == TNX_BF16, "qkv_write: values are written by tiles in bfloat16 only");
