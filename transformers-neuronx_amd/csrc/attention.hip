@@ -1779,6 +1779,38 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, 
   const int h = blockIdx.x, dz = blockIdx.y;
   const int run = decode_runs[dz];            // where the result goes is asked for beside the partial results
   const size_t base = ((size_t)dz * num_heads + h) * num_splits;
+  if (num_splits <= 8) {
+    // The usual case. Everything is asked for before anything is computed, so that the kernel waits for
+    // memory once (shares beyond the last read the last one again and are left out of the sums); the sums
+    // are made in the order of the loop below, to the same bits.
+    float ms[8], ls[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const size_t i = base + min(s, num_splits - 1);
+      ms[s] = part_ml[i * 2];
+      ls[s] = part_ml[i * 2 + 1];
+    }
+    const int t = run_start[run];
+    for (int d = threadIdx.x; d < head_size; d += blockDim.x) {
+      float os[8];
+#pragma unroll
+      for (int s = 0; s < 8; ++s) os[s] = part_o[(base + min(s, num_splits - 1)) * head_size + d];
+      float mm = -INFINITY;
+#pragma unroll
+      for (int s = 0; s < 8; ++s)
+        if (s < num_splits) mm = fmaxf(mm, ms[s]);
+      float ll = 0.f, oo = 0.f;
+#pragma unroll
+      for (int s = 0; s < 8; ++s)
+        if (s < num_splits) {
+          const float f = ms[s] == -INFINITY ? 0.f : __expf(ms[s] - mm);
+          ll += ls[s] * f;
+          oo += os[s] * f;
+        }
+      out[((size_t)t * num_heads + h) * head_size + d] = (bf16_t)(oo / ll);
+    }
+    return;
+  }
   float mm = -INFINITY;
   for (int s = 0; s < num_splits; ++s) mm = fmaxf(mm, part_ml[(base + s) * 2]);
   const int t = run_start[run];

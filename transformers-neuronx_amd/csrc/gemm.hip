@@ -1128,8 +1128,21 @@ gemm_mid_sum_kernel(const float* __restrict__ partial, const float* __restrict__
                     int shares) {
   const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
   if (i >= (size_t)M * N) return;
-  f32x4 v = *(const f32x4*)(partial + i);
-  for (int s = 1; s < shares; ++s) v += *(const f32x4*)(partial + (size_t)s * M * N + i);
+  f32x4 v;
+  if (shares <= 8) {
+    // every share is asked for before the first is added (shares beyond the last read the last one again and
+    // are left out), so that the kernel waits for memory once; the order of the sum stays
+    f32x4 p[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) p[s] = *(const f32x4*)(partial + (size_t)min(s, shares - 1) * M * N + i);
+    v = p[0];
+#pragma unroll
+    for (int s = 1; s < 8; ++s)
+      if (s < shares) v += p[s];
+  } else {
+    v = *(const f32x4*)(partial + i);
+    for (int s = 1; s < shares; ++s) v += *(const f32x4*)(partial + (size_t)s * M * N + i);
+  }
   const int m = (int)(i / N), n = (int)(i % N);
 #pragma unroll
   for (int e = 0; e < 4; ++e) epilogue_store(v[e], m, n + e, N, bias, residual, out, out_dtype, act);
