@@ -809,7 +809,7 @@ class HipOps:
             num_pages = self._check_pages(k_pages, v_pages, num_kv_write, head_size, view.page_size)
         _want(view.block_table, "block table", torch.int32, (ctx.num_requests, view.width))
         q = torch.empty(t, num_heads * head_size, dtype=self.dtype, device=qkv.device)
-        # the values of runs of several tokens are written by tiles (transposed through LDS)
+        # the values of runs of several tokens are written by tiles (8 positions by 8 elements a thread, 16 bytes a store)
         by_tiles = (self.dtype == torch.bfloat16 and self.value_tiles and num_kv_write
                     and ctx.plan.get("tile_run") is not None and ctx.plan["tile_run"].numel() > 0)
         self._call("attention", "tnx_qkv_write", _ptr(qkv), _code(self.dtype), _ptr(bias), float(scale),
